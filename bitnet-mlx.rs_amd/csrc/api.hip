@@ -1,0 +1,623 @@
+// extern "C" entry points: argument validation, error records, and the BitLinear / decoder objects.
+// No arithmetic lives here; every result comes from the kernels behind the launch_* functions.
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <shared_mutex>
+#include <vector>
+
+#include "kernels.hpp"
+
+namespace bitnet {
+
+ErrorRecord &error_record()
+{
+    static thread_local ErrorRecord rec;
+    return rec;
+}
+
+int fail(int code, const char *fmt, ...)
+{
+    ErrorRecord &r = error_record();
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(r.msg, sizeof r.msg, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int fail_shape(const size_t *expected, int erank, const size_t *actual, int arank, const char *what)
+{
+    ErrorRecord &r = error_record();
+    r.expected_rank = erank > 4 ? 4 : erank;
+    r.actual_rank = arank > 4 ? 4 : arank;
+    for (int i = 0; i < r.expected_rank; ++i) r.expected[i] = expected[i];
+    for (int i = 0; i < r.actual_rank; ++i) r.actual[i] = actual[i];
+    char e[96] = {0}, a[96] = {0};
+    size_t eo = 0, ao = 0;
+    for (int i = 0; i < r.expected_rank; ++i)
+        eo += snprintf(e + eo, sizeof e - eo, i ? ", %zu" : "%zu", expected[i]);
+    for (int i = 0; i < r.actual_rank; ++i)
+        ao += snprintf(a + ao, sizeof a - ao, i ? ", %zu" : "%zu", actual[i]);
+    snprintf(r.msg, sizeof r.msg, "Shape mismatch (%s): expected [%s], got [%s]", what, e, a);
+    return BITNET_HIP_SHAPE_MISMATCH;
+}
+
+namespace {
+
+// Device buffer freed when it goes out of scope (after the stream it was used on has been drained).
+struct DeviceTemp {
+    void *ptr = nullptr;
+    ~DeviceTemp() { if (ptr) (void)hipFree(ptr); }
+    int alloc(size_t bytes)
+    {
+        hipError_t e = hipMalloc(&ptr, bytes ? bytes : 1);
+        if (e != hipSuccess) {
+            ptr = nullptr;
+            return fail(BITNET_HIP_MEMORY_ERROR, "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+        }
+        return BITNET_HIP_OK;
+    }
+};
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+}  // namespace bitnet
+
+using namespace bitnet;
+
+// ---------------------------------------------------------------------------------------------------
+// BitLinear object
+// ---------------------------------------------------------------------------------------------------
+struct bitnet_hip_bitlinear {
+    size_t in_features = 0;
+    size_t out_features = 0;
+    bool use_bias = false;
+    bool has_weights = false;
+    uint8_t *packed = nullptr;  // reference byte format, [out, in] flat
+    uint8_t *tiled = nullptr;   // streaming layout
+    float *w_scale = nullptr;   // one float, device
+    float *bias = nullptr;      // [out], device (zeros until set, like the reference's Tensor::zeros)
+    // readers: forward; writer: set_weights / set_bias (the reference guards weights with a RwLock)
+    mutable std::shared_mutex lock;
+
+    ~bitnet_hip_bitlinear()
+    {
+        if (packed) (void)hipFree(packed);
+        if (tiled) (void)hipFree(tiled);
+        if (w_scale) (void)hipFree(w_scale);
+        if (bias) (void)hipFree(bias);
+    }
+};
+
+extern "C" {
+
+const char *bitnet_hip_last_error(void) { return error_record().msg; }
+
+int bitnet_hip_last_shape_mismatch(size_t expected[4], size_t actual[4], int *actual_rank)
+{
+    ErrorRecord &r = error_record();
+    for (int i = 0; i < r.expected_rank; ++i) expected[i] = r.expected[i];
+    for (int i = 0; i < r.actual_rank; ++i) actual[i] = r.actual[i];
+    if (actual_rank) *actual_rank = r.actual_rank;
+    return r.expected_rank;
+}
+
+int bitnet_hip_init(int device)
+{
+    int count = 0;
+    BITNET_HIP_TRY(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count)
+        return fail(BITNET_HIP_INVALID_CONFIG, "device %d out of range (%d visible)", device, count);
+    BITNET_HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    BITNET_HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(BITNET_HIP_UNSUPPORTED, "device %d is %s; this library carries gfx950 code only", device,
+                    prop.gcnArchName);
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_device_info(char *arch_name, size_t arch_name_len, int *compute_units, int *clock_mhz,
+                           size_t *total_mem_bytes)
+{
+    int device = 0;
+    BITNET_HIP_TRY(hipGetDevice(&device));
+    hipDeviceProp_t prop;
+    BITNET_HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (arch_name && arch_name_len) {
+        strncpy(arch_name, prop.gcnArchName, arch_name_len - 1);
+        arch_name[arch_name_len - 1] = 0;
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (clock_mhz) *clock_mhz = prop.clockRate / 1000;
+    if (total_mem_bytes) *total_mem_bytes = prop.totalGlobalMem;
+    return BITNET_HIP_OK;
+}
+
+// ---- activation side ------------------------------------------------------------------------------
+
+int bitnet_hip_quantize_activations_i8(const float *x, const float *x2, size_t ldx, size_t m, size_t k,
+                                       int input_mode, size_t gqa_group, size_t head_dim, const float *gamma,
+                                       float eps, int sum_order, int8_t *q, float *a_scale, int32_t *a_sum,
+                                       float *y_f32, void *stream)
+{
+    if (m == 0 || k == 0) return BITNET_HIP_OK;
+    if (!x || !q || !a_scale) return fail(BITNET_HIP_NULL_POINTER, "quantize_activations_i8: x, q and a_scale are required");
+    if (k > 0x7fffffffu) return fail(BITNET_HIP_UNSUPPORTED, "quantize_activations_i8: k=%zu too large", k);
+    if (sum_order != BITNET_HIP_SUM_SEQUENTIAL && sum_order != BITNET_HIP_SUM_WAVE64)
+        return fail(BITNET_HIP_INVALID_CONFIG, "quantize_activations_i8: unknown sum_order %d", sum_order);
+    size_t src_cols = k;
+    switch (input_mode) {
+        case BITNET_HIP_INPUT_PLAIN: break;
+        case BITNET_HIP_INPUT_RELU2_MUL:
+            if (!x2) return fail(BITNET_HIP_NULL_POINTER, "quantize_activations_i8: RELU2_MUL needs x2");
+            break;
+        case BITNET_HIP_INPUT_GQA_BROADCAST:
+            if (gqa_group == 0 || head_dim == 0 || k % (gqa_group * head_dim) != 0)
+                return fail(BITNET_HIP_INVALID_CONFIG,
+                            "quantize_activations_i8: k=%zu is not a multiple of gqa_group*head_dim=%zu*%zu", k,
+                            gqa_group, head_dim);
+            src_cols = k / gqa_group;
+            break;
+        default: return fail(BITNET_HIP_INVALID_CONFIG, "quantize_activations_i8: unknown input_mode %d", input_mode);
+    }
+    if (ldx < src_cols) {
+        size_t e[2] = {m, src_cols}, a[2] = {m, ldx};
+        return fail_shape(e, 2, a, 2, "row stride smaller than the row");
+    }
+    return launch_act_quant(x, x2, ldx, m, k, input_mode, gqa_group, head_dim, gamma, eps, sum_order, q, a_scale,
+                            a_sum, y_f32, as_stream(stream));
+}
+
+// ---- weight side -----------------------------------------------------------------------------------
+
+size_t bitnet_hip_packed_size(size_t count) { return (count + 3) / 4; }
+
+int bitnet_hip_pack_ternary_2bit(const int8_t *q, size_t count, uint8_t *packed, void *stream)
+{
+    if (count == 0) return BITNET_HIP_OK;
+    if (!q || !packed) return fail(BITNET_HIP_NULL_POINTER, "pack_ternary_2bit: null buffer");
+    return launch_pack_2bit(q, count, packed, as_stream(stream));
+}
+
+int bitnet_hip_unpack_ternary_2bit(const uint8_t *packed, size_t count, int8_t *q, void *stream)
+{
+    if (count == 0) return BITNET_HIP_OK;
+    if (!q || !packed) return fail(BITNET_HIP_NULL_POINTER, "unpack_ternary_2bit: null buffer");
+    return launch_unpack_2bit(packed, count, q, as_stream(stream));
+}
+
+int bitnet_hip_quantize_weights(const float *w, size_t n, size_t k, int method, float threshold_factor,
+                                uint8_t *packed, float *w_scale, int8_t *q_i8, void *stream)
+{
+    if (!w_scale) return fail(BITNET_HIP_NULL_POINTER, "quantize_weights: w_scale is required");
+    if (n * k != 0 && (!w || !packed)) return fail(BITNET_HIP_NULL_POINTER, "quantize_weights: null buffer");
+    if (method != BITNET_HIP_TERNARY_ABSMEAN_ROUNDCLIP && method != BITNET_HIP_TERNARY_MEAN_THRESHOLD)
+        return fail(BITNET_HIP_INVALID_CONFIG, "quantize_weights: unknown method %d", method);
+    DeviceTemp row_sums;
+    int rc = row_sums.alloc(sizeof(double) * (n ? n : 1));
+    if (rc != BITNET_HIP_OK) return rc;
+    rc = launch_quantize_weights(w, n, k, method, threshold_factor, static_cast<double *>(row_sums.ptr), packed,
+                                 w_scale, q_i8, as_stream(stream));
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipStreamSynchronize(as_stream(stream)));  // row_sums is released on return
+    return BITNET_HIP_OK;
+}
+
+size_t bitnet_hip_tiled_size(size_t n, size_t k) { return tiled_bytes(n, k); }
+
+int bitnet_hip_retile_weights(const uint8_t *packed, size_t n, size_t k, int layout, uint8_t *tiled, void *stream)
+{
+    if (n * k == 0) return BITNET_HIP_OK;
+    if (!packed || !tiled) return fail(BITNET_HIP_NULL_POINTER, "retile_weights: null buffer");
+    if (layout != BITNET_HIP_LAYOUT_OUT_IN && layout != BITNET_HIP_LAYOUT_IN_OUT)
+        return fail(BITNET_HIP_INVALID_CONFIG, "retile_weights: unknown layout %d", layout);
+    if (reinterpret_cast<uintptr_t>(tiled) % 16)
+        return fail(BITNET_HIP_INVALID_CONFIG, "retile_weights: tiled buffer must be 16-byte aligned");
+    return launch_retile(packed, n, k, layout, tiled, as_stream(stream));
+}
+
+int bitnet_hip_untile_weights(const uint8_t *tiled, size_t n, size_t k, uint8_t *packed, void *stream)
+{
+    if (n * k == 0) return BITNET_HIP_OK;
+    if (!packed || !tiled) return fail(BITNET_HIP_NULL_POINTER, "untile_weights: null buffer");
+    return launch_untile(tiled, n, k, packed, as_stream(stream));
+}
+
+// ---- contraction -----------------------------------------------------------------------------------
+
+int bitnet_hip_gemv_w2a8(const uint8_t *weights, const int8_t *activations, int32_t *output, size_t m, size_t k,
+                         void *stream)
+{
+    if (m == 0) return BITNET_HIP_OK;
+    if (!output) return fail(BITNET_HIP_NULL_POINTER, "gemv_w2a8: output is NULL");
+    if (k != 0 && (!weights || !activations)) return fail(BITNET_HIP_NULL_POINTER, "gemv_w2a8: null input buffer");
+    return launch_gemv_rowmajor(weights, activations, output, m, k, as_stream(stream));
+}
+
+int bitnet_hip_gemv_w2a8_checked(const uint8_t *weights, size_t weights_len, const int8_t *activations,
+                                 size_t activations_len, int32_t *output, size_t output_len, size_t m, size_t k,
+                                 void *stream)
+{
+    // same three checks, same order, as validate_w2a8_dimensions (bitnet-cuda/src/backend.rs:217-257)
+    size_t expected_w = (m * k + 3) / 4;
+    if (weights_len != expected_w) {
+        size_t e[1] = {expected_w}, a[1] = {weights_len};
+        return fail_shape(e, 1, a, 1, "weight bytes for an m x k matrix");
+    }
+    if (activations_len != k) {
+        size_t e[1] = {k}, a[1] = {activations_len};
+        return fail_shape(e, 1, a, 1, "activation elements");
+    }
+    if (output_len != m) {
+        size_t e[1] = {m}, a[1] = {output_len};
+        return fail_shape(e, 1, a, 1, "output elements");
+    }
+    return bitnet_hip_gemv_w2a8(weights, activations, output, m, k, stream);
+}
+
+int bitnet_hip_matmul_w2a8(const uint8_t *tiled, const int8_t *a, size_t m, size_t n, size_t k, int32_t *acc,
+                           const float *w_scale, const float *a_scale, const float *bias, const float *residual,
+                           float *out, void *stream)
+{
+    if (m == 0 || n == 0) return BITNET_HIP_OK;
+    if (!tiled || !a) return fail(BITNET_HIP_NULL_POINTER, "matmul_w2a8: null input buffer");
+    if (!acc && !out) return fail(BITNET_HIP_NULL_POINTER, "matmul_w2a8: give acc, out or both");
+    if (out && (!w_scale || !a_scale)) return fail(BITNET_HIP_NULL_POINTER, "matmul_w2a8: out needs w_scale and a_scale");
+    if (reinterpret_cast<uintptr_t>(tiled) % 16)
+        return fail(BITNET_HIP_INVALID_CONFIG, "matmul_w2a8: tiled weights must be 16-byte aligned");
+    if (n > 0x7fffffffu || k > 0x7fffffffu) return fail(BITNET_HIP_UNSUPPORTED, "matmul_w2a8: dimension too large");
+    if (m <= (size_t)GEMV_MAX_M)
+        return launch_gemv_tiled(tiled, a, m, n, k, acc, w_scale, a_scale, bias, residual, out, as_stream(stream));
+    return launch_gemm_tiled(tiled, a, m, n, k, acc, w_scale, a_scale, bias, residual, out, as_stream(stream));
+}
+
+// ---- BitLinear layer object -------------------------------------------------------------------------
+
+int bitnet_hip_bitlinear_create(size_t in_features, size_t out_features, int use_bias, bitnet_hip_bitlinear **layer)
+{
+    if (!layer) return fail(BITNET_HIP_NULL_POINTER, "bitlinear_create: layer is NULL");
+    *layer = nullptr;
+    if (in_features == 0 || out_features == 0)
+        return fail(BITNET_HIP_INVALID_CONFIG, "bitlinear_create: in_features=%zu out_features=%zu must be positive",
+                    in_features, out_features);
+    bitnet_hip_bitlinear *l = new (std::nothrow) bitnet_hip_bitlinear;
+    if (!l) return fail(BITNET_HIP_MEMORY_ERROR, "bitlinear_create: out of host memory");
+    l->in_features = in_features;
+    l->out_features = out_features;
+    l->use_bias = use_bias != 0;
+    hipError_t e = hipMalloc(&l->packed, (in_features * out_features + 3) / 4);
+    if (e == hipSuccess) e = hipMalloc(&l->tiled, tiled_bytes(out_features, in_features));
+    if (e == hipSuccess) e = hipMalloc(&l->w_scale, sizeof(float));
+    if (e == hipSuccess && l->use_bias) {
+        e = hipMalloc(&l->bias, sizeof(float) * out_features);
+        if (e == hipSuccess) e = hipMemset(l->bias, 0, sizeof(float) * out_features);
+    }
+    if (e != hipSuccess) {
+        delete l;
+        return fail(BITNET_HIP_MEMORY_ERROR, "bitlinear_create: device allocation failed: %s", hipGetErrorString(e));
+    }
+    *layer = l;
+    return BITNET_HIP_OK;
+}
+
+void bitnet_hip_bitlinear_destroy(bitnet_hip_bitlinear *layer) { delete layer; }
+
+int bitnet_hip_bitlinear_set_weights_f32(bitnet_hip_bitlinear *layer, const float *w, size_t rows, size_t cols,
+                                         int layout, int on_device, int method, float threshold_factor, void *stream)
+{
+    if (!layer || !w) return fail(BITNET_HIP_NULL_POINTER, "set_weights_f32: null argument");
+    if (layout != BITNET_HIP_LAYOUT_OUT_IN && layout != BITNET_HIP_LAYOUT_IN_OUT)
+        return fail(BITNET_HIP_INVALID_CONFIG, "set_weights_f32: unknown layout %d", layout);
+    const size_t n = layer->out_features, k = layer->in_features;
+    const size_t er = layout == BITNET_HIP_LAYOUT_OUT_IN ? n : k, ec = layout == BITNET_HIP_LAYOUT_OUT_IN ? k : n;
+    if (rows != er || cols != ec) {
+        size_t e[2] = {er, ec}, a[2] = {rows, cols};
+        return fail_shape(e, 2, a, 2, "weight matrix");  // BitLinear::update_weights, layer.rs:301-307
+    }
+    hipStream_t s = as_stream(stream);
+    DeviceTemp w_dev, flat;
+    const float *src = w;
+    if (!on_device) {
+        int rc = w_dev.alloc(sizeof(float) * n * k);
+        if (rc != BITNET_HIP_OK) return rc;
+        BITNET_HIP_TRY(hipMemcpyAsync(w_dev.ptr, w, sizeof(float) * n * k, hipMemcpyHostToDevice, s));
+        src = static_cast<const float *>(w_dev.ptr);
+    }
+    int rc = flat.alloc((n * k + 3) / 4);
+    if (rc != BITNET_HIP_OK) return rc;
+    std::unique_lock<std::shared_mutex> guard(layer->lock);
+    rc = bitnet_hip_quantize_weights(src, rows, cols, method, threshold_factor, static_cast<uint8_t *>(flat.ptr),
+                                     layer->w_scale, nullptr, stream);
+    if (rc != BITNET_HIP_OK) return rc;
+    rc = launch_retile(static_cast<const uint8_t *>(flat.ptr), n, k, layout, layer->tiled, s);
+    if (rc != BITNET_HIP_OK) return rc;
+    rc = launch_untile(layer->tiled, n, k, layer->packed, s);  // canonical [out, in] bytes
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipStreamSynchronize(s));
+    layer->has_weights = true;
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_bitlinear_set_weights_packed(bitnet_hip_bitlinear *layer, const uint8_t *packed, size_t packed_len,
+                                            float w_scale, int on_device, void *stream)
+{
+    if (!layer || !packed) return fail(BITNET_HIP_NULL_POINTER, "set_weights_packed: null argument");
+    const size_t n = layer->out_features, k = layer->in_features, need = (n * k + 3) / 4;
+    if (packed_len < need) {
+        // WeightConverter::convert_ternary_weights rejects short buffers (weight_conversion.rs:153-158)
+        size_t e[1] = {need}, a[1] = {packed_len};
+        return fail_shape(e, 1, a, 1, "packed weight bytes");
+    }
+    hipStream_t s = as_stream(stream);
+    std::unique_lock<std::shared_mutex> guard(layer->lock);
+    BITNET_HIP_TRY(hipMemcpyAsync(layer->packed, packed, need, on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, s));
+    BITNET_HIP_TRY(hipMemcpyAsync(layer->w_scale, &w_scale, sizeof(float), hipMemcpyHostToDevice, s));
+    int rc = launch_retile(layer->packed, n, k, BITNET_HIP_LAYOUT_OUT_IN, layer->tiled, s);
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipStreamSynchronize(s));  // w_scale is read from the caller's stack
+    layer->has_weights = true;
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_bitlinear_set_bias(bitnet_hip_bitlinear *layer, const float *bias, size_t len, int on_device, void *stream)
+{
+    if (!layer || !bias) return fail(BITNET_HIP_NULL_POINTER, "set_bias: null argument");
+    if (!layer->use_bias) return fail(BITNET_HIP_INVALID_CONFIG, "Bias is not enabled for this layer");
+    if (len != layer->out_features) {
+        size_t e[1] = {layer->out_features}, a[1] = {len};
+        return fail_shape(e, 1, a, 1, "bias");
+    }
+    std::unique_lock<std::shared_mutex> guard(layer->lock);
+    BITNET_HIP_TRY(hipMemcpyAsync(layer->bias, bias, sizeof(float) * len,
+                                  on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, as_stream(stream)));
+    BITNET_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_bitlinear_get_quantized(bitnet_hip_bitlinear *layer, float *w_scale, uint8_t *packed, size_t packed_len)
+{
+    if (!layer) return fail(BITNET_HIP_NULL_POINTER, "get_quantized: layer is NULL");
+    std::shared_lock<std::shared_mutex> guard(layer->lock);
+    if (!layer->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "get_quantized: the layer has no weights yet");
+    BITNET_HIP_TRY(hipDeviceSynchronize());
+    if (w_scale) BITNET_HIP_TRY(hipMemcpy(w_scale, layer->w_scale, sizeof(float), hipMemcpyDeviceToHost));
+    if (packed) {
+        size_t need = (layer->in_features * layer->out_features + 3) / 4;
+        if (packed_len < need) {
+            size_t e[1] = {need}, a[1] = {packed_len};
+            return fail_shape(e, 1, a, 1, "packed weight bytes");
+        }
+        BITNET_HIP_TRY(hipMemcpy(packed, layer->packed, need, hipMemcpyDeviceToHost));
+    }
+    return BITNET_HIP_OK;
+}
+
+size_t bitnet_hip_bitlinear_workspace_size(const bitnet_hip_bitlinear *layer, size_t m)
+{
+    if (!layer) return 0;
+    return align_up(m * layer->in_features, 256) + align_up(m * sizeof(float), 256) + 256;
+}
+
+int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, const size_t *dims, int rank,
+                                 const float *gamma, float eps, int sum_order, const float *residual, float *out,
+                                 void *workspace, size_t workspace_bytes, int8_t *dbg_q, float *dbg_a_scale,
+                                 int32_t *dbg_acc, void *stream)
+{
+    if (!layer) return fail(BITNET_HIP_NULL_POINTER, "forward: layer is NULL");
+    const size_t in = layer->in_features, nout = layer->out_features;
+    // shape rules of BitLinearForward::forward (forward.rs:60-76) and quantized_matmul (:179-214)
+    if (rank <= 0 || !dims) {
+        size_t e[2] = {1, in};
+        return fail_shape(e, 2, dims, 0, "input");
+    }
+    if (dims[rank - 1] != in) {
+        size_t e[2] = {dims[0], in};
+        return fail_shape(e, 2, dims, rank, "last input dimension");
+    }
+    if (rank != 2 && rank != 3) {
+        size_t e[2] = {1, in};
+        return fail_shape(e, 2, dims, rank, "input rank");
+    }
+    const size_t m = rank == 2 ? dims[0] : dims[0] * dims[1];
+    if (m == 0) return BITNET_HIP_OK;
+    if (!x || !out) return fail(BITNET_HIP_NULL_POINTER, "forward: x and out are required");
+
+    std::shared_lock<std::shared_mutex> guard(layer->lock);
+    if (!layer->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "forward: the layer has no weights yet");
+
+    hipStream_t s = as_stream(stream);
+    void *ws = workspace;
+    bool own_ws = false;
+    const size_t need = bitnet_hip_bitlinear_workspace_size(layer, m);
+    if (!ws) {
+        hipError_t e = hipMallocAsync(&ws, need, s);
+        if (e != hipSuccess) return fail(BITNET_HIP_MEMORY_ERROR, "forward: hipMallocAsync(%zu) failed: %s", need, hipGetErrorString(e));
+        own_ws = true;
+    } else if (workspace_bytes < need) {
+        return fail(BITNET_HIP_MEMORY_ERROR, "forward: workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    }
+    uintptr_t base = align_up(reinterpret_cast<uintptr_t>(ws), 256);
+    int8_t *q = dbg_q ? dbg_q : reinterpret_cast<int8_t *>(base);
+    float *a_scale = dbg_a_scale ? dbg_a_scale : reinterpret_cast<float *>(base + align_up(m * in, 256));
+
+    int rc = launch_act_quant(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, 1, gamma, eps, sum_order, q, a_scale,
+                              nullptr, nullptr, s);
+    if (rc == BITNET_HIP_OK)
+        rc = bitnet_hip_matmul_w2a8(layer->tiled, q, m, nout, in, dbg_acc, layer->w_scale, a_scale,
+                                    layer->use_bias ? layer->bias : nullptr, residual, out, stream);
+    if (own_ws) {
+        hipError_t e = hipFreeAsync(ws, s);
+        if (rc == BITNET_HIP_OK && e != hipSuccess)
+            rc = fail(BITNET_HIP_MEMORY_ERROR, "forward: hipFreeAsync failed: %s", hipGetErrorString(e));
+    }
+    return rc;
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------------------------
+// Decoder projections
+// ---------------------------------------------------------------------------------------------------
+struct bitnet_hip_decoder {
+    size_t layers = 0, hidden = 0, ffn = 0, q_heads = 0, kv_heads = 0, head_dim = 0, max_tokens = 0;
+    float eps = 1e-5f;
+    int sum_order = BITNET_HIP_SUM_WAVE64;
+    std::vector<bitnet_hip_bitlinear *> proj;  // layers * 7
+    float *gamma = nullptr;                    // [layers][2][hidden]
+    // activation buffers, sized for max_tokens
+    int8_t *a8 = nullptr;
+    float *a_scale = nullptr;
+    float *qb = nullptr, *kb = nullptr, *vb = nullptr, *x1 = nullptr, *gate = nullptr, *up = nullptr;
+    float *ping = nullptr;
+
+    ~bitnet_hip_decoder()
+    {
+        for (auto *p : proj) delete p;
+        void *bufs[] = {gamma, a8, a_scale, qb, kb, vb, x1, gate, up, ping};
+        for (void *b : bufs)
+            if (b) (void)hipFree(b);
+    }
+};
+
+extern "C" {
+
+int bitnet_hip_decoder_create(size_t layers, size_t hidden, size_t ffn, size_t q_heads, size_t kv_heads,
+                              size_t head_dim, float eps, int sum_order, size_t max_tokens, bitnet_hip_decoder **dec)
+{
+    if (!dec) return fail(BITNET_HIP_NULL_POINTER, "decoder_create: dec is NULL");
+    *dec = nullptr;
+    if (!layers || !hidden || !ffn || !q_heads || !kv_heads || !head_dim || !max_tokens)
+        return fail(BITNET_HIP_INVALID_CONFIG, "decoder_create: every size must be positive");
+    if (q_heads * head_dim != hidden || q_heads % kv_heads != 0)
+        return fail(BITNET_HIP_INVALID_CONFIG,
+                    "decoder_create: q_heads*head_dim=%zu must equal hidden=%zu and q_heads %% kv_heads must be 0",
+                    q_heads * head_dim, hidden);
+    bitnet_hip_decoder *d = new (std::nothrow) bitnet_hip_decoder;
+    if (!d) return fail(BITNET_HIP_MEMORY_ERROR, "decoder_create: out of host memory");
+    d->layers = layers; d->hidden = hidden; d->ffn = ffn; d->q_heads = q_heads; d->kv_heads = kv_heads;
+    d->head_dim = head_dim; d->eps = eps; d->sum_order = sum_order; d->max_tokens = max_tokens;
+    const size_t kv_dim = kv_heads * head_dim;
+    const size_t outs[7] = {hidden, kv_dim, kv_dim, hidden, ffn, ffn, hidden};
+    const size_t ins[7] = {hidden, hidden, hidden, hidden, hidden, hidden, ffn};
+    int rc = BITNET_HIP_OK;
+    for (size_t l = 0; l < layers && rc == BITNET_HIP_OK; ++l)
+        for (int p = 0; p < 7 && rc == BITNET_HIP_OK; ++p) {
+            bitnet_hip_bitlinear *bl = nullptr;
+            rc = bitnet_hip_bitlinear_create(ins[p], outs[p], 0, &bl);
+            if (rc == BITNET_HIP_OK) d->proj.push_back(bl);
+        }
+    const size_t widest = hidden > ffn ? hidden : ffn;
+    auto dev_alloc = [&](auto **ptr, size_t bytes) {
+        if (rc != BITNET_HIP_OK) return;
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(ptr), bytes);
+        if (e != hipSuccess) rc = fail(BITNET_HIP_MEMORY_ERROR, "decoder_create: hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    };
+    dev_alloc(&d->gamma, sizeof(float) * layers * 2 * hidden);
+    dev_alloc(&d->a8, max_tokens * widest);
+    dev_alloc(&d->a_scale, sizeof(float) * max_tokens);
+    dev_alloc(&d->qb, sizeof(float) * max_tokens * hidden);
+    dev_alloc(&d->kb, sizeof(float) * max_tokens * kv_dim);
+    dev_alloc(&d->vb, sizeof(float) * max_tokens * kv_dim);
+    dev_alloc(&d->x1, sizeof(float) * max_tokens * hidden);
+    dev_alloc(&d->gate, sizeof(float) * max_tokens * ffn);
+    dev_alloc(&d->up, sizeof(float) * max_tokens * ffn);
+    dev_alloc(&d->ping, sizeof(float) * max_tokens * hidden);
+    if (rc == BITNET_HIP_OK) {
+        // RMSNorm weights start at one
+        std::vector<float> ones(layers * 2 * hidden, 1.0f);
+        hipError_t e = hipMemcpy(d->gamma, ones.data(), sizeof(float) * ones.size(), hipMemcpyHostToDevice);
+        if (e != hipSuccess) rc = fail(BITNET_HIP_DEVICE_ERROR, "decoder_create: hipMemcpy failed: %s", hipGetErrorString(e));
+    }
+    if (rc != BITNET_HIP_OK) {
+        delete d;
+        return rc;
+    }
+    *dec = d;
+    return BITNET_HIP_OK;
+}
+
+void bitnet_hip_decoder_destroy(bitnet_hip_decoder *dec) { delete dec; }
+
+int bitnet_hip_decoder_projection(bitnet_hip_decoder *dec, size_t layer, int proj, bitnet_hip_bitlinear **out)
+{
+    if (!dec || !out) return fail(BITNET_HIP_NULL_POINTER, "decoder_projection: null argument");
+    if (layer >= dec->layers || proj < 0 || proj > 6)
+        return fail(BITNET_HIP_INVALID_CONFIG, "decoder_projection: layer %zu / projection %d out of range", layer, proj);
+    *out = dec->proj[layer * 7 + (size_t)proj];
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_decoder_set_norm(bitnet_hip_decoder *dec, size_t layer, int which, const float *gamma, int on_device,
+                                void *stream)
+{
+    if (!dec || !gamma) return fail(BITNET_HIP_NULL_POINTER, "decoder_set_norm: null argument");
+    if (layer >= dec->layers || which < 0 || which > 1)
+        return fail(BITNET_HIP_INVALID_CONFIG, "decoder_set_norm: layer %zu / which %d out of range", layer, which);
+    float *dst = dec->gamma + (layer * 2 + (size_t)which) * dec->hidden;
+    BITNET_HIP_TRY(hipMemcpyAsync(dst, gamma, sizeof(float) * dec->hidden,
+                                  on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, as_stream(stream)));
+    BITNET_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    return BITNET_HIP_OK;
+}
+
+size_t bitnet_hip_decoder_weight_bytes(const bitnet_hip_decoder *dec)
+{
+    if (!dec) return 0;
+    size_t total = 0;
+    for (auto *p : dec->proj) total += p->in_features * p->out_features / 4;
+    return total;
+}
+
+int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t m, float *x_out, float *q_last,
+                              float *k_last, void *stream)
+{
+    if (!dec || !x_in || !x_out) return fail(BITNET_HIP_NULL_POINTER, "decoder_decode: null argument");
+    if (m == 0) return BITNET_HIP_OK;
+    if (m > dec->max_tokens) {
+        size_t e[2] = {dec->max_tokens, dec->hidden}, a[2] = {m, dec->hidden};
+        return fail_shape(e, 2, a, 2, "tokens per decode step exceed max_tokens");
+    }
+    for (auto *p : dec->proj)
+        if (!p->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "decoder_decode: a projection has no weights yet");
+    hipStream_t s = as_stream(stream);
+    const size_t H = dec->hidden, F = dec->ffn, KV = dec->kv_heads * dec->head_dim;
+    const size_t group = dec->q_heads / dec->kv_heads;
+    int rc = BITNET_HIP_OK;
+    auto mm = [&](bitnet_hip_bitlinear *bl, const float *residual, float *out) {
+        if (rc != BITNET_HIP_OK) return;
+        rc = bitnet_hip_matmul_w2a8(bl->tiled, dec->a8, m, bl->out_features, bl->in_features, nullptr, bl->w_scale,
+                                    dec->a_scale, nullptr, residual, out, stream);
+    };
+    auto quant = [&](const float *x, const float *x2, size_t ldx, size_t k, int mode, const float *gamma) {
+        if (rc != BITNET_HIP_OK) return;
+        rc = launch_act_quant(x, x2, ldx, m, k, mode, group, dec->head_dim, gamma, dec->eps, dec->sum_order, dec->a8,
+                              dec->a_scale, nullptr, nullptr, s);
+    };
+    const float *x = x_in;
+    for (size_t l = 0; l < dec->layers; ++l) {
+        bitnet_hip_bitlinear **P = &dec->proj[l * 7];
+        const float *g_attn = dec->gamma + (l * 2) * H, *g_ffn = g_attn + H;
+        const bool last = l + 1 == dec->layers;
+        // hidden states alternate between x_out and the internal buffer so that the last block writes x_out
+        float *x2 = ((dec->layers - 1 - l) % 2 == 0) ? x_out : dec->ping;
+        quant(x, nullptr, H, H, BITNET_HIP_INPUT_PLAIN, g_attn);
+        mm(P[BITNET_HIP_PROJ_Q], nullptr, (last && q_last) ? q_last : dec->qb);
+        mm(P[BITNET_HIP_PROJ_K], nullptr, (last && k_last) ? k_last : dec->kb);
+        mm(P[BITNET_HIP_PROJ_V], nullptr, dec->vb);
+        quant(dec->vb, nullptr, KV, H, BITNET_HIP_INPUT_GQA_BROADCAST, nullptr);
+        mm(P[BITNET_HIP_PROJ_O], x, dec->x1);
+        quant(dec->x1, nullptr, H, H, BITNET_HIP_INPUT_PLAIN, g_ffn);
+        mm(P[BITNET_HIP_PROJ_GATE], nullptr, dec->gate);
+        mm(P[BITNET_HIP_PROJ_UP], nullptr, dec->up);
+        quant(dec->gate, dec->up, F, F, BITNET_HIP_INPUT_RELU2_MUL, nullptr);
+        mm(P[BITNET_HIP_PROJ_DOWN], dec->x1, x2);
+        x = x2;
+    }
+    return rc;
+}
+
+}  // extern "C"

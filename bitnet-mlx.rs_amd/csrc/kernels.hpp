@@ -1,0 +1,45 @@
+// Internal launchers, one per kernel family.  Arguments are validated by the C-ABI layer (api.hip);
+// these only pick a kernel variant and launch it.  All return a bitnet_hip_status.
+#pragma once
+#include "common.hpp"
+
+namespace bitnet {
+
+// ---- geometry of the re-tiled weight layout (see weight_prep.hip) ----
+constexpr int TILE_ROWS = 16;    // output rows per tile
+constexpr int TILE_K = 256;      // input columns per tile
+constexpr int TILE_BYTES = 1024; // TILE_ROWS * TILE_K / 4
+inline size_t row_blocks(size_t n) { return (n + TILE_ROWS - 1) / TILE_ROWS; }
+inline size_t k_tiles(size_t k) { return (k + TILE_K - 1) / TILE_K; }
+inline size_t tiled_bytes(size_t n, size_t k) { return row_blocks(n) * k_tiles(k) * (size_t)TILE_BYTES; }
+
+// act_quant.hip
+int launch_act_quant(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
+                     size_t gqa_group, size_t head_dim, const float *gamma, float eps, int sum_order,
+                     int8_t *q, float *a_scale, int32_t *a_sum, float *y, hipStream_t stream);
+
+// weight_prep.hip
+int launch_pack_2bit(const int8_t *q, size_t count, uint8_t *packed, hipStream_t stream);
+int launch_unpack_2bit(const uint8_t *packed, size_t count, int8_t *q, hipStream_t stream);
+// row_sums: device scratch of n doubles
+int launch_quantize_weights(const float *w, size_t n, size_t k, int method, float threshold_factor,
+                            double *row_sums, uint8_t *packed, float *w_scale, int8_t *q_i8,
+                            hipStream_t stream);
+int launch_retile(const uint8_t *packed, size_t n, size_t k, int layout, uint8_t *tiled, hipStream_t stream);
+int launch_untile(const uint8_t *tiled, size_t n, size_t k, uint8_t *packed, hipStream_t stream);
+
+// gemv_w2a8.hip
+int launch_gemv_rowmajor(const uint8_t *packed, const int8_t *a, int32_t *out, size_t n, size_t k,
+                         hipStream_t stream);
+// m <= GEMV_MAX_M tokens per launch
+constexpr int GEMV_MAX_M = 8;
+int launch_gemv_tiled(const uint8_t *tiled, const int8_t *a, size_t m, size_t n, size_t k, int32_t *acc,
+                      const float *w_scale, const float *a_scale, const float *bias, const float *residual,
+                      float *out, hipStream_t stream);
+
+// gemm_w2a8.hip
+int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, size_t m, size_t n, size_t k, int32_t *acc,
+                      const float *w_scale, const float *a_scale, const float *bias, const float *residual,
+                      float *out, hipStream_t stream);
+
+}  // namespace bitnet

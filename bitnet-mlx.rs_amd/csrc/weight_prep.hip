@@ -1,0 +1,221 @@
+// Weight-side kernels: ternarisation, 2-bit packing in the reference's byte format, and the re-tiling
+// into the layout the contraction kernels stream.  All of them run once per weight update.
+//
+// Reference byte format (bitnet-quant/src/quantization/packing.rs:353-394 over
+// bitnet-quant/src/quantization/utils.rs:434-451): code = w + 1 in {0,1,2}; flat element i lives in
+// byte i/4 at bits 2*(i mod 4); missing tail elements leave 0 bits.  Decoding maps 0,1,2,3 to
+// -1,0,+1,0 (bitnet-inference/src/engine/weight_conversion.rs:169-184).
+//
+// Re-tiled layout: the [n, k] matrix is cut into tiles of TILE_ROWS(16) rows x TILE_K(256) columns.  A
+// tile is 1 KiB = 64 slots of 16 bytes.  Slot s = kq*16 + r (kq = 0..3, r = 0..15) holds, for row r of the
+// tile, the 64 columns 64*kq .. 64*kq+63 as four dwords (dword t = columns 64*kq + 16t .. +15).  Inside a
+// dword the weight with column offset 4j + b sits at bits 2j + 8b, so that (dword >> 2j) & 0x03030303
+// yields the four code bytes of columns 4j..4j+3 in activation byte order.  Tiles are stored row-block
+// major: tile (rb, kt) starts at byte ((rb * k_tiles) + kt) * 1024.  A wavefront whose lane l loads slot
+// l reads one tile as a single contiguous 1 KiB burst; lanes l, l+16, l+32, l+48 share a row, which is
+// also the operand order of the 16x16x64 int8 MFMA (row/column = lane mod 16, k block = lane / 16).
+// Positions outside the matrix hold code 1 (weight 0) and code 3 is rewritten to code 1, so the
+// contraction kernels never see code 3.
+#include "kernels.hpp"
+
+namespace bitnet {
+
+namespace {
+
+__global__ __launch_bounds__(256) void pack_2bit_kernel(const int8_t *q, size_t count, uint8_t *packed,
+                                                        size_t nbytes)
+{
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nbytes) return;
+    unsigned byte = 0;
+    for (int j = 0; j < 4; ++j) {
+        size_t i = 4 * b + j;
+        if (i < count) byte |= ((unsigned)(q[i] + 1) & 3u) << (2 * j);
+    }
+    packed[b] = (uint8_t)byte;
+}
+
+__global__ __launch_bounds__(256) void unpack_2bit_kernel(const uint8_t *packed, size_t count, int8_t *q)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    unsigned code = (packed[i >> 2] >> (2 * (i & 3))) & 3u;
+    q[i] = code == 0 ? -1 : (code == 2 ? 1 : 0);
+}
+
+__device__ __forceinline__ double wave_sum_f64(double p)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) p = p + __shfl_xor(p, off, 64);
+    return p;
+}
+
+// Sum of |w| of one row in f64: lane l adds columns l, l+64, ... in ascending order, then the
+// butterfly.  One wavefront per row.
+__global__ __launch_bounds__(256) void absmean_rows_kernel(const float *w, size_t n, size_t k, double *row_sums)
+{
+    const int lane = threadIdx.x;
+    const size_t row = (size_t)blockIdx.x * blockDim.y + threadIdx.y;
+    if (row >= n) return;
+    const float *wr = w + row * k;
+    double s = 0.0;
+    for (size_t c = lane; c < k; c += 64) s = s + (double)fabsf(wr[c]);
+    s = wave_sum_f64(s);
+    if (lane == 0) row_sums[row] = s;
+}
+
+// Combines the row sums the same way (lane l takes rows l, l+64, ...) and writes mean|W| as f32.
+__global__ __launch_bounds__(64) void absmean_final_kernel(const double *row_sums, size_t n, size_t k, float *w_scale)
+{
+    const int lane = threadIdx.x;
+    double s = 0.0;
+    for (size_t r = lane; r < n; r += 64) s = s + row_sums[r];
+    s = wave_sum_f64(s);
+    if (lane == 0) *w_scale = (n == 0 || k == 0) ? 0.0f : (float)(s / ((double)n * (double)k));
+}
+
+__device__ __forceinline__ int ternarize_one(float w, int method, float s, float thr)
+{
+    if (method == BITNET_HIP_TERNARY_ABSMEAN_ROUNDCLIP) {
+        // RoundClip(w / s, -1, 1); s == 0 gives 0
+        if (s == 0.0f) return 0;
+        float r = roundf(__fdiv_rn(w, s));
+        if (r != r) return 0;
+        r = fminf(fmaxf(r, -1.0f), 1.0f);
+        return (int)r;
+    }
+    return w > thr ? 1 : (w < -thr ? -1 : 0);  // strict comparisons, bitnet-quant/src/simd/ternary.rs:75-83
+}
+
+__global__ __launch_bounds__(256) void ternarize_pack_kernel(const float *w, size_t count, int method,
+                                                             float factor, const float *w_scale,
+                                                             uint8_t *packed, int8_t *q_i8, size_t nbytes)
+{
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nbytes) return;
+    const float s = *w_scale;
+    const float thr = __fmul_rn(factor, s);
+    unsigned byte = 0;
+    for (int j = 0; j < 4; ++j) {
+        size_t i = 4 * b + j;
+        if (i < count) {
+            int t = ternarize_one(w[i], method, s, thr);
+            if (q_i8) q_i8[i] = (int8_t)t;
+            byte |= ((unsigned)(t + 1) & 3u) << (2 * j);
+        }
+    }
+    packed[b] = (uint8_t)byte;
+}
+
+__device__ __forceinline__ unsigned code_at(const uint8_t *packed, size_t e)
+{
+    return (packed[e >> 2] >> (2 * (e & 3))) & 3u;
+}
+
+// One thread builds one dword (16 weights of one row) of the tiled layout.
+__global__ __launch_bounds__(256) void retile_kernel(const uint8_t *packed, size_t n, size_t k, int layout,
+                                                     uint32_t *tiled, size_t kt_count, size_t total_dwords)
+{
+    size_t d = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (d >= total_dwords) return;
+    size_t tile = d >> 8;
+    unsigned wd = (unsigned)(d & 255);
+    unsigned slot = wd >> 2, t = wd & 3;
+    unsigned r = slot & 15, g = 4 * (slot >> 4) + t;
+    size_t rb = tile / kt_count, kt = tile % kt_count;
+    size_t row = rb * TILE_ROWS + r;
+    size_t kbase = kt * TILE_K + (size_t)g * 16;
+    uint32_t word = 0;
+    for (int j = 0; j < 16; ++j) {
+        size_t kk = kbase + j;
+        unsigned code = 1;
+        if (row < n && kk < k) {
+            size_t e = layout == BITNET_HIP_LAYOUT_OUT_IN ? row * k + kk : kk * n + row;
+            code = code_at(packed, e);
+            if (code == 3) code = 1;
+        }
+        word |= code << (2 * (j >> 2) + 8 * (j & 3));
+    }
+    tiled[d] = word;
+}
+
+// Inverse: one thread rebuilds one byte of the flat [n, k] packing.
+__global__ __launch_bounds__(256) void untile_kernel(const uint32_t *tiled, size_t n, size_t k, uint8_t *packed,
+                                                     size_t kt_count, size_t nbytes)
+{
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nbytes) return;
+    const size_t count = n * k;
+    unsigned byte = 0;
+    for (int j = 0; j < 4; ++j) {
+        size_t e = 4 * b + j;
+        if (e >= count) break;
+        size_t row = e / k, kk = e % k;
+        size_t tile = (row / TILE_ROWS) * kt_count + kk / TILE_K;
+        unsigned g = (unsigned)((kk % TILE_K) / 16), c = (unsigned)(kk % 16);
+        unsigned wd = (((g >> 2) * 16 + (unsigned)(row % TILE_ROWS)) << 2) + (g & 3);
+        uint32_t word = tiled[tile * 256 + wd];
+        byte |= ((word >> (2 * (c >> 2) + 8 * (c & 3))) & 3u) << (2 * j);
+    }
+    packed[b] = (uint8_t)byte;
+}
+
+inline unsigned blocks_for(size_t items, unsigned per_block) { return (unsigned)((items + per_block - 1) / per_block); }
+
+}  // namespace
+
+int launch_pack_2bit(const int8_t *q, size_t count, uint8_t *packed, hipStream_t stream)
+{
+    size_t nbytes = (count + 3) / 4;
+    if (nbytes == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL(pack_2bit_kernel, dim3(blocks_for(nbytes, 256)), dim3(256), 0, stream, q, count, packed, nbytes);
+    BITNET_HIP_CHECK_LAUNCH("pack_2bit_kernel");
+    return BITNET_HIP_OK;
+}
+
+int launch_unpack_2bit(const uint8_t *packed, size_t count, int8_t *q, hipStream_t stream)
+{
+    if (count == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL(unpack_2bit_kernel, dim3(blocks_for(count, 256)), dim3(256), 0, stream, packed, count, q);
+    BITNET_HIP_CHECK_LAUNCH("unpack_2bit_kernel");
+    return BITNET_HIP_OK;
+}
+
+int launch_quantize_weights(const float *w, size_t n, size_t k, int method, float threshold_factor,
+                            double *row_sums, uint8_t *packed, float *w_scale, int8_t *q_i8, hipStream_t stream)
+{
+    if (n > 0 && k > 0) {
+        hipLaunchKernelGGL(absmean_rows_kernel, dim3(blocks_for(n, 4)), dim3(64, 4), 0, stream, w, n, k, row_sums);
+        BITNET_HIP_CHECK_LAUNCH("absmean_rows_kernel");
+    }
+    hipLaunchKernelGGL(absmean_final_kernel, dim3(1), dim3(64), 0, stream, row_sums, n, k, w_scale);
+    BITNET_HIP_CHECK_LAUNCH("absmean_final_kernel");
+    size_t count = n * k, nbytes = (count + 3) / 4;
+    if (nbytes == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL(ternarize_pack_kernel, dim3(blocks_for(nbytes, 256)), dim3(256), 0, stream, w, count,
+                       method, threshold_factor, w_scale, packed, q_i8, nbytes);
+    BITNET_HIP_CHECK_LAUNCH("ternarize_pack_kernel");
+    return BITNET_HIP_OK;
+}
+
+int launch_retile(const uint8_t *packed, size_t n, size_t k, int layout, uint8_t *tiled, hipStream_t stream)
+{
+    size_t total_dwords = tiled_bytes(n, k) / 4;
+    if (total_dwords == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL(retile_kernel, dim3(blocks_for(total_dwords, 256)), dim3(256), 0, stream, packed, n, k,
+                       layout, reinterpret_cast<uint32_t *>(tiled), k_tiles(k), total_dwords);
+    BITNET_HIP_CHECK_LAUNCH("retile_kernel");
+    return BITNET_HIP_OK;
+}
+
+int launch_untile(const uint8_t *tiled, size_t n, size_t k, uint8_t *packed, hipStream_t stream)
+{
+    size_t nbytes = (n * k + 3) / 4;
+    if (nbytes == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL(untile_kernel, dim3(blocks_for(nbytes, 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint32_t *>(tiled), n, k, packed, k_tiles(k), nbytes);
+    BITNET_HIP_CHECK_LAUNCH("untile_kernel");
+    return BITNET_HIP_OK;
+}
+
+}  // namespace bitnet

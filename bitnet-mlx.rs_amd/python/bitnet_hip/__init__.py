@@ -1,0 +1,440 @@
+"""ctypes binding of libbitnet_hip.so (the C ABI declared in include/bitnet_hip.h).
+
+The library is the product; this module only moves pointers.  torch is used for device memory and
+streams, nothing else: no function here computes a result on the host or through torch operators, and
+loading fails loudly if the HIP library has not been built.
+
+Class and method names mirror the reference's Rust API so call sites read alike:
+  BitLinearConfig / BitLinear      bitnet-quant/src/bitlinear/layer.rs:20-109, forward.rs:14-51
+  TernaryProcessor                 bitnet-inference/src/engine/ternary_operations.rs:56-172
+  BitPacked2BitPacker              bitnet-quant/src/quantization/packing.rs:350-394
+  W2A8Backend.w2a8_gemv            bitnet-cuda/src/backend.rs:129-157
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from dataclasses import dataclass
+from pathlib import Path
+from typing import Optional, Sequence
+
+import torch
+
+_PKG_ROOT = Path(__file__).resolve().parents[2]
+LIB_PATH = _PKG_ROOT / "lib" / "libbitnet_hip.so"
+HEADER_PATH = _PKG_ROOT.parent / "include" / "bitnet_hip.h"
+
+OK = 0
+SHAPE_MISMATCH = 1
+INVALID_CONFIG = 2
+DEVICE_ERROR = 3
+MEMORY_ERROR = 4
+QUANTIZATION_ERROR = 5
+NOT_INITIALIZED = 6
+KERNEL_ERROR = 7
+NULL_POINTER = 8
+UNSUPPORTED = 9
+
+SUM_SEQUENTIAL = 0
+SUM_WAVE64 = 1
+LAYOUT_OUT_IN = 0
+LAYOUT_IN_OUT = 1
+TERNARY_ABSMEAN_ROUNDCLIP = 0
+TERNARY_MEAN_THRESHOLD = 1
+INPUT_PLAIN = 0
+INPUT_RELU2_MUL = 1
+INPUT_GQA_BROADCAST = 2
+PROJ_NAMES = ("q", "k", "v", "o", "gate", "up", "down")
+
+_STATUS_NAMES = {
+    1: "ShapeMismatch", 2: "InvalidConfig", 3: "DeviceError", 4: "MemoryError", 5: "QuantizationError",
+    6: "NotInitialized", 7: "KernelError", 8: "NullPointer", 9: "Unsupported",
+}
+
+
+class BitLinearError(RuntimeError):
+    """Mirror of BitLinearError (bitnet-quant/src/bitlinear/error.rs:10-84): `kind` is the variant name."""
+
+    def __init__(self, status: int, message: str, expected=None, actual=None):
+        super().__init__(f"{_STATUS_NAMES.get(status, status)}: {message}")
+        self.status = status
+        self.kind = _STATUS_NAMES.get(status, str(status))
+        self.expected = expected
+        self.actual = actual
+
+
+_lib = None
+
+
+def load_library() -> C.CDLL:
+    """Loads the built library; raises if it is missing (there is no fallback path)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise ImportError(
+            f"{LIB_PATH} is not built: run `make -C {_PKG_ROOT}` (needs hipcc); "
+            "the BitLinear HIP path has no CPU or PyTorch fallback"
+        )
+    lib = C.CDLL(str(LIB_PATH))
+    vp, sz, i32, f32 = C.c_void_p, C.c_size_t, C.c_int, C.c_float
+    sig = {
+        "bitnet_hip_last_error": (C.c_char_p, []),
+        "bitnet_hip_last_shape_mismatch": (i32, [C.POINTER(sz), C.POINTER(sz), C.POINTER(i32)]),
+        "bitnet_hip_init": (i32, [i32]),
+        "bitnet_hip_device_info": (i32, [C.c_char_p, sz, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz)]),
+        "bitnet_hip_quantize_activations_i8": (i32, [vp, vp, sz, sz, sz, i32, sz, sz, vp, f32, i32, vp, vp, vp, vp, vp]),
+        "bitnet_hip_packed_size": (sz, [sz]),
+        "bitnet_hip_pack_ternary_2bit": (i32, [vp, sz, vp, vp]),
+        "bitnet_hip_unpack_ternary_2bit": (i32, [vp, sz, vp, vp]),
+        "bitnet_hip_quantize_weights": (i32, [vp, sz, sz, i32, f32, vp, vp, vp, vp]),
+        "bitnet_hip_tiled_size": (sz, [sz, sz]),
+        "bitnet_hip_retile_weights": (i32, [vp, sz, sz, i32, vp, vp]),
+        "bitnet_hip_untile_weights": (i32, [vp, sz, sz, vp, vp]),
+        "bitnet_hip_gemv_w2a8": (i32, [vp, vp, vp, sz, sz, vp]),
+        "bitnet_hip_gemv_w2a8_checked": (i32, [vp, sz, vp, sz, vp, sz, sz, sz, vp]),
+        "bitnet_hip_matmul_w2a8": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp, vp, vp]),
+        "bitnet_hip_bitlinear_create": (i32, [sz, sz, i32, C.POINTER(vp)]),
+        "bitnet_hip_bitlinear_destroy": (None, [vp]),
+        "bitnet_hip_bitlinear_set_weights_f32": (i32, [vp, vp, sz, sz, i32, i32, i32, f32, vp]),
+        "bitnet_hip_bitlinear_set_weights_packed": (i32, [vp, vp, sz, f32, i32, vp]),
+        "bitnet_hip_bitlinear_set_bias": (i32, [vp, vp, sz, i32, vp]),
+        "bitnet_hip_bitlinear_get_quantized": (i32, [vp, C.POINTER(f32), vp, sz]),
+        "bitnet_hip_bitlinear_workspace_size": (sz, [vp, sz]),
+        "bitnet_hip_bitlinear_forward": (i32, [vp, vp, C.POINTER(sz), i32, vp, f32, i32, vp, vp, vp, sz, vp, vp, vp, vp]),
+        "bitnet_hip_decoder_create": (i32, [sz, sz, sz, sz, sz, sz, f32, i32, sz, C.POINTER(vp)]),
+        "bitnet_hip_decoder_destroy": (None, [vp]),
+        "bitnet_hip_decoder_projection": (i32, [vp, sz, i32, C.POINTER(vp)]),
+        "bitnet_hip_decoder_set_norm": (i32, [vp, sz, i32, vp, i32, vp]),
+        "bitnet_hip_decoder_weight_bytes": (sz, [vp]),
+        "bitnet_hip_decoder_decode": (i32, [vp, vp, sz, vp, vp, vp, vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    lib._bitnet_declared = tuple(sig)
+    _lib = lib
+    return lib
+
+
+def declared_symbols():
+    """Entry points this binding declares; tests compare them with the header and with the library."""
+    lib = load_library()
+    return sorted(lib._bitnet_declared)
+
+
+def _check(status: int):
+    if status == OK:
+        return
+    lib = load_library()
+    msg = lib.bitnet_hip_last_error().decode()
+    expected = actual = None
+    if status == SHAPE_MISMATCH:
+        e = (C.c_size_t * 4)()
+        a = (C.c_size_t * 4)()
+        ar = C.c_int(0)
+        er = lib.bitnet_hip_last_shape_mismatch(e, a, C.byref(ar))
+        expected, actual = list(e[:er]), list(a[: ar.value])
+    raise BitLinearError(status, msg, expected, actual)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream(stream=None):
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return C.c_void_p(s.cuda_stream)
+
+
+def _dev(t: torch.Tensor, dtype, name: str):
+    if not t.is_cuda:
+        raise BitLinearError(DEVICE_ERROR, f"{name} must live on the GPU")
+    if t.dtype != dtype:
+        raise BitLinearError(INVALID_CONFIG, f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise BitLinearError(INVALID_CONFIG, f"{name} must be contiguous")
+    return t
+
+
+def init(device: int = 0):
+    _check(load_library().bitnet_hip_init(device))
+
+
+def device_info():
+    lib = load_library()
+    name = C.create_string_buffer(64)
+    cus, mhz, mem = C.c_int(0), C.c_int(0), C.c_size_t(0)
+    _check(lib.bitnet_hip_device_info(name, 64, C.byref(cus), C.byref(mhz), C.byref(mem)))
+    return {"arch": name.value.decode(), "compute_units": cus.value, "clock_mhz": mhz.value, "total_mem": mem.value}
+
+
+# ---- raw operators ------------------------------------------------------------------------------
+
+def quantize_activations_i8(x: torch.Tensor, gamma: Optional[torch.Tensor] = None, eps: float = 1e-5,
+                            sum_order: int = SUM_WAVE64, x2: Optional[torch.Tensor] = None,
+                            input_mode: int = INPUT_PLAIN, gqa_group: int = 1, head_dim: int = 1,
+                            want_sum: bool = False, want_y: bool = False, stream=None):
+    """Fused RMSNorm (if gamma) + per-token absmax int8 quantisation of a [m, k] f32 matrix."""
+    lib = load_library()
+    _dev(x, torch.float32, "x")
+    m, src_cols = x.shape
+    k = src_cols * gqa_group if input_mode == INPUT_GQA_BROADCAST else src_cols
+    q = torch.empty((m, k), dtype=torch.int8, device=x.device)
+    a_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
+    a_sum = torch.empty((m,), dtype=torch.int32, device=x.device) if want_sum else None
+    y = torch.empty((m, k), dtype=torch.float32, device=x.device) if want_y else None
+    _check(lib.bitnet_hip_quantize_activations_i8(_ptr(x), _ptr(x2), src_cols, m, k, input_mode, gqa_group, head_dim,
+                                                  _ptr(gamma), eps, sum_order, _ptr(q), _ptr(a_scale), _ptr(a_sum),
+                                                  _ptr(y), _stream(stream)))
+    return q, a_scale, a_sum, y
+
+
+def packed_size(count: int) -> int:
+    return load_library().bitnet_hip_packed_size(count)
+
+
+def tiled_size(n: int, k: int) -> int:
+    return load_library().bitnet_hip_tiled_size(n, k)
+
+
+def pack_ternary_2bit(q: torch.Tensor, stream=None) -> torch.Tensor:
+    _dev(q, torch.int8, "q")
+    out = torch.empty((packed_size(q.numel()),), dtype=torch.uint8, device=q.device)
+    _check(load_library().bitnet_hip_pack_ternary_2bit(_ptr(q), q.numel(), _ptr(out), _stream(stream)))
+    return out
+
+
+def unpack_ternary_2bit(packed: torch.Tensor, count: int, stream=None) -> torch.Tensor:
+    _dev(packed, torch.uint8, "packed")
+    if packed.numel() < packed_size(count):
+        raise BitLinearError(SHAPE_MISMATCH, "packed buffer too short", [packed_size(count)], [packed.numel()])
+    out = torch.empty((count,), dtype=torch.int8, device=packed.device)
+    _check(load_library().bitnet_hip_unpack_ternary_2bit(_ptr(packed), count, _ptr(out), _stream(stream)))
+    return out
+
+
+def quantize_weights(w: torch.Tensor, method: int = TERNARY_ABSMEAN_ROUNDCLIP, threshold_factor: float = 0.5,
+                     want_i8: bool = False, stream=None):
+    """Ternarise + pack an [n, k] f32 matrix on the GPU.  Returns (packed u8, w_scale f32[1], q i8 or None)."""
+    _dev(w, torch.float32, "w")
+    n, k = w.shape
+    packed = torch.empty((packed_size(n * k),), dtype=torch.uint8, device=w.device)
+    w_scale = torch.empty((1,), dtype=torch.float32, device=w.device)
+    q = torch.empty((n, k), dtype=torch.int8, device=w.device) if want_i8 else None
+    _check(load_library().bitnet_hip_quantize_weights(_ptr(w), n, k, method, threshold_factor, _ptr(packed),
+                                                      _ptr(w_scale), _ptr(q), _stream(stream)))
+    return packed, w_scale, q
+
+
+def retile_weights(packed: torch.Tensor, n: int, k: int, layout: int = LAYOUT_OUT_IN, stream=None) -> torch.Tensor:
+    _dev(packed, torch.uint8, "packed")
+    if packed.numel() < packed_size(n * k):
+        raise BitLinearError(SHAPE_MISMATCH, "packed buffer too short", [packed_size(n * k)], [packed.numel()])
+    tiled = torch.empty((tiled_size(n, k),), dtype=torch.uint8, device=packed.device)
+    _check(load_library().bitnet_hip_retile_weights(_ptr(packed), n, k, layout, _ptr(tiled), _stream(stream)))
+    return tiled
+
+
+def untile_weights(tiled: torch.Tensor, n: int, k: int, stream=None) -> torch.Tensor:
+    _dev(tiled, torch.uint8, "tiled")
+    packed = torch.empty((packed_size(n * k),), dtype=torch.uint8, device=tiled.device)
+    _check(load_library().bitnet_hip_untile_weights(_ptr(tiled), n, k, _ptr(packed), _stream(stream)))
+    return packed
+
+
+def matmul_w2a8(tiled: torch.Tensor, a: torch.Tensor, n: int, w_scale: Optional[torch.Tensor] = None,
+                a_scale: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+                residual: Optional[torch.Tensor] = None, want_acc: bool = True, want_out: bool = True, stream=None):
+    """acc[m,n] (int32) and/or out[m,n] (f32) from re-tiled weights and int8 activations [m, k]."""
+    _dev(tiled, torch.uint8, "tiled")
+    _dev(a, torch.int8, "a")
+    m, k = a.shape
+    if tiled.numel() < tiled_size(n, k):
+        raise BitLinearError(SHAPE_MISMATCH, "tiled buffer too short", [tiled_size(n, k)], [tiled.numel()])
+    acc = torch.empty((m, n), dtype=torch.int32, device=a.device) if want_acc else None
+    out = torch.empty((m, n), dtype=torch.float32, device=a.device) if want_out else None
+    _check(load_library().bitnet_hip_matmul_w2a8(_ptr(tiled), _ptr(a), m, n, k, _ptr(acc), _ptr(w_scale), _ptr(a_scale),
+                                                 _ptr(bias), _ptr(residual), _ptr(out), _stream(stream)))
+    return acc, out
+
+
+class W2A8Backend:
+    """Mirror of CudaBackend's W2A8 entry (bitnet-cuda/src/backend.rs:129-157)."""
+
+    def w2a8_gemv(self, weights: torch.Tensor, activations: torch.Tensor, output: torch.Tensor, m: int, k: int,
+                  stream=None):
+        _dev(weights, torch.uint8, "weights")
+        _dev(activations, torch.int8, "activations")
+        _dev(output, torch.int32, "output")
+        _check(load_library().bitnet_hip_gemv_w2a8_checked(_ptr(weights), weights.numel(), _ptr(activations),
+                                                           activations.numel(), _ptr(output), output.numel(), m, k,
+                                                           _stream(stream)))
+
+
+class BitPacked2BitPacker:
+    """Mirror of BitPacked2BitPacker (bitnet-quant/src/quantization/packing.rs:350-394)."""
+
+    def pack(self, weights: torch.Tensor) -> torch.Tensor:
+        return pack_ternary_2bit(weights.reshape(-1))
+
+    def unpack(self, packed: torch.Tensor, element_count: int) -> torch.Tensor:
+        return unpack_ternary_2bit(packed, element_count)
+
+
+class TernaryProcessor:
+    """Mirror of TernaryProcessor (bitnet-inference/src/engine/ternary_operations.rs:56-172), int8 kept."""
+
+    def quantize_activations(self, x: torch.Tensor):
+        x2 = x.reshape(-1, x.shape[-1]) if x.dim() != 2 else x
+        q, a_scale, _, _ = quantize_activations_i8(x2.contiguous())
+        return q, a_scale
+
+
+# ---- BitLinear ------------------------------------------------------------------------------------
+
+@dataclass
+class BitLinearConfig:
+    """Subset of BitLinearConfig (layer.rs:20-75) that affects arithmetic."""
+    in_features: int = 512
+    out_features: int = 512
+    use_bias: bool = False
+    ternary_method: int = TERNARY_ABSMEAN_ROUNDCLIP
+    threshold_factor: float = 0.5
+    rms_norm_eps: float = 1e-5
+    sum_order: int = SUM_WAVE64
+
+
+class BitLinear:
+    """Mirror of BitLinear + BitLinearForward (layer.rs:82-109,113-179; forward.rs:14-136)."""
+
+    def __init__(self, config: BitLinearConfig, layer_name: str = "", _handle=None, _owner=None):
+        self.config = config
+        self.layer_name = layer_name
+        self._owner = _owner
+        lib = load_library()
+        if _handle is not None:
+            self._h = _handle
+            return
+        h = C.c_void_p()
+        _check(lib.bitnet_hip_bitlinear_create(config.in_features, config.out_features, int(config.use_bias), C.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        if getattr(self, "_owner", None) is None and getattr(self, "_h", None) and _lib is not None:
+            _lib.bitnet_hip_bitlinear_destroy(self._h)
+            self._h = None
+
+    def update_weights(self, w: torch.Tensor, layout: int = LAYOUT_OUT_IN, stream=None):
+        """BitLinear::update_weights (layer.rs:299-326): latent f32 weights, host or device."""
+        if w.dtype != torch.float32 or w.dim() != 2 or not w.is_contiguous():
+            raise BitLinearError(INVALID_CONFIG, "weights must be a contiguous 2-D f32 tensor")
+        _check(load_library().bitnet_hip_bitlinear_set_weights_f32(
+            self._h, _ptr(w), w.shape[0], w.shape[1], layout, int(w.is_cuda), self.config.ternary_method,
+            self.config.threshold_factor, _stream(stream)))
+
+    def set_quantized_weights(self, packed: torch.Tensor, w_scale: float, stream=None):
+        if packed.dtype != torch.uint8 or not packed.is_contiguous():
+            raise BitLinearError(INVALID_CONFIG, "packed weights must be contiguous u8")
+        _check(load_library().bitnet_hip_bitlinear_set_weights_packed(self._h, _ptr(packed), packed.numel(), w_scale,
+                                                                      int(packed.is_cuda), _stream(stream)))
+
+    def update_bias(self, bias: torch.Tensor, stream=None):
+        if bias.dtype != torch.float32 or not bias.is_contiguous():
+            raise BitLinearError(INVALID_CONFIG, "bias must be contiguous f32")
+        _check(load_library().bitnet_hip_bitlinear_set_bias(self._h, _ptr(bias), bias.numel(), int(bias.is_cuda),
+                                                            _stream(stream)))
+
+    def get_quantized_weights(self):
+        """(packed bytes as a CPU u8 tensor in the reference format, w_scale)."""
+        n = packed_size(self.config.in_features * self.config.out_features)
+        buf = torch.empty((n,), dtype=torch.uint8)
+        s = C.c_float(0)
+        _check(load_library().bitnet_hip_bitlinear_get_quantized(self._h, C.byref(s), _ptr(buf), n))
+        return buf, s.value
+
+    def forward(self, x: torch.Tensor, gamma: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None,
+                debug: bool = False, stream=None):
+        """BitLinearForward::forward (forward.rs:55-92).  x: [m,in] or [b,s,in] f32 on the GPU."""
+        _dev(x, torch.float32, "input")
+        lib = load_library()
+        dims = (C.c_size_t * max(x.dim(), 1))(*x.shape)
+        nout = self.config.out_features
+        out_shape = tuple(x.shape[:-1]) + (nout,) if x.dim() >= 1 else (nout,)
+        m = 1
+        for d in x.shape[:-1]:
+            m *= d
+        out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
+        q = a_scale = acc = None
+        if debug and x.dim() in (2, 3) and x.shape[-1] == self.config.in_features:
+            q = torch.empty((m, self.config.in_features), dtype=torch.int8, device=x.device)
+            a_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
+            acc = torch.empty((m, nout), dtype=torch.int32, device=x.device)
+        _check(lib.bitnet_hip_bitlinear_forward(self._h, _ptr(x), dims, x.dim(), _ptr(gamma), self.config.rms_norm_eps,
+                                                self.config.sum_order, _ptr(residual), _ptr(out), None, 0, _ptr(q),
+                                                _ptr(a_scale), _ptr(acc), _stream(stream)))
+        if debug:
+            return out, q, a_scale, acc
+        return out
+
+    def forward_batch(self, x: torch.Tensor):
+        """BitLinear::forward_batch (forward.rs:270-297): rank >= 2 required."""
+        if x.dim() < 2:
+            raise BitLinearError(SHAPE_MISMATCH, "forward_batch needs at least 2 dimensions",
+                                 [1, 1, self.config.in_features], list(x.shape))
+        return self.forward(x)
+
+
+class DecoderProjections:
+    """The seven BitLinear projections of a stack of decoder blocks at decode time."""
+
+    def __init__(self, layers: int, hidden: int = 2560, ffn: int = 6912, q_heads: int = 20, kv_heads: int = 5,
+                 head_dim: int = 128, eps: float = 1e-5, sum_order: int = SUM_WAVE64, max_tokens: int = 8):
+        lib = load_library()
+        h = C.c_void_p()
+        _check(lib.bitnet_hip_decoder_create(layers, hidden, ffn, q_heads, kv_heads, head_dim, eps, sum_order,
+                                             max_tokens, C.byref(h)))
+        self._h = h
+        self.layers, self.hidden, self.ffn = layers, hidden, ffn
+        self.q_heads, self.kv_heads, self.head_dim = q_heads, kv_heads, head_dim
+        self.kv_dim = kv_heads * head_dim
+        self.eps, self.sum_order = eps, sum_order
+
+    def __del__(self):
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.bitnet_hip_decoder_destroy(self._h)
+            self._h = None
+
+    def proj_shape(self, proj: int):
+        outs = (self.hidden, self.kv_dim, self.kv_dim, self.hidden, self.ffn, self.ffn, self.hidden)
+        ins = (self.hidden,) * 6 + (self.ffn,)
+        return outs[proj], ins[proj]
+
+    def projection(self, layer: int, proj: int) -> BitLinear:
+        h = C.c_void_p()
+        _check(load_library().bitnet_hip_decoder_projection(self._h, layer, proj, C.byref(h)))
+        n, k = self.proj_shape(proj)
+        return BitLinear(BitLinearConfig(in_features=k, out_features=n, rms_norm_eps=self.eps,
+                                         sum_order=self.sum_order), f"layer{layer}.{PROJ_NAMES[proj]}",
+                         _handle=h, _owner=self)
+
+    def set_norm(self, layer: int, which: int, gamma: torch.Tensor, stream=None):
+        if gamma.dtype != torch.float32 or gamma.numel() != self.hidden or not gamma.is_contiguous():
+            raise BitLinearError(SHAPE_MISMATCH, "norm weight", [self.hidden], list(gamma.shape))
+        _check(load_library().bitnet_hip_decoder_set_norm(self._h, layer, which, _ptr(gamma), int(gamma.is_cuda),
+                                                          _stream(stream)))
+
+    def weight_bytes(self) -> int:
+        return load_library().bitnet_hip_decoder_weight_bytes(self._h)
+
+    def decode(self, x: torch.Tensor, out: Optional[torch.Tensor] = None, want_qk: bool = False, stream=None):
+        _dev(x, torch.float32, "x")
+        m = x.shape[0]
+        if out is None:
+            out = torch.empty_like(x)
+        q = torch.empty((m, self.hidden), dtype=torch.float32, device=x.device) if want_qk else None
+        k = torch.empty((m, self.kv_dim), dtype=torch.float32, device=x.device) if want_qk else None
+        _check(load_library().bitnet_hip_decoder_decode(self._h, _ptr(x), m, _ptr(out), _ptr(q), _ptr(k),
+                                                        _stream(stream)))
+        return (out, q, k) if want_qk else out

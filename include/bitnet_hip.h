@@ -1,0 +1,238 @@
+/*
+ * bitnet_hip.h — C ABI of the MI355X (gfx950) BitLinear W1.58A8 forward path.
+ *
+ * This is the boundary a Rust `extern "C"` block (or any FFI) binds.  Plain pointers and sizes only.
+ * Unless a parameter is marked HOST, every data pointer is a DEVICE pointer owned by the caller, the
+ * call is asynchronous on `stream` (a hipStream_t passed as void*, NULL = the null stream), and the
+ * caller keeps the buffers alive until the stream has passed the call.
+ *
+ * Every function returns a bitnet_hip_status.  On failure nothing is launched and a message is kept
+ * per thread (bitnet_hip_last_error).  Nothing here aborts or throws.
+ *
+ * Each entry point cites the reference interface it replaces (paths relative to the root of
+ * leizerowicz/bitnet-mlx.rs).
+ */
+#ifndef BITNET_HIP_H
+#define BITNET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  One per error variant of the reference that can occur on this path:
+ * BitLinearError (bitnet-quant/src/bitlinear/error.rs:10-84) and CudaError
+ * (bitnet-cuda/src/error.rs:7-60). */
+typedef enum bitnet_hip_status {
+    BITNET_HIP_OK = 0,
+    BITNET_HIP_SHAPE_MISMATCH = 1,  /* BitLinearError::ShapeMismatch / CudaError::IncompatibleShapes */
+    BITNET_HIP_INVALID_CONFIG = 2,  /* BitLinearError::ConfigError, InvalidConfig / CudaError::InvalidConfig */
+    BITNET_HIP_DEVICE_ERROR = 3,    /* BitLinearError::DeviceError / CudaError::DeviceError */
+    BITNET_HIP_MEMORY_ERROR = 4,    /* BitLinearError::MemoryError / CudaError::MemoryAllocation */
+    BITNET_HIP_QUANTIZATION_ERROR = 5, /* BitLinearError::QuantizationError */
+    BITNET_HIP_NOT_INITIALIZED = 6, /* BitLinearError::NotInitialized (weights never set) */
+    BITNET_HIP_KERNEL_ERROR = 7,    /* CudaError::KernelExecution */
+    BITNET_HIP_NULL_POINTER = 8,    /* a required pointer argument was NULL */
+    BITNET_HIP_UNSUPPORTED = 9      /* CudaError::UnsupportedOperation */
+} bitnet_hip_status;
+
+/* Order of the f32 sum of squares inside RMSNorm. */
+#define BITNET_HIP_SUM_SEQUENTIAL 0 /* one running sum, k ascending: the literal order of
+                                       bitnet-inference/src/engine/inference_integration.rs:476 (slow) */
+#define BITNET_HIP_SUM_WAVE64 1     /* 64 lane-strided partials + xor butterfly (default, one wavefront pass) */
+
+/* Weight matrix orientation handed to set_weights. */
+#define BITNET_HIP_LAYOUT_OUT_IN 0 /* [out_features, in_features], bitnet-quant/src/bitlinear/layer.rs:86,122 */
+#define BITNET_HIP_LAYOUT_IN_OUT 1 /* [in_features, out_features], bitnet-inference/src/engine/inference_integration.rs:431 */
+
+/* Weight ternarisation recipes (TernaryMethod, bitnet-quant/src/quantization/weights.rs:17-30). */
+#define BITNET_HIP_TERNARY_ABSMEAN_ROUNDCLIP 0 /* w_scale = mean|W|, q = RoundClip(W / w_scale, -1, 1):
+                                                  BitNet b1.58; RoundClip = quantization/utils.rs:391-393 */
+#define BITNET_HIP_TERNARY_MEAN_THRESHOLD 1    /* q = sign(w) * [|w| > factor * mean|w|], scale = mean|W|
+                                                  (bitnet-quant/src/simd/ternary.rs:27-41,87-101) */
+
+/* Input transform fused in front of the activation quantiser. */
+#define BITNET_HIP_INPUT_PLAIN 0     /* row = x[m, :] */
+#define BITNET_HIP_INPUT_RELU2_MUL 1 /* row = x2[m, :] * relu(x[m, :])^2   (x = gate, x2 = up):
+                                        bitnet-inference/src/engine/transformer_layers.rs:307-316,605-618 */
+#define BITNET_HIP_INPUT_GQA_BROADCAST 2 /* row[h*hd + d] = x[m, (h / group)*hd + d]: one-token attention,
+                                            every query head reads its KV group's value head */
+
+/* ---- library ---------------------------------------------------------------------------------- */
+
+/* Message of the last failing call on this thread ("" if none).  Never NULL. */
+const char *bitnet_hip_last_error(void);
+
+/* Expected / actual dimensions recorded by the last BITNET_HIP_SHAPE_MISMATCH on this thread
+ * (BitLinearError::ShapeMismatch{expected, actual}).  Each array receives up to 4 entries; the
+ * return value is the number of valid entries in `expected` (actual_rank likewise). */
+int bitnet_hip_last_shape_mismatch(size_t expected[4], size_t actual[4], int *actual_rank);
+
+/* Selects `device`, checks that it is a gfx950 part and prepares per-device state.  Replaces
+ * CudaBackend::new + check_device_capabilities (bitnet-cuda/src/backend.rs:42-93,192-213). */
+int bitnet_hip_init(int device);
+
+/* Name (gcnArchName), compute-unit count and memory clock of the current device.  HOST outputs. */
+int bitnet_hip_device_info(char *arch_name, size_t arch_name_len, int *compute_units, int *clock_mhz,
+                           size_t *total_mem_bytes);
+
+/* ---- activation side -------------------------------------------------------------------------- */
+
+/* Fused RMSNorm + per-token absmax int8 quantiser (one wavefront per token row).
+ *   replaces LayerOperation::rms_normalize (bitnet-inference/src/engine/inference_integration.rs:449-493)
+ *   followed by TernaryProcessor::quantize_activations (bitnet-inference/src/engine/ternary_operations.rs:117-172).
+ *   x        [m, k] f32, row stride ldx elements
+ *   x2       second input for BITNET_HIP_INPUT_RELU2_MUL (same shape/stride), else NULL
+ *   gamma    [k] f32 RMSNorm weight, or NULL for no normalisation (plain quantize_activations)
+ *   q        [m, k] int8 out;  a_scale [m] f32 out (127/absmax, 1.0 for an all-zero row)
+ *   a_sum    [m] int32 out or NULL: sum over k of q[m, k]
+ *   y_f32    [m, k] f32 out or NULL: the normalised row before quantisation
+ *   gqa_group / head_dim: only for BITNET_HIP_INPUT_GQA_BROADCAST (x is then [m, k / gqa_group]). */
+int bitnet_hip_quantize_activations_i8(const float *x, const float *x2, size_t ldx, size_t m, size_t k,
+                                       int input_mode, size_t gqa_group, size_t head_dim,
+                                       const float *gamma, float eps, int sum_order, int8_t *q,
+                                       float *a_scale, int32_t *a_sum, float *y_f32, void *stream);
+
+/* ---- weight side ------------------------------------------------------------------------------ */
+
+/* Bytes of `count` ternary values in the reference's 2-bit format: (count + 3) / 4
+ * (bitnet-quant/src/quantization/packing.rs:353-376, bitnet-cuda/src/backend.rs:226). */
+size_t bitnet_hip_packed_size(size_t count);
+
+/* 2-bit pack / unpack in the reference's byte format: code = w + 1, element i of a byte at bits
+ * 2*(i mod 4); decode 0,1,2,3 -> -1,0,+1,0.
+ *   replaces BitPacked2BitPacker::{pack,unpack} (bitnet-quant/src/quantization/packing.rs:353-394),
+ *   BitUtils::{pack_bits,unpack_bits} (bitnet-quant/src/quantization/utils.rs:434-475) and
+ *   WeightConverter::convert_ternary_weights (bitnet-inference/src/engine/weight_conversion.rs:143-191). */
+int bitnet_hip_pack_ternary_2bit(const int8_t *q, size_t count, uint8_t *packed, void *stream);
+int bitnet_hip_unpack_ternary_2bit(const uint8_t *packed, size_t count, int8_t *q, void *stream);
+
+/* Ternarise an f32 weight matrix [n, k] (row-major) and pack it in the reference's byte format.
+ *   replaces SimdTernaryOps::{compute_absmean, quantize_batch} (bitnet-quant/src/simd/ternary.rs:27-66)
+ *   / BitNetWeightQuantizer::quantize (bitnet-quant/src/quantization/weights.rs:568-611) + the packer.
+ *   method   BITNET_HIP_TERNARY_*;  threshold_factor only for MEAN_THRESHOLD (reference: 0.5 / 0.7)
+ *   packed   [(n*k+3)/4] u8 out;  w_scale  1 f32 out (device);  q_i8 [n*k] int8 out or NULL. */
+int bitnet_hip_quantize_weights(const float *w, size_t n, size_t k, int method, float threshold_factor,
+                                uint8_t *packed, float *w_scale, int8_t *q_i8, void *stream);
+
+/* Device layout the decode GEMV streams: tiles of 16 rows x 256 columns, 1 KiB each, stored
+ * [row_block][k_tile][row][64 bytes]; rows/columns past n/k are zero weights; code 3 is rewritten to
+ * code 1 (both decode to 0).  bitnet_hip_tiled_size gives the byte size for an [n, k] matrix.
+ * retile/untile are inverse bijections on the n*k valid positions (up to the code 3 -> 1 rewrite). */
+size_t bitnet_hip_tiled_size(size_t n, size_t k);
+int bitnet_hip_retile_weights(const uint8_t *packed, size_t n, size_t k, int layout, uint8_t *tiled,
+                              void *stream);
+int bitnet_hip_untile_weights(const uint8_t *tiled, size_t n, size_t k, uint8_t *packed, void *stream);
+
+/* ---- contraction ------------------------------------------------------------------------------ */
+
+/* W2A8 GEMV on the reference's flat row-major packing: out[n] = sum_k w[n,k] * a[k] in int32.
+ *   replaces launch_w2a8_gemv_optimized (bitnet-cuda/src/kernels/w2a8_gemv.cu:188-214) and
+ *   CudaBackend::w2a8_gemv + validate_w2a8_dimensions (bitnet-cuda/src/backend.rs:129-157,217-257).
+ *   weights [(m*k+3)/4] u8, activations [k] i8, output [m] i32; m = output features, k = input features
+ *   (the reference's naming).  The *_checked form also takes the element counts of the three buffers
+ *   and returns BITNET_HIP_SHAPE_MISMATCH exactly where validate_w2a8_dimensions errs. */
+int bitnet_hip_gemv_w2a8(const uint8_t *weights, const int8_t *activations, int32_t *output, size_t m,
+                         size_t k, void *stream);
+int bitnet_hip_gemv_w2a8_checked(const uint8_t *weights, size_t weights_len, const int8_t *activations,
+                                 size_t activations_len, int32_t *output, size_t output_len, size_t m,
+                                 size_t k, void *stream);
+
+/* BitLinear contraction + epilogue on re-tiled weights, any token count m:
+ *   acc[t, n] = sum_k a[t, k] * w[n, k]                          (int32, exact)
+ *   out[t, n] = (float(acc) * *w_scale) / a_scale[t] (+ bias[n]) (+ residual[t, n])
+ *   replaces SimdMatrixOps::{ternary_gemv_scalar, ternary_gemm_scalar}
+ *   (bitnet-quant/src/simd/matrix.rs:471-490, :256-282), BitLinear::quantized_matmul
+ *   (bitnet-quant/src/bitlinear/forward.rs:153-223) and TernaryProcessor::ternary_matmul
+ *   (bitnet-inference/src/engine/ternary_operations.rs:87-113,283-338).
+ *   Small m runs the HBM-bound decode GEMV, large m the int8 MFMA GEMM.
+ *   acc / out may each be NULL (at least one must be given); out needs w_scale and a_scale. */
+int bitnet_hip_matmul_w2a8(const uint8_t *tiled, const int8_t *a, size_t m, size_t n, size_t k,
+                           int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,
+                           const float *residual, float *out, void *stream);
+
+/* ---- BitLinear layer object ------------------------------------------------------------------- */
+
+typedef struct bitnet_hip_bitlinear bitnet_hip_bitlinear; /* opaque; mirrors BitLinear, layer.rs:82-109 */
+
+/* BitLinear::new(BitLinearConfig{in_features,out_features,use_bias,..}) (layer.rs:113-179).  The layer
+ * holds no weights until one of the set_weights calls (forward then returns NOT_INITIALIZED). */
+int bitnet_hip_bitlinear_create(size_t in_features, size_t out_features, int use_bias,
+                                bitnet_hip_bitlinear **layer);
+void bitnet_hip_bitlinear_destroy(bitnet_hip_bitlinear *layer);
+
+/* BitLinear::update_weights (layer.rs:299-326) + get_quantized_weights (layer.rs:236-294): takes the
+ * latent f32 matrix (`layout` orientation; HOST pointer if on_device == 0), ternarises it with `method`
+ * on the GPU, packs and re-tiles it.  `rows`/`cols` are checked against the layer's shape. */
+int bitnet_hip_bitlinear_set_weights_f32(bitnet_hip_bitlinear *layer, const float *w, size_t rows,
+                                         size_t cols, int layout, int on_device, int method,
+                                         float threshold_factor, void *stream);
+/* Pre-quantised weights in the reference's 2-bit byte format ([out,in] flat), plus their scale:
+ * BitLinearForward::forward_with_quantized_weights (forward.rs:46-50) / GGUF-decoded tensors. */
+int bitnet_hip_bitlinear_set_weights_packed(bitnet_hip_bitlinear *layer, const uint8_t *packed,
+                                            size_t packed_len, float w_scale, int on_device, void *stream);
+/* BitLinear::update_bias (layer.rs:329-352): INVALID_CONFIG if the layer was created without bias. */
+int bitnet_hip_bitlinear_set_bias(bitnet_hip_bitlinear *layer, const float *bias, size_t len, int on_device,
+                                  void *stream);
+
+/* HOST outputs: the scale and the packed bytes the layer holds (the reference's QuantizedWeight,
+ * bitnet-quant/src/quantization/weights.rs:158-175).  Synchronises the device. */
+int bitnet_hip_bitlinear_get_quantized(bitnet_hip_bitlinear *layer, float *w_scale, uint8_t *packed,
+                                       size_t packed_len);
+
+/* Bytes of device workspace forward needs for m tokens. */
+size_t bitnet_hip_bitlinear_workspace_size(const bitnet_hip_bitlinear *layer, size_t m);
+
+/* BitLinearForward::forward (forward.rs:55-92) / BitLinearLayer::forward (transformer_layers.rs:119-201):
+ * x has `rank` dimensions `dims` (HOST array); rank 2 [m, in] or rank 3 [b, s, in] (flattened to
+ * [b*s, in]); anything else, or a last dimension != in_features, is BITNET_HIP_SHAPE_MISMATCH.
+ *   gamma      NULL, or the RMSNorm weight [in] applied before quantisation (eps, sum_order as above)
+ *   residual   NULL or [m, out] f32 added after the bias
+ *   workspace  device buffer of at least workspace_size(m) bytes, or NULL to let the call allocate
+ *              stream-ordered scratch itself
+ *   debug outputs (each may be NULL): q [m,in] int8, a_scale [m] f32, acc [m,out] int32. */
+int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, const size_t *dims, int rank,
+                                 const float *gamma, float eps, int sum_order, const float *residual,
+                                 float *out, void *workspace, size_t workspace_bytes, int8_t *dbg_q,
+                                 float *dbg_a_scale, int32_t *dbg_acc, void *stream);
+
+/* ---- decoder projections (seven BitLinear layers per block) ------------------------------------ */
+
+typedef struct bitnet_hip_decoder bitnet_hip_decoder; /* opaque */
+
+#define BITNET_HIP_PROJ_Q 0
+#define BITNET_HIP_PROJ_K 1
+#define BITNET_HIP_PROJ_V 2
+#define BITNET_HIP_PROJ_O 3
+#define BITNET_HIP_PROJ_GATE 4
+#define BITNET_HIP_PROJ_UP 5
+#define BITNET_HIP_PROJ_DOWN 6
+
+/* A stack of `layers` decoder blocks' BitLinear projections (TransformerBlock,
+ * bitnet-inference/src/engine/transformer_layers.rs:626-710; MultiHeadAttention q/k/v/o :470-475,545;
+ * FeedForwardNetwork :603-623) at decode time with no KV history: per block
+ *   a = quant(rmsnorm(x, g_attn)); q,k,v = Wq a, Wk a, Wv a; x1 = x + Wo quant(gqa_broadcast(v));
+ *   b = quant(rmsnorm(x1, g_ffn)); x2 = x1 + Wd quant(Wu b * relu(Wg b)^2).
+ * max_tokens bounds m of decode() and sizes the internal activation buffers. */
+int bitnet_hip_decoder_create(size_t layers, size_t hidden, size_t ffn, size_t q_heads, size_t kv_heads,
+                              size_t head_dim, float eps, int sum_order, size_t max_tokens,
+                              bitnet_hip_decoder **dec);
+void bitnet_hip_decoder_destroy(bitnet_hip_decoder *dec);
+/* The BitLinear object of projection `proj` of block `layer` (owned by the decoder). */
+int bitnet_hip_decoder_projection(bitnet_hip_decoder *dec, size_t layer, int proj, bitnet_hip_bitlinear **out);
+/* RMSNorm weights of a block: which = 0 (before attention) or 1 (before the FFN); [hidden] f32. */
+int bitnet_hip_decoder_set_norm(bitnet_hip_decoder *dec, size_t layer, int which, const float *gamma,
+                                int on_device, void *stream);
+/* Packed-weight bytes one decode step streams (sum of n*k/4 over all projections). */
+size_t bitnet_hip_decoder_weight_bytes(const bitnet_hip_decoder *dec);
+/* One decode step: x_in [m, hidden] -> x_out [m, hidden] through all blocks.  q_last / k_last (may be
+ * NULL) receive the last block's q [m, hidden] and k [m, kv_heads*head_dim] projections. */
+int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t m, float *x_out,
+                              float *q_last, float *k_last, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITNET_HIP_H */

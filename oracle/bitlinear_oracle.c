@@ -1,0 +1,476 @@
+/*
+ * CPU oracle for the BitLinear W1.58A8 forward path.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  It is a plain-C restatement of the
+ * arithmetic of the reference (BitNet-Rust, leizerowicz/bitnet-mlx.rs) for one path only, so that
+ * the HIP kernels can be checked bit for bit.  Only tests, the smoke check and the CPU-baseline leg
+ * of the benchmark may load it; the shipped library never links or calls it.
+ *
+ * Every f32 operation below is a single IEEE-754 binary32 operation, round-to-nearest-even.  The
+ * file must be compiled with -ffp-contract=off and without any fast-math option (see the Makefile
+ * next to it); round() is C roundf (halves away from zero), which is what Rust's f32::round does.
+ *
+ * Parity status of each function (what pins it besides this restatement):
+ *   orc_pack_2bit / orc_unpack_2bit      pinned: byte fixtures and round trips held by the reference's tests
+ *   orc_round_clip, orc_ternarize_*      pinned: reference tables (round_clip ties, strict '>' threshold)
+ *   orc_absmean                          pinned: reference vector [1,-2,3,-4] -> 2.5; order declared here
+ *   orc_gemv_w2a8 / orc_gemm_w2a8        pinned: reference 3x4 GEMV / 2x3x2 GEMM vectors + brute force
+ *   orc_quantize_activations_i8          pinned by invariants (max|q|=127, oddness, zero rows, exact ties);
+ *                                        the reference holds no exact-value vector for it
+ *   orc_rmsnorm                          the reference holds NO fixture: pinned by closed forms (constant
+ *                                        rows, one-hot rows), scale equivariance and an f64 bound; the
+ *                                        bits of the ORC_SUM_WAVE64 order are a declaration of this build
+ *   orc_epilogue                         two IEEE f32 operations; closed form
+ *   orc_quantize_weights_reference       PARITY UNPINNED for the f32 statistics: the reference computes
+ *                                        mean/sum with candle-core 0.8 (third party, not vendored), whose
+ *                                        summation order is not visible; this restatement accumulates in
+ *                                        f64.  Ternary values are pinned by the threshold tests.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_SUM_SEQUENTIAL 0 /* literal order of the reference: one running f32 sum, k ascending   */
+#define ORC_SUM_WAVE64 1     /* declared order the HIP kernel follows: 64 strided partials + butterfly */
+
+/* ------------------------------------------------------------------------------------------------
+ * R1  RMSNorm.   reference: bitnet-inference/src/engine/inference_integration.rs:449-493
+ *   sum_squares = sum(x*x)            (:476, f32, sequential)
+ *   rms = sqrt(sum_squares / K + eps) (:477)
+ *   y[i] = (x[i] / rms) * g[i]        (:481)  divide first, then multiply
+ * ---------------------------------------------------------------------------------------------- */
+
+/* Sum of squares of one row in the requested order.
+ *
+ * ORC_SUM_WAVE64: the row is cut into chunks of 4 consecutive elements; chunk c belongs to lane
+ * c mod 64; a lane adds the squares of its chunks in ascending chunk order and, inside a chunk, in
+ * ascending element order, starting from +0.  Elements past K count as 0.  The 64 partials are then
+ * combined by a butterfly: for off = 32,16,8,4,2,1: p[l] = p[l] + p[l ^ off].  IEEE addition is
+ * commutative, so all lanes end with the same value; lane 0's is returned. */
+float orc_sum_squares(const float *x, size_t k, int order)
+{
+    if (order == ORC_SUM_SEQUENTIAL) {
+        float s = 0.0f;
+        for (size_t i = 0; i < k; ++i) {
+            float sq = x[i] * x[i];
+            s = s + sq;
+        }
+        return s;
+    }
+    float p[64], t[64];
+    for (int l = 0; l < 64; ++l) p[l] = 0.0f;
+    size_t chunks = (k + 3) / 4;
+    for (size_t c = 0; c < chunks; ++c) {
+        int l = (int)(c % 64);
+        for (size_t j = 0; j < 4; ++j) {
+            size_t i = 4 * c + j;
+            float v = i < k ? x[i] : 0.0f;
+            float sq = v * v;
+            p[l] = p[l] + sq;
+        }
+    }
+    for (int off = 32; off >= 1; off >>= 1) {
+        for (int l = 0; l < 64; ++l) t[l] = p[l] + p[l ^ off];
+        memcpy(p, t, sizeof p);
+    }
+    return p[0];
+}
+
+void orc_rmsnorm(const float *x, const float *g, float eps, size_t m, size_t k, int order, float *y)
+{
+    for (size_t r = 0; r < m; ++r) {
+        const float *xr = x + r * k;
+        float *yr = y + r * k;
+        float ss = orc_sum_squares(xr, k, order);
+        float mean = ss / (float)k;
+        float rms = sqrtf(mean + eps);
+        for (size_t i = 0; i < k; ++i) {
+            float n = xr[i] / rms;
+            yr[i] = n * g[i];
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * A1  per-token absmax int8 quantisation.
+ *   reference: bitnet-inference/src/engine/ternary_operations.rs:117-172
+ *   absmax = fold(0, max) of |x|                  (:143-145; f32::max ignores a NaN operand)
+ *   scale  = absmax > 0 ? 127 / absmax : 1.0      (:147-151)
+ *   q      = clamp(round(x * scale), -128, 127)   (:158-161)
+ * The reference then returns q / scale as f32 (:162); the integer q is what the build keeps.  A NaN
+ * survives round/clamp in Rust and would cast to 0 with `as i8`; the same is done here.
+ * row_sum (optional) receives sum_k q[k] as int32; the kernels use it to undo their +1 weight code.
+ * ---------------------------------------------------------------------------------------------- */
+static int8_t orc_q8(float v, float scale)
+{
+    float t = roundf(v * scale);
+    if (t != t) return 0;
+    if (t < -128.0f) t = -128.0f;
+    if (t > 127.0f) t = 127.0f;
+    return (int8_t)t;
+}
+
+void orc_quantize_activations_i8(const float *x, size_t m, size_t k, int8_t *q, float *a_scale,
+                                 int32_t *row_sum)
+{
+    for (size_t r = 0; r < m; ++r) {
+        const float *xr = x + r * k;
+        float absmax = 0.0f;
+        for (size_t i = 0; i < k; ++i) absmax = fmaxf(absmax, fabsf(xr[i]));
+        float scale = absmax > 0.0f ? 127.0f / absmax : 1.0f;
+        int32_t s = 0;
+        for (size_t i = 0; i < k; ++i) {
+            int8_t v = orc_q8(xr[i], scale);
+            q[r * k + i] = v;
+            s += v;
+        }
+        a_scale[r] = scale;
+        if (row_sum) row_sum[r] = s;
+    }
+}
+
+/* The reference's own return value: fake-quantised activations q / scale (ternary_operations.rs:162). */
+void orc_fake_quantize_activations(const float *x, size_t m, size_t k, float *out)
+{
+    for (size_t r = 0; r < m; ++r) {
+        const float *xr = x + r * k;
+        float absmax = 0.0f;
+        for (size_t i = 0; i < k; ++i) absmax = fmaxf(absmax, fabsf(xr[i]));
+        float scale = absmax > 0.0f ? 127.0f / absmax : 1.0f;
+        for (size_t i = 0; i < k; ++i) {
+            float t = roundf(xr[i] * scale);
+            if (t < -128.0f) t = -128.0f;
+            if (t > 127.0f) t = 127.0f;
+            out[r * k + i] = t / scale;
+        }
+    }
+}
+
+/* Fused form the HIP kernel implements: RMSNorm (if g != NULL) followed by A1 on the normalised row. */
+void orc_rmsnorm_quantize_i8(const float *x, const float *g, float eps, size_t m, size_t k, int order,
+                             int8_t *q, float *a_scale, int32_t *row_sum)
+{
+    if (!g) {
+        orc_quantize_activations_i8(x, m, k, q, a_scale, row_sum);
+        return;
+    }
+    float *y = (float *)malloc(sizeof(float) * (k ? k : 1));
+    for (size_t r = 0; r < m; ++r) {
+        orc_rmsnorm(x + r * k, g, eps, 1, k, order, y);
+        orc_quantize_activations_i8(y, 1, k, q + r * k, a_scale + r, row_sum ? row_sum + r : NULL);
+    }
+    free(y);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * W1  weight ternarisation.
+ * ---------------------------------------------------------------------------------------------- */
+
+/* RoundClip.  reference: bitnet-quant/src/quantization/utils.rs:391-393  x.round().clamp(lo, hi) */
+float orc_round_clip(float x, float lo, float hi)
+{
+    float r = roundf(x);
+    if (r < lo) r = lo;
+    if (r > hi) r = hi;
+    return r;
+}
+
+/* mean|W| of a [rows, cols] tensor.
+ *   reference: bitnet-quant/src/simd/ternary.rs:103-106 (sum of |x| / len) and
+ *              bitnet-quant/src/bitlinear/memory/scaling_factors.rs:505-515 (abs().mean_all()).
+ * The reference sums in f32; a running f32 sum over millions of values of size 0.016 stops growing
+ * once the addend falls under half an ulp, so the order is declared here instead and carried in
+ * f64: per row, lane l (of 64) adds |w[k]| for k = l, l+64, ... in ascending order; the 64 partials
+ * are combined by the butterfly off = 32..1 (p[l] += p[l^off]); the row sums are then combined the
+ * same way (lane l takes rows l, l+64, ...; butterfly).  The mean is total / (rows*cols) in f64,
+ * rounded once to f32.  rows*cols == 0 gives 0 (ternary.rs:61-63). */
+static double orc_wave64_sum_f64(const double *v, size_t n)
+{
+    double p[64], t[64];
+    for (int l = 0; l < 64; ++l) p[l] = 0.0;
+    for (size_t i = 0; i < n; ++i) p[i % 64] = p[i % 64] + v[i];
+    for (int off = 32; off >= 1; off >>= 1) {
+        for (int l = 0; l < 64; ++l) t[l] = p[l] + p[l ^ off];
+        memcpy(p, t, sizeof p);
+    }
+    return p[0];
+}
+
+float orc_absmean(const float *w, size_t rows, size_t cols)
+{
+    if (rows == 0 || cols == 0) return 0.0f;
+    double *row_sum = (double *)malloc(sizeof(double) * rows);
+    double *tmp = (double *)malloc(sizeof(double) * cols);
+    for (size_t r = 0; r < rows; ++r) {
+        for (size_t c = 0; c < cols; ++c) tmp[c] = (double)fabsf(w[r * cols + c]);
+        row_sum[r] = orc_wave64_sum_f64(tmp, cols);
+    }
+    double total = orc_wave64_sum_f64(row_sum, rows);
+    free(tmp);
+    free(row_sum);
+    return (float)(total / ((double)rows * (double)cols));
+}
+
+/* BitNet b1.58 recipe: q = RoundClip(w / w_scale, -1, 1), w_scale = mean|W|; w_scale == 0 gives q = 0. */
+void orc_ternarize_roundclip(const float *w, size_t n, float w_scale, int8_t *q)
+{
+    for (size_t i = 0; i < n; ++i) {
+        if (w_scale == 0.0f) { q[i] = 0; continue; }
+        float r = orc_round_clip(w[i] / w_scale, -1.0f, 1.0f);
+        q[i] = (r != r) ? 0 : (int8_t)r;
+    }
+}
+
+/* Threshold form.  reference: bitnet-quant/src/simd/ternary.rs:68-85 and
+ * bitnet-quant/src/quantization/weights.rs:482-496: +1 if w > thr, -1 if w < -thr, else 0 (strict). */
+void orc_ternarize_threshold(const float *w, size_t n, float thr, int8_t *q)
+{
+    for (size_t i = 0; i < n; ++i) q[i] = w[i] > thr ? 1 : (w[i] < -thr ? -1 : 0);
+}
+
+/* Dequantise.  reference: bitnet-quant/src/simd/ternary.rs:87-101 */
+void orc_dequantize_ternary(const int8_t *q, size_t n, float scale, float *out)
+{
+    for (size_t i = 0; i < n; ++i) out[i] = q[i] == 1 ? scale : (q[i] == -1 ? -scale : 0.0f);
+}
+
+/* The reference's default BitLinear weight recipe.
+ *   reference: bitnet-quant/src/quantization/weights.rs:568-611 with
+ *     normalize_before_quantize :671-686   (w - mean) / sqrt(var + 1e-8)
+ *     handle_outliers           :688-699   clamp to mean' +- t * mean|w'|   (t = outlier_threshold)
+ *     mean-threshold ternarise  :384-394   thr = factor * mean|w''|, strict '>' (:482-496)
+ *     compute_ternary_scale     :546-559   sum(w''*q) / sum(q*q), 1.0 if the denominator < f32::EPSILON
+ * Statistics are accumulated sequentially in f64 and rounded to f32 where the reference holds an f32
+ * scalar (candle's own order is not visible: parity unpinned for those scalars). */
+float orc_quantize_weights_reference(const float *w, size_t n, int normalize, float outlier_threshold,
+                                     float threshold_factor, int8_t *q, float *processed /* n, scratch */)
+{
+    if (n == 0) return 1.0f;
+    for (size_t i = 0; i < n; ++i) processed[i] = w[i];
+    if (normalize) {
+        double s = 0.0;
+        for (size_t i = 0; i < n; ++i) s += processed[i];
+        float mean = (float)(s / (double)n);
+        double v = 0.0;
+        for (size_t i = 0; i < n; ++i) {
+            float d = processed[i] - mean;
+            v += (double)(d * d);
+        }
+        float var = (float)(v / (double)n);
+        float sd = sqrtf(var + 1e-8f);
+        for (size_t i = 0; i < n; ++i) processed[i] = (processed[i] - mean) / sd;
+    }
+    if (outlier_threshold > 0.0f) {
+        double s = 0.0, a = 0.0;
+        for (size_t i = 0; i < n; ++i) { s += processed[i]; a += fabsf(processed[i]); }
+        float mean = (float)(s / (double)n);
+        float mad = (float)(a / (double)n);
+        float lo = mean - outlier_threshold * mad, hi = mean + outlier_threshold * mad;
+        for (size_t i = 0; i < n; ++i) {
+            float t = processed[i];
+            processed[i] = t < lo ? lo : (t > hi ? hi : t);
+        }
+    }
+    double a = 0.0;
+    for (size_t i = 0; i < n; ++i) a += fabsf(processed[i]);
+    float mean_abs = (float)(a / (double)n);
+    float thr = mean_abs * threshold_factor;
+    orc_ternarize_threshold(processed, n, thr, q);
+    double num = 0.0, den = 0.0;
+    for (size_t i = 0; i < n; ++i) {
+        num += (double)(processed[i] * (float)q[i]);
+        den += (double)((float)q[i] * (float)q[i]);
+    }
+    float fnum = (float)num, fden = (float)den;
+    if (fabsf(fden) < 1.1920929e-07f) return 1.0f;
+    return fnum / fden;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * P1  2-bit packing.
+ *   reference: bitnet-quant/src/quantization/packing.rs:353-394 (code = w + 1) through
+ *              bitnet-quant/src/quantization/utils.rs:434-475 (element i of a byte at bits 2*(i mod 4),
+ *              missing tail elements contribute 0 bits)
+ *   decode:    bitnet-inference/src/engine/weight_conversion.rs:169-184 and
+ *              bitnet-inference/src/gguf.rs:1130-1141: 0 -> -1, 1 -> 0, 2 -> +1, 3 -> 0
+ * ---------------------------------------------------------------------------------------------- */
+size_t orc_packed_size(size_t n) { return (n + 3) / 4; }
+
+size_t orc_pack_2bit(const int8_t *q, size_t n, uint8_t *out)
+{
+    size_t nb = orc_packed_size(n);
+    memset(out, 0, nb);
+    for (size_t i = 0; i < n; ++i) {
+        uint8_t code = (uint8_t)(q[i] + 1) & 3u;
+        out[i / 4] |= (uint8_t)(code << (2 * (i % 4)));
+    }
+    return nb;
+}
+
+void orc_unpack_2bit(const uint8_t *packed, size_t n, int8_t *q)
+{
+    static const int8_t lut[4] = {-1, 0, 1, 0};
+    for (size_t i = 0; i < n; ++i) q[i] = lut[(packed[i / 4] >> (2 * (i % 4))) & 3u];
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * G1 / G2  contraction in int32 over packed weights.
+ *   I/O contract: bitnet-cuda/src/kernels/w2a8_gemv.cu:100-105 (u8 [n*k/4], i8 [k] -> i32 [n])
+ *   semantics:    bitnet-quant/src/simd/matrix.rs:471-490 (GEMV), :256-282 (GEMM), with the f32
+ *                 accumulation replaced by exact int32 (|acc| <= 127*K)
+ *   weights are [n_out, k] row-major, flat-packed (element index n*k + kk), as the reference packs them.
+ * ---------------------------------------------------------------------------------------------- */
+void orc_gemm_w2a8(const uint8_t *packed, const int8_t *a, int32_t *acc, size_t m, size_t n_out, size_t k)
+{
+    static const int8_t lut[4] = {-1, 0, 1, 0};
+    /* integer arithmetic: exact and order-free, so the rows may be shared among threads */
+#pragma omp parallel
+    {
+        int8_t *wrow = (int8_t *)malloc(k ? k : 1);
+#pragma omp for schedule(static)
+        for (long long n = 0; n < (long long)n_out; ++n) {
+            for (size_t kk = 0; kk < k; ++kk) {
+                size_t i = (size_t)n * k + kk;
+                wrow[kk] = lut[(packed[i / 4] >> (2 * (i % 4))) & 3u];
+            }
+            for (size_t r = 0; r < m; ++r) {
+                const int8_t *ar = a + r * k;
+                int32_t s = 0;
+                for (size_t kk = 0; kk < k; ++kk) s += (int32_t)ar[kk] * (int32_t)wrow[kk];
+                acc[r * n_out + (size_t)n] = s;
+            }
+        }
+        free(wrow);
+    }
+}
+
+void orc_gemv_w2a8(const uint8_t *packed, const int8_t *a, int32_t *out, size_t n_out, size_t k)
+{
+    orc_gemm_w2a8(packed, a, out, 1, n_out, k);
+}
+
+/* Same contraction on unpacked ternary weights (for the reference's i8-matrix fixtures). */
+void orc_gemm_ternary_i8(const int8_t *w, const int8_t *a, int32_t *acc, size_t m, size_t n_out, size_t k)
+{
+    for (size_t r = 0; r < m; ++r)
+        for (size_t n = 0; n < n_out; ++n) {
+            int32_t s = 0;
+            for (size_t kk = 0; kk < k; ++kk) s += (int32_t)a[r * k + kk] * (int32_t)w[n * k + kk];
+            acc[r * n_out + n] = s;
+        }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * E1  epilogue:  out = (float(acc) * w_scale) / a_scale[m]  (+ bias[n]) (+ residual[m,n])
+ *   reference: weight scale multiply bitnet-quant/src/bitlinear/forward.rs:253-255; the division
+ *   by the activation scale is ternary_operations.rs:162; bias add forward.rs:117-130; the residual
+ *   add is the block's `x + sublayer(x)` (bitnet-inference/src/engine/transformer_layers.rs:689-699).
+ * ---------------------------------------------------------------------------------------------- */
+void orc_epilogue(const int32_t *acc, float w_scale, const float *a_scale, const float *bias,
+                  const float *residual, size_t m, size_t n_out, float *out)
+{
+    for (size_t r = 0; r < m; ++r)
+        for (size_t n = 0; n < n_out; ++n) {
+            float v = (float)acc[r * n_out + n] * w_scale;
+            v = v / a_scale[r];
+            if (bias) v = v + bias[n];
+            if (residual) v = v + residual[r * n_out + n];
+            out[r * n_out + n] = v;
+        }
+}
+
+/* Whole BitLinear forward on packed weights: (RMSNorm) -> A1 -> contraction -> E1.
+ * q_out / a_scale_out / acc_out may be NULL. */
+void orc_bitlinear_forward(const float *x, size_t m, size_t k, const float *g, float eps, int order,
+                           const uint8_t *packed, size_t n_out, float w_scale, const float *bias,
+                           const float *residual, float *out, int8_t *q_out, float *a_scale_out,
+                           int32_t *acc_out)
+{
+    int8_t *q = q_out ? q_out : (int8_t *)malloc(m * k + 1);
+    float *as = a_scale_out ? a_scale_out : (float *)malloc(sizeof(float) * (m ? m : 1));
+    int32_t *acc = acc_out ? acc_out : (int32_t *)malloc(sizeof(int32_t) * (m * n_out + 1));
+    orc_rmsnorm_quantize_i8(x, g, eps, m, k, order, q, as, NULL);
+    orc_gemm_w2a8(packed, q, acc, m, n_out, k);
+    orc_epilogue(acc, w_scale, as, bias, residual, m, n_out, out);
+    if (!q_out) free(q);
+    if (!a_scale_out) free(as);
+    if (!acc_out) free(acc);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * L1  layer composition.
+ *   ReLU^2: bitnet-inference/src/engine/transformer_layers.rs:307-316  max(0,x) then squared
+ *   FFN:    :603-623  down( up(x) * relu2(gate(x)) )
+ * ---------------------------------------------------------------------------------------------- */
+void orc_relu2_mul(const float *gate, const float *up, size_t n, float *h)
+{
+    for (size_t i = 0; i < n; ++i) {
+        float r = gate[i] > 0.0f ? gate[i] : 0.0f;
+        float sq = r * r;
+        h[i] = up[i] * sq;
+    }
+}
+
+/* Single-token attention stand-in used by the decode-layer workload: with one query and one key the
+ * softmax weight is 1, so each query head's output equals its KV group's value head.
+ * v: [m, kv_heads*head_dim]  ->  out: [m, q_heads*head_dim]. */
+void orc_gqa_broadcast_v(const float *v, size_t m, size_t q_heads, size_t kv_heads, size_t head_dim, float *out)
+{
+    size_t group = q_heads / kv_heads;
+    for (size_t r = 0; r < m; ++r)
+        for (size_t h = 0; h < q_heads; ++h)
+            memcpy(out + (r * q_heads + h) * head_dim, v + (r * kv_heads + h / group) * head_dim,
+                   sizeof(float) * head_dim);
+}
+
+/* One decoder layer's seven projections at decode time (no KV history):
+ *   a  = quant(rmsnorm(x, g_attn));  q = Wq a; k = Wk a; v = Wv a
+ *   o  = Wo quant(gqa_broadcast(v));  x1 = x + o
+ *   b  = quant(rmsnorm(x1, g_ffn));  gate = Wg b; up = Wu b
+ *   x2 = x1 + Wd quant(up * relu2(gate))
+ * Weight pointers are packed [n_out, k]; scales per projection in w_scale[7] ordered q,k,v,o,gate,up,down.
+ * q_out/k_out ([m,hidden], [m,kv_dim]) receive the otherwise unused q and k projections. */
+void orc_decoder_layer(const float *x, size_t m, size_t hidden, size_t ffn, size_t q_heads, size_t kv_heads,
+                       size_t head_dim, const float *g_attn, const float *g_ffn, float eps, int order,
+                       const uint8_t *const w[7], const float w_scale[7], float *x_out, float *q_out,
+                       float *k_out)
+{
+    size_t kv_dim = kv_heads * head_dim;
+    int8_t *a8 = (int8_t *)malloc(m * (hidden > ffn ? hidden : ffn));
+    float *as = (float *)malloc(sizeof(float) * m);
+    int32_t *acc = (int32_t *)malloc(sizeof(int32_t) * m * (hidden > ffn ? hidden : ffn));
+    float *v = (float *)malloc(sizeof(float) * m * kv_dim);
+    float *att = (float *)malloc(sizeof(float) * m * hidden);
+    float *x1 = (float *)malloc(sizeof(float) * m * hidden);
+    float *gate = (float *)malloc(sizeof(float) * m * ffn);
+    float *up = (float *)malloc(sizeof(float) * m * ffn);
+    float *h = (float *)malloc(sizeof(float) * m * ffn);
+
+    orc_rmsnorm_quantize_i8(x, g_attn, eps, m, hidden, order, a8, as, NULL);
+    orc_gemm_w2a8(w[0], a8, acc, m, hidden, hidden);
+    orc_epilogue(acc, w_scale[0], as, NULL, NULL, m, hidden, q_out);
+    orc_gemm_w2a8(w[1], a8, acc, m, kv_dim, hidden);
+    orc_epilogue(acc, w_scale[1], as, NULL, NULL, m, kv_dim, k_out);
+    orc_gemm_w2a8(w[2], a8, acc, m, kv_dim, hidden);
+    orc_epilogue(acc, w_scale[2], as, NULL, NULL, m, kv_dim, v);
+
+    orc_gqa_broadcast_v(v, m, q_heads, kv_heads, head_dim, att);
+    orc_quantize_activations_i8(att, m, hidden, a8, as, NULL);
+    orc_gemm_w2a8(w[3], a8, acc, m, hidden, hidden);
+    orc_epilogue(acc, w_scale[3], as, NULL, x, m, hidden, x1);
+
+    orc_rmsnorm_quantize_i8(x1, g_ffn, eps, m, hidden, order, a8, as, NULL);
+    orc_gemm_w2a8(w[4], a8, acc, m, ffn, hidden);
+    orc_epilogue(acc, w_scale[4], as, NULL, NULL, m, ffn, gate);
+    orc_gemm_w2a8(w[5], a8, acc, m, ffn, hidden);
+    orc_epilogue(acc, w_scale[5], as, NULL, NULL, m, ffn, up);
+
+    orc_relu2_mul(gate, up, m * ffn, h);
+    orc_quantize_activations_i8(h, m, ffn, a8, as, NULL);
+    orc_gemm_w2a8(w[6], a8, acc, m, hidden, ffn);
+    orc_epilogue(acc, w_scale[6], as, NULL, x1, m, hidden, x_out);
+
+    free(a8); free(as); free(acc); free(v); free(att); free(x1); free(gate); free(up); free(h);
+}

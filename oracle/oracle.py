@@ -1,0 +1,276 @@
+"""numpy-facing wrapper of the CPU oracle (oracle/libbitnet_oracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the benchmark's CPU-baseline
+leg.  The shipped package never imports it.  Build the library with `make -C oracle`.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+_DIR = Path(__file__).resolve().parent
+LIB_PATH = _DIR / "libbitnet_oracle.so"
+
+SUM_SEQUENTIAL = 0
+SUM_WAVE64 = 1
+
+_lib = None
+
+
+def build():
+    subprocess.run(["make", "-C", str(_DIR)], check=True, capture_output=True)
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            build()
+        _lib = C.CDLL(str(LIB_PATH))
+        _lib.orc_sum_squares.restype = C.c_float
+        _lib.orc_absmean.restype = C.c_float
+        _lib.orc_round_clip.restype = C.c_float
+        _lib.orc_quantize_weights_reference.restype = C.c_float
+        _lib.orc_pack_2bit.restype = C.c_size_t
+        _lib.orc_packed_size.restype = C.c_size_t
+        _lib.cpu_baseline_max_threads.restype = C.c_int
+        _lib.cpu_baseline_isa.restype = C.c_int
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _sz(v):
+    return C.c_size_t(int(v))
+
+
+def sum_squares(x, order=SUM_WAVE64) -> np.float32:
+    x = _f32(x).reshape(-1)
+    return np.float32(lib().orc_sum_squares(_p(x), _sz(x.size), C.c_int(order)))
+
+
+def rmsnorm(x, g, eps, order=SUM_WAVE64):
+    x = _f32(x)
+    g = _f32(g)
+    m, k = x.shape
+    y = np.empty_like(x)
+    lib().orc_rmsnorm(_p(x), _p(g), C.c_float(eps), _sz(m), _sz(k), C.c_int(order), _p(y))
+    return y
+
+
+def quantize_activations_i8(x):
+    """A1: returns (q int8 [m,k], a_scale f32 [m], row_sum int32 [m])."""
+    x = _f32(x)
+    m, k = x.shape
+    q = np.empty((m, k), dtype=np.int8)
+    s = np.empty((m,), dtype=np.float32)
+    rs = np.empty((m,), dtype=np.int32)
+    lib().orc_quantize_activations_i8(_p(x), _sz(m), _sz(k), _p(q), _p(s), _p(rs))
+    return q, s, rs
+
+
+def fake_quantize_activations(x):
+    x = _f32(x)
+    m, k = x.shape
+    out = np.empty_like(x)
+    lib().orc_fake_quantize_activations(_p(x), _sz(m), _sz(k), _p(out))
+    return out
+
+
+def rmsnorm_quantize_i8(x, g, eps, order=SUM_WAVE64):
+    x = _f32(x)
+    g = None if g is None else _f32(g)
+    m, k = x.shape
+    q = np.empty((m, k), dtype=np.int8)
+    s = np.empty((m,), dtype=np.float32)
+    rs = np.empty((m,), dtype=np.int32)
+    lib().orc_rmsnorm_quantize_i8(_p(x), _p(g), C.c_float(eps), _sz(m), _sz(k), C.c_int(order), _p(q), _p(s), _p(rs))
+    return q, s, rs
+
+
+def round_clip(x, lo=-1.0, hi=1.0) -> float:
+    return float(lib().orc_round_clip(C.c_float(x), C.c_float(lo), C.c_float(hi)))
+
+
+def absmean(w) -> np.float32:
+    w = _f32(w)
+    if w.ndim == 1:
+        w = w.reshape(1, -1)
+    rows, cols = w.shape
+    return np.float32(lib().orc_absmean(_p(w), _sz(rows), _sz(cols)))
+
+
+def ternarize_roundclip(w, w_scale):
+    w = _f32(w)
+    q = np.empty(w.shape, dtype=np.int8)
+    lib().orc_ternarize_roundclip(_p(w), _sz(w.size), C.c_float(w_scale), _p(q))
+    return q
+
+
+def ternarize_threshold(w, thr):
+    w = _f32(w)
+    q = np.empty(w.shape, dtype=np.int8)
+    lib().orc_ternarize_threshold(_p(w), _sz(w.size), C.c_float(thr), _p(q))
+    return q
+
+
+def dequantize_ternary(q, scale):
+    q = np.ascontiguousarray(q, dtype=np.int8)
+    out = np.empty(q.shape, dtype=np.float32)
+    lib().orc_dequantize_ternary(_p(q), _sz(q.size), C.c_float(scale), _p(out))
+    return out
+
+
+def quantize_weights_absmean(w):
+    """BitNet b1.58 recipe: (q int8 [n,k], w_scale f32)."""
+    w = _f32(w)
+    s = absmean(w)
+    return ternarize_roundclip(w, s), s
+
+
+def quantize_weights_reference(w, normalize=True, outlier_threshold=3.0, threshold_factor=0.7):
+    w = _f32(w)
+    q = np.empty(w.shape, dtype=np.int8)
+    scratch = np.empty(w.size, dtype=np.float32)
+    s = lib().orc_quantize_weights_reference(_p(w), _sz(w.size), C.c_int(int(normalize)), C.c_float(outlier_threshold),
+                                             C.c_float(threshold_factor), _p(q), _p(scratch))
+    return q, np.float32(s)
+
+
+def pack_2bit(q):
+    q = np.ascontiguousarray(q, dtype=np.int8).reshape(-1)
+    out = np.empty(((q.size + 3) // 4,), dtype=np.uint8)
+    lib().orc_pack_2bit(_p(q), _sz(q.size), _p(out))
+    return out
+
+
+def unpack_2bit(packed, n):
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    assert packed.size >= (n + 3) // 4
+    q = np.empty((n,), dtype=np.int8)
+    lib().orc_unpack_2bit(_p(packed), _sz(n), _p(q))
+    return q
+
+
+def gemm_w2a8(packed, a, n_out):
+    """acc int32 [m, n_out] from flat-packed [n_out, k] weights and int8 activations [m, k]."""
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    a = np.ascontiguousarray(a, dtype=np.int8)
+    if a.ndim == 1:
+        a = a.reshape(1, -1)
+    m, k = a.shape
+    assert packed.size >= (n_out * k + 3) // 4
+    acc = np.empty((m, n_out), dtype=np.int32)
+    lib().orc_gemm_w2a8(_p(packed), _p(a), _p(acc), _sz(m), _sz(n_out), _sz(k))
+    return acc
+
+
+def gemv_w2a8(packed, a, n_out):
+    return gemm_w2a8(packed, np.asarray(a).reshape(1, -1), n_out)[0]
+
+
+def gemm_ternary_i8(w, a):
+    w = np.ascontiguousarray(w, dtype=np.int8)
+    a = np.ascontiguousarray(a, dtype=np.int8)
+    if a.ndim == 1:
+        a = a.reshape(1, -1)
+    n_out, k = w.shape
+    m = a.shape[0]
+    acc = np.empty((m, n_out), dtype=np.int32)
+    lib().orc_gemm_ternary_i8(_p(w), _p(a), _p(acc), _sz(m), _sz(n_out), _sz(k))
+    return acc
+
+
+def epilogue(acc, w_scale, a_scale, bias=None, residual=None):
+    acc = np.ascontiguousarray(acc, dtype=np.int32)
+    m, n = acc.shape
+    a_scale = _f32(a_scale)
+    bias = None if bias is None else _f32(bias)
+    residual = None if residual is None else _f32(residual)
+    out = np.empty((m, n), dtype=np.float32)
+    lib().orc_epilogue(_p(acc), C.c_float(w_scale), _p(a_scale), _p(bias), _p(residual), _sz(m), _sz(n), _p(out))
+    return out
+
+
+def bitlinear_forward(x, packed, n_out, w_scale, g=None, eps=1e-5, order=SUM_WAVE64, bias=None, residual=None):
+    """Returns (out f32 [m,n], q int8 [m,k], a_scale f32 [m], acc int32 [m,n])."""
+    x = _f32(x)
+    m, k = x.shape
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    g = None if g is None else _f32(g)
+    bias = None if bias is None else _f32(bias)
+    residual = None if residual is None else _f32(residual)
+    out = np.empty((m, n_out), dtype=np.float32)
+    q = np.empty((m, k), dtype=np.int8)
+    a_scale = np.empty((m,), dtype=np.float32)
+    acc = np.empty((m, n_out), dtype=np.int32)
+    lib().orc_bitlinear_forward(_p(x), _sz(m), _sz(k), _p(g), C.c_float(eps), C.c_int(order), _p(packed), _sz(n_out),
+                                C.c_float(w_scale), _p(bias), _p(residual), _p(out), _p(q), _p(a_scale), _p(acc))
+    return out, q, a_scale, acc
+
+
+def relu2_mul(gate, up):
+    gate, up = _f32(gate), _f32(up)
+    h = np.empty_like(gate)
+    lib().orc_relu2_mul(_p(gate), _p(up), _sz(gate.size), _p(h))
+    return h
+
+
+def gqa_broadcast_v(v, q_heads, kv_heads, head_dim):
+    v = _f32(v)
+    m = v.shape[0]
+    out = np.empty((m, q_heads * head_dim), dtype=np.float32)
+    lib().orc_gqa_broadcast_v(_p(v), _sz(m), _sz(q_heads), _sz(kv_heads), _sz(head_dim), _p(out))
+    return out
+
+
+def decoder_layer(x, weights, w_scales, hidden, ffn, q_heads, kv_heads, head_dim, g_attn, g_ffn, eps=1e-5,
+                  order=SUM_WAVE64):
+    """weights: 7 flat-packed u8 arrays (q,k,v,o,gate,up,down); returns (x_out, q, k)."""
+    x = _f32(x)
+    m = x.shape[0]
+    ws = [np.ascontiguousarray(w, dtype=np.uint8) for w in weights]
+    arr = (C.c_void_p * 7)(*[w.ctypes.data for w in ws])
+    scales = (C.c_float * 7)(*[float(s) for s in w_scales])
+    g_attn, g_ffn = _f32(g_attn), _f32(g_ffn)
+    x_out = np.empty((m, hidden), dtype=np.float32)
+    q = np.empty((m, hidden), dtype=np.float32)
+    k = np.empty((m, kv_heads * head_dim), dtype=np.float32)
+    lib().orc_decoder_layer(_p(x), _sz(m), _sz(hidden), _sz(ffn), _sz(q_heads), _sz(kv_heads), _sz(head_dim), _p(g_attn),
+                            _p(g_ffn), C.c_float(eps), C.c_int(order), arr, scales, _p(x_out), _p(q), _p(k))
+    return x_out, q, k
+
+
+# ---- CPU baselines (timed by the benchmark, never used for results) ----------------------------------
+
+def cpu_threads() -> int:
+    return int(lib().cpu_baseline_max_threads())
+
+
+def cpu_set_threads(n: int):
+    lib().cpu_baseline_set_threads(C.c_int(n))
+
+
+def cpu_isa() -> str:
+    return {0: "scalar", 1: "avx2+fma", 2: "avx512f"}[int(lib().cpu_baseline_isa())]
+
+
+def cpu_ref_f32_forward(x, q, scale, wf_scratch, out):
+    m, k = x.shape
+    n = q.shape[0]
+    lib().cpu_ref_f32_forward(_p(x), _p(q), C.c_float(scale), None, _p(wf_scratch), _p(out), _sz(m), _sz(n), _sz(k))
+
+
+def cpu_ref_simd_gemv(q, x, y, scale):
+    m, k = x.shape
+    n = q.shape[0]
+    lib().cpu_ref_simd_gemv(_p(q), _p(x), _p(y), C.c_float(scale), _sz(m), _sz(n), _sz(k))

@@ -1,0 +1,118 @@
+"""The C-ABI library: it loads, exports exactly what include/bitnet_hip.h declares, the Python binding
+declares the same set, and argument validation that needs no device behaves like the reference's
+validation code.  No GPU needed (no kernel is launched)."""
+import ctypes as C
+import re
+import subprocess
+
+import pytest
+
+import bitnet_hip as bh
+
+
+def header_functions():
+    text = bh.HEADER_PATH.read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bitnet_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_is_built_and_loads():
+    assert bh.LIB_PATH.exists(), "build the library first: make -C bitnet-mlx.rs_amd"
+    assert bh.load_library() is not None
+
+
+def test_exports_match_header_and_binding():
+    declared = header_functions()
+    assert len(declared) >= 25
+    out = subprocess.run(["nm", "-D", "--defined-only", str(bh.LIB_PATH)], capture_output=True, text=True, check=True).stdout
+    exported = sorted(set(re.findall(r" T (bitnet_hip_[a-z0-9_]+)", out)))
+    assert exported == declared
+    assert bh.declared_symbols() == declared
+    lib = bh.load_library()
+    for name in declared:
+        assert getattr(lib, name) is not None
+
+
+def test_library_carries_gfx950_code_only():
+    blob = bh.LIB_PATH.read_bytes()
+    targets = set(re.findall(rb"amdgcn-amd-amdhsa--(gfx[0-9a-z]+)", blob))
+    assert targets == {b"gfx950"}
+
+
+def test_sizes_match_reference_formulas():
+    # (count + 3) / 4: bitnet-cuda/src/backend.rs:226, bitnet-inference/src/engine/weight_conversion.rs:151
+    for count in (0, 1, 3, 4, 5, 2560 * 2560, 6912 * 2560):
+        assert bh.packed_size(count) == (count + 3) // 4
+    assert bh.packed_size(2560 * 2560) == 1_638_400
+    assert bh.packed_size(640 * 2560) == 409_600
+    assert bh.packed_size(6912 * 2560) == 4_423_680
+    # tiles of 16 rows x 256 columns, 1 KiB each: no padding at the BitNet-2B shapes
+    assert bh.tiled_size(2560, 2560) == 1_638_400
+    assert bh.tiled_size(6912, 2560) == 4_423_680
+    assert bh.tiled_size(2560, 6912) == 4_423_680
+    assert bh.tiled_size(17, 257) == 2 * 2 * 1024
+    assert bh.tiled_size(0, 10) == 0
+
+
+def _last_error():
+    return bh.load_library().bitnet_hip_last_error().decode()
+
+
+def test_w2a8_dimension_validation_matches_reference_order():
+    """validate_w2a8_dimensions (bitnet-cuda/src/backend.rs:217-257): weights, then activations, then output."""
+    lib = bh.load_library()
+    m, k = 8, 16
+    dummy = C.c_void_p(0x1000)  # never dereferenced: validation fails first
+    rc = lib.bitnet_hip_gemv_w2a8_checked(dummy, 31, dummy, k, dummy, m, m, k, None)
+    assert rc == bh.SHAPE_MISMATCH and "weight bytes" in _last_error()
+    e, a, ar = (C.c_size_t * 4)(), (C.c_size_t * 4)(), C.c_int()
+    assert lib.bitnet_hip_last_shape_mismatch(e, a, C.byref(ar)) == 1
+    assert (e[0], a[0], ar.value) == ((m * k + 3) // 4, 31, 1)
+    rc = lib.bitnet_hip_gemv_w2a8_checked(dummy, 32, dummy, k + 1, dummy, m, m, k, None)
+    assert rc == bh.SHAPE_MISMATCH and "activation" in _last_error()
+    rc = lib.bitnet_hip_gemv_w2a8_checked(dummy, 32, dummy, k, dummy, m - 1, m, k, None)
+    assert rc == bh.SHAPE_MISMATCH and "output" in _last_error()
+
+
+def test_null_and_config_validation_without_device():
+    lib = bh.load_library()
+    dummy = C.c_void_p(0x1000)
+    assert lib.bitnet_hip_gemv_w2a8(None, None, None, 4, 4, None) == bh.NULL_POINTER
+    assert lib.bitnet_hip_gemv_w2a8(dummy, dummy, dummy, 0, 4, None) == bh.OK  # nothing to do
+    assert lib.bitnet_hip_matmul_w2a8(None, dummy, 1, 1, 16, dummy, None, None, None, None, None, None) == bh.NULL_POINTER
+    assert lib.bitnet_hip_matmul_w2a8(dummy, dummy, 1, 1, 16, None, None, None, None, None, None, None) == bh.NULL_POINTER
+    # out without scales
+    assert lib.bitnet_hip_matmul_w2a8(dummy, dummy, 1, 1, 16, None, None, None, None, None, dummy, None) == bh.NULL_POINTER
+    # misaligned tiled buffer
+    assert lib.bitnet_hip_matmul_w2a8(C.c_void_p(0x1004), dummy, 1, 1, 16, dummy, None, None, None, None, None, None) == bh.INVALID_CONFIG
+    rc = lib.bitnet_hip_quantize_activations_i8(dummy, None, 16, 1, 16, 7, 1, 1, None, 1e-5, 1, dummy, dummy, None, None, None)
+    assert rc == bh.INVALID_CONFIG and "input_mode" in _last_error()
+    rc = lib.bitnet_hip_quantize_activations_i8(dummy, None, 16, 1, 16, 0, 1, 1, None, 1e-5, 5, dummy, dummy, None, None, None)
+    assert rc == bh.INVALID_CONFIG and "sum_order" in _last_error()
+    rc = lib.bitnet_hip_quantize_activations_i8(dummy, None, 16, 1, 16, bh.INPUT_RELU2_MUL, 1, 1, None, 1e-5, 1, dummy, dummy, None, None, None)
+    assert rc == bh.NULL_POINTER
+    rc = lib.bitnet_hip_quantize_activations_i8(dummy, None, 8, 1, 16, 0, 1, 1, None, 1e-5, 1, dummy, dummy, None, None, None)
+    assert rc == bh.SHAPE_MISMATCH
+    rc = lib.bitnet_hip_quantize_weights(dummy, 4, 4, 9, 0.5, dummy, dummy, None, None)
+    assert rc == bh.INVALID_CONFIG
+    h = C.c_void_p()
+    assert lib.bitnet_hip_bitlinear_create(0, 4, 0, C.byref(h)) == bh.INVALID_CONFIG and not h.value
+    assert lib.bitnet_hip_bitlinear_create(4, 4, 0, None) == bh.NULL_POINTER
+    d = C.c_void_p()
+    # q_heads * head_dim must equal hidden
+    assert lib.bitnet_hip_decoder_create(1, 64, 96, 4, 2, 8, 1e-5, 1, 1, C.byref(d)) == bh.INVALID_CONFIG
+
+
+def test_binding_rejects_host_tensors_loudly():
+    import torch
+
+    with pytest.raises(bh.BitLinearError) as ei:
+        bh.quantize_activations_i8(torch.zeros(2, 16))
+    assert ei.value.kind == "DeviceError"
+
+
+def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
+    monkeypatch.setattr(bh, "_lib", None)
+    monkeypatch.setattr(bh, "LIB_PATH", tmp_path / "libbitnet_hip.so")
+    with pytest.raises(ImportError):
+        bh.load_library()

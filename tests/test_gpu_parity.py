@@ -1,0 +1,467 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle on the same seeded inputs.
+
+Bar: int8 activations, packed bytes and int32 accumulators bit-exact; f32 scales and outputs compared
+bit-exact where the oracle and the kernel perform the same IEEE operations, and in any case within
+1e-5 relative error (the tolerance the path's specification states)."""
+import numpy as np
+import pytest
+import torch
+
+import bitnet_hip as bh
+from helpers import golden_vectors, rel_err, synth_activations, synth_weights
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+G = golden_vectors()
+f32 = np.float32
+REL_TOL = 1e-5
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    bh.init(0)
+    info = bh.device_info()
+    assert info["arch"].startswith("gfx950")
+    yield
+    torch.cuda.synchronize()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+# ---- P1 ------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("case", G["unpack_2bit"], ids=lambda c: c["source"].split(":")[0].split("/")[-1])
+def test_unpack_reference_bytes(case):
+    got = host(bh.unpack_ternary_2bit(dev(np.array(case["bytes"], dtype=np.uint8)), case["count"]))
+    assert got.tolist() == case["expected"]
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 63, 64, 65, 1000, 10000, 2560 * 640])
+def test_pack_unpack_match_oracle(n):
+    rng = np.random.default_rng(n)
+    w = rng.integers(-1, 2, size=n).astype(np.int8) if n not in (1000, 10000) else (np.arange(n) % 3 - 1).astype(np.int8)
+    packed = bh.BitPacked2BitPacker().pack(dev(w))
+    assert np.array_equal(host(packed), orc.pack_2bit(w))
+    assert np.array_equal(host(bh.BitPacked2BitPacker().unpack(packed, n)), w)
+
+
+def test_unpack_every_byte_value():
+    allb = np.arange(256, dtype=np.uint8)
+    assert np.array_equal(host(bh.unpack_ternary_2bit(dev(allb), 1024)), orc.unpack_2bit(allb, 1024))
+
+
+@pytest.mark.parametrize("n,k", [(16, 256), (17, 257), (5, 7), (33, 100), (640, 2560), (2560, 6912)])
+@pytest.mark.parametrize("layout", [bh.LAYOUT_OUT_IN, bh.LAYOUT_IN_OUT])
+def test_retile_is_a_bijection(n, k, layout):
+    rng = np.random.default_rng(n * 7 + k)
+    w = rng.integers(-1, 2, size=(n, k)).astype(np.int8)
+    src = w if layout == bh.LAYOUT_OUT_IN else np.ascontiguousarray(w.T)
+    tiled = bh.retile_weights(dev(orc.pack_2bit(src)), n, k, layout)
+    assert tiled.numel() == bh.tiled_size(n, k)
+    back = host(bh.untile_weights(tiled, n, k))
+    assert np.array_equal(back, orc.pack_2bit(w))
+
+
+def test_retile_canonicalises_code_three():
+    # code 3 decodes to weight 0 in every reference decoder; the tiled layout stores it as code 1
+    n, k = 16, 256
+    packed = np.full((n * k // 4,), 0xFF, dtype=np.uint8)
+    tiled = bh.retile_weights(dev(packed), n, k)
+    assert np.all(host(tiled) == 0x55)
+    a = dev(np.full((1, k), 77, dtype=np.int8))
+    acc, _ = bh.matmul_w2a8(tiled, a, n, want_out=False)
+    assert not host(acc).any()
+
+
+# ---- W1 ------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("n,k", [(4, 4), (3, 5), (64, 128), (640, 2560), (2560, 2560)])
+def test_quantize_weights_absmean_bit_exact(n, k):
+    rng = np.random.default_rng(n + k)
+    w = synth_weights(rng, n, k)
+    packed, w_scale, q = bh.quantize_weights(dev(w), want_i8=True)
+    q_ref, s_ref = orc.quantize_weights_absmean(w)
+    assert host(w_scale)[0] == s_ref
+    assert np.array_equal(host(q), q_ref)
+    assert np.array_equal(host(packed), orc.pack_2bit(q_ref))
+
+
+def test_quantize_weights_reference_vectors():
+    c = G["quantize_batch"]
+    w = np.array([c["input"]], dtype=f32)
+    # threshold form with the reference's factor 0.5 on its own vector (mean|w| of this vector is 1.2167)
+    _, s, q = bh.quantize_weights(dev(w), method=bh.TERNARY_MEAN_THRESHOLD, threshold_factor=0.5, want_i8=True)
+    assert host(s)[0] == orc.absmean(w)
+    assert host(q)[0].tolist() == orc.ternarize_threshold(w, f32(0.5) * orc.absmean(w))[0].tolist()
+    for case in G["absmean"]:
+        _, s, _ = bh.quantize_weights(dev(np.array([case["input"]], dtype=f32)))
+        assert abs(float(host(s)[0]) - case["expected"]) < 1e-6
+    # ties and a zero matrix
+    w = np.array([[0.5, -0.5, 0.25, 1.5, -7.0, 0.0, 1.0, -1.0]], dtype=f32)
+    _, s, q = bh.quantize_weights(dev(w), want_i8=True)
+    assert np.array_equal(host(q), orc.ternarize_roundclip(w, host(s)[0]))
+    _, s, q = bh.quantize_weights(dev(np.zeros((4, 8), dtype=f32)), want_i8=True)
+    assert host(s)[0] == 0.0 and not host(q).any()
+
+
+# ---- R1 + A1 -------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("m,k", [(1, 2560), (4, 2560), (3, 6912), (2, 1024), (5, 4096), (2, 8192), (2, 12000),
+                                 (3, 7), (2, 257), (1, 4), (9, 64)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_activation_quant_bit_exact(m, k, norm):
+    rng = np.random.default_rng(m * 100003 + k)
+    x = synth_activations(rng, m, k, outliers=True)
+    g = rng.standard_normal(k, dtype=f32) if norm else None
+    q, s, asum, y = bh.quantize_activations_i8(dev(x), dev(g) if norm else None, eps=1e-5, want_sum=True, want_y=norm)
+    q_ref, s_ref, rs_ref = orc.rmsnorm_quantize_i8(x, g, 1e-5, orc.SUM_WAVE64)
+    assert np.array_equal(host(s), s_ref)
+    assert np.array_equal(host(q), q_ref)
+    assert np.array_equal(host(asum), rs_ref)
+    if norm:
+        assert np.array_equal(host(y), orc.rmsnorm(x, g, 1e-5, orc.SUM_WAVE64))
+
+
+@pytest.mark.parametrize("k", [2560, 300])
+def test_activation_quant_sequential_order_bit_exact(k):
+    """The reference's literal summation order (one running f32 sum) is available and also bit-exact."""
+    rng = np.random.default_rng(k)
+    x = synth_activations(rng, 3, k)
+    g = rng.standard_normal(k, dtype=f32)
+    q, s, _, y = bh.quantize_activations_i8(dev(x), dev(g), eps=1e-6, sum_order=bh.SUM_SEQUENTIAL, want_y=True)
+    q_ref, s_ref, _ = orc.rmsnorm_quantize_i8(x, g, 1e-6, orc.SUM_SEQUENTIAL)
+    assert np.array_equal(host(y), orc.rmsnorm(x, g, 1e-6, orc.SUM_SEQUENTIAL))
+    assert np.array_equal(host(s), s_ref) and np.array_equal(host(q), q_ref)
+
+
+def test_activation_quant_edge_rows():
+    x = np.zeros((4, 256), dtype=f32)
+    x[1, :9] = [127.0, 0.5, -0.5, 1.5, 2.5, -2.5, 0.49999997, -126.5, 126.4999]
+    x[2, 3] = np.nan
+    x[2, 4] = 2.0
+    x[3, :] = 1e-30
+    q, s, asum, _ = bh.quantize_activations_i8(dev(x), want_sum=True)
+    q_ref, s_ref, rs_ref = orc.quantize_activations_i8(x)
+    assert np.array_equal(host(q), q_ref) and np.array_equal(host(s), s_ref) and np.array_equal(host(asum), rs_ref)
+    assert host(s)[0] == 1.0 and not host(q)[0].any()
+    assert host(q)[1, :9].tolist() == [127, 1, -1, 2, 3, -3, 0, -127, 126]
+    # the reference's own property test (ternary_operations.rs:445-461)
+    xin = np.array([G["activation_quant_properties"]["input"]], dtype=f32)
+    q, s, _, _ = bh.quantize_activations_i8(dev(xin))
+    fq = host(q)[0].astype(f32) / host(s)[0]
+    assert fq[1] > fq[0] and fq[2] < 0 and fq[3] < fq[2]
+    c = G["absmax_8bit_scale"]
+    _, s, _, _ = bh.quantize_activations_i8(dev(np.array([c["input"]], dtype=f32)))
+    assert host(s)[0] == f32(127.0) / f32(c["absmax"])
+
+
+def test_activation_quant_fused_inputs():
+    rng = np.random.default_rng(21)
+    m, ffn = 3, 6912
+    gate, up = synth_activations(rng, m, ffn), synth_activations(rng, m, ffn)
+    q, s, _, _ = bh.quantize_activations_i8(dev(gate), x2=dev(up), input_mode=bh.INPUT_RELU2_MUL)
+    q_ref, s_ref, _ = orc.quantize_activations_i8(orc.relu2_mul(gate, up))
+    assert np.array_equal(host(q), q_ref) and np.array_equal(host(s), s_ref)
+    v = synth_activations(rng, m, 640)
+    q, s, _, _ = bh.quantize_activations_i8(dev(v), input_mode=bh.INPUT_GQA_BROADCAST, gqa_group=4, head_dim=128)
+    q_ref, s_ref, _ = orc.quantize_activations_i8(orc.gqa_broadcast_v(v, 20, 5, 128))
+    assert np.array_equal(host(q), q_ref) and np.array_equal(host(s), s_ref)
+
+
+def test_activation_quant_prefill_size_properties():
+    """Full prefill size (2048 x 2560): size-independent properties plus a sampled comparison."""
+    rng = np.random.default_rng(22)
+    x = synth_activations(rng, 2048, 2560, outliers=True)
+    g = np.ones(2560, dtype=f32)
+    xd = dev(x)
+    q, s, asum, _ = bh.quantize_activations_i8(xd, dev(g), want_sum=True)
+    qh = host(q)
+    assert np.all(np.abs(qh.astype(np.int32)).max(axis=1) == 127)
+    assert np.array_equal(host(asum), qh.astype(np.int64).sum(axis=1))
+    qn, sn, _, _ = bh.quantize_activations_i8(-xd, dev(g))
+    assert np.array_equal(host(qn), -qh) and np.array_equal(host(sn), host(s))
+    rows = rng.choice(2048, size=64, replace=False)
+    q_ref, s_ref, _ = orc.rmsnorm_quantize_i8(x[rows], g, 1e-5)
+    assert np.array_equal(qh[rows], q_ref) and np.array_equal(host(s)[rows], s_ref)
+
+
+# ---- G1: reference contract on the reference's byte layout ---------------------------------------------------
+
+@pytest.mark.parametrize("case", G["gemv"], ids=lambda c: f'{c["m"]}x{c["k"]}')
+def test_w2a8_gemv_reference_vectors(case):
+    w = np.array(case["a"], dtype=np.int8).reshape(case["m"], case["k"])
+    out = torch.zeros(case["m"], dtype=torch.int32, device="cuda")
+    bh.W2A8Backend().w2a8_gemv(dev(orc.pack_2bit(w)), dev(np.array(case["x"], dtype=np.int8)), out, case["m"], case["k"])
+    assert (host(out) * case["scale"]).tolist() == case["expected"]
+
+
+@pytest.mark.parametrize("n,k", [(1, 1), (3, 5), (7, 33), (64, 256), (100, 1000), (640, 2560), (2560, 6912)])
+def test_w2a8_gemv_rowmajor_bit_exact(n, k):
+    rng = np.random.default_rng(n * 31 + k)
+    w = rng.integers(-1, 2, size=(n, k)).astype(np.int8)
+    a = rng.integers(-128, 128, size=k).astype(np.int8)
+    packed = orc.pack_2bit(w)
+    out = torch.zeros(n, dtype=torch.int32, device="cuda")
+    bh.W2A8Backend().w2a8_gemv(dev(packed), dev(a), out, n, k)
+    assert np.array_equal(host(out), orc.gemv_w2a8(packed, a, n))
+
+
+def test_w2a8_gemv_shape_errors():
+    b = bh.W2A8Backend()
+    w, a, o = dev(np.zeros(32, np.uint8)), dev(np.zeros(16, np.int8)), torch.zeros(8, dtype=torch.int32, device="cuda")
+    with pytest.raises(bh.BitLinearError) as ei:
+        b.w2a8_gemv(w[:31].contiguous(), a, o, 8, 16)
+    assert ei.value.kind == "ShapeMismatch" and ei.value.expected == [32] and ei.value.actual == [31]
+    with pytest.raises(bh.BitLinearError):
+        b.w2a8_gemv(w, a[:15].contiguous(), o, 8, 16)
+    with pytest.raises(bh.BitLinearError):
+        b.w2a8_gemv(w, a, o[:7].contiguous(), 8, 16)
+
+
+# ---- G1 / G2 / E1 on the tiled layout ---------------------------------------------------------------------
+
+SHAPES = [(2560, 2560), (640, 2560), (6912, 2560), (2560, 6912)]
+
+
+def make_problem(rng, m, n, k, outliers=False, full_range=False):
+    w = synth_weights(rng, n, k)
+    qw, ws = orc.quantize_weights_absmean(w)
+    packed = orc.pack_2bit(qw)
+    if full_range:
+        a = rng.integers(-128, 128, size=(m, k)).astype(np.int8)
+        a_scale = (rng.random(m, dtype=f32) * 50 + 1).astype(f32)
+    else:
+        a, a_scale, _ = orc.quantize_activations_i8(synth_activations(rng, m, k, outliers))
+    return packed, ws, a, a_scale
+
+
+@pytest.mark.parametrize("n,k", SHAPES)
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8])
+def test_decode_gemv_bit_exact(m, n, k):
+    rng = np.random.default_rng(m * 1000 + n + k)
+    packed, ws, a, a_scale = make_problem(rng, m, n, k, outliers=True)
+    tiled = bh.retile_weights(dev(packed), n, k)
+    acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale))
+    acc_ref = orc.gemm_w2a8(packed, a, n)
+    assert np.array_equal(host(acc), acc_ref)
+    out_ref = orc.epilogue(acc_ref, ws, a_scale)
+    assert np.array_equal(host(out), out_ref)
+    assert rel_err(host(out), out_ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (1, 5, 7), (2, 17, 257), (3, 33, 100), (1, 16, 255), (4, 15, 512),
+                                   (1, 48, 16384), (8, 31, 3000)])
+def test_decode_gemv_ragged_shapes(m, n, k):
+    rng = np.random.default_rng(m + 10 * n + 100 * k)
+    packed, ws, a, a_scale = make_problem(rng, m, n, k, full_range=True)
+    tiled = bh.retile_weights(dev(packed), n, k)
+    bias = rng.standard_normal(n, dtype=f32)
+    res = rng.standard_normal((m, n), dtype=f32)
+    acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale), dev(bias), dev(res))
+    acc_ref = orc.gemm_w2a8(packed, a, n)
+    assert np.array_equal(host(acc), acc_ref)
+    assert np.array_equal(host(out), orc.epilogue(acc_ref, ws, a_scale, bias, res))
+
+
+def test_decode_gemv_extremes_and_identities():
+    k, n = 6912, 32
+    tiled_neg = bh.retile_weights(dev(orc.pack_2bit(-np.ones((n, k), np.int8))), n, k)
+    acc, _ = bh.matmul_w2a8(tiled_neg, dev(np.full((1, k), -128, np.int8)), n, want_out=False)
+    assert np.all(host(acc) == 128 * k)
+    tiled_pos = bh.retile_weights(dev(orc.pack_2bit(np.ones((n, k), np.int8))), n, k)
+    rng = np.random.default_rng(5)
+    a = rng.integers(-128, 128, size=(2, k)).astype(np.int8)
+    acc, _ = bh.matmul_w2a8(tiled_pos, dev(a), n, want_out=False)
+    assert np.array_equal(host(acc), np.repeat(a.astype(np.int64).sum(1)[:, None], n, axis=1))
+    # linearity in the activations: acc(a1 + a2) = acc(a1) + acc(a2) while a1 + a2 stays in int8
+    w = rng.integers(-1, 2, size=(n, k)).astype(np.int8)
+    tiled = bh.retile_weights(dev(orc.pack_2bit(w)), n, k)
+    a1 = rng.integers(-60, 60, size=(1, k)).astype(np.int8)
+    a2 = rng.integers(-60, 60, size=(1, k)).astype(np.int8)
+    r1, _ = bh.matmul_w2a8(tiled, dev(a1), n, want_out=False)
+    r2, _ = bh.matmul_w2a8(tiled, dev(a2), n, want_out=False)
+    r12, _ = bh.matmul_w2a8(tiled, dev((a1 + a2).astype(np.int8)), n, want_out=False)
+    assert np.array_equal(host(r12), host(r1) + host(r2))
+
+
+@pytest.mark.parametrize("m", [16, 64])
+@pytest.mark.parametrize("n,k", [(6912, 2560), (2560, 6912)])
+def test_batched_decode_sweep_bit_exact(m, n, k):
+    rng = np.random.default_rng(m + n)
+    packed, ws, a, a_scale = make_problem(rng, m, n, k, outliers=True)
+    tiled = bh.retile_weights(dev(packed), n, k)
+    acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale))
+    acc_ref = orc.gemm_w2a8(packed, a, n)
+    assert np.array_equal(host(acc), acc_ref)
+    assert np.array_equal(host(out), orc.epilogue(acc_ref, ws, a_scale))
+
+
+@pytest.mark.parametrize("n,k", [(6912, 2560), (2560, 6912)])
+def test_prefill_gemm_full_size(n, k):
+    """M = 2048 at the two prefill shapes: sampled rows bit-exact against the oracle, whole result through
+    order-free identities (column sums of acc against a one-row contraction of the summed activations)."""
+    m = 2048
+    rng = np.random.default_rng(n)
+    packed, ws, a, a_scale = make_problem(rng, m, n, k, outliers=False)
+    tiled = bh.retile_weights(dev(packed), n, k)
+    acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale))
+    acc_h, out_h = host(acc), host(out)
+    rows = np.sort(rng.choice(m, size=48, replace=False))
+    acc_ref = orc.gemm_w2a8(packed, a[rows], n)
+    assert np.array_equal(acc_h[rows], acc_ref)
+    assert np.array_equal(out_h[rows], orc.epilogue(acc_ref, ws, a_scale[rows]))
+    # sum over tokens of acc[t, n] == sum_k (sum_t a[t, k]) * w[n, k]
+    w = orc.unpack_2bit(packed, n * k).reshape(n, k).astype(np.int64)
+    assert np.array_equal(acc_h.astype(np.int64).sum(axis=0), w @ a.astype(np.int64).sum(axis=0))
+    assert np.array_equal(out_h, orc.epilogue(acc_h, ws, a_scale))
+
+
+# ---- L1: BitLinear object ----------------------------------------------------------------------------------
+
+def test_bitlinear_forward_config1_bit_exact():
+    """BASELINE config 1: M=1, K=2560, N=2560, seed 0, W ~ N(0, 0.02), X ~ N(0, 1)."""
+    rng = np.random.default_rng(0)
+    w = synth_weights(rng, 2560, 2560)
+    x = synth_activations(rng, 1, 2560)
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=2560, out_features=2560), "config1")
+    layer.update_weights(torch.from_numpy(w))  # host weights, quantised on the GPU
+    out, q, a_scale, acc = layer.forward(dev(x), debug=True)
+    qw, ws = orc.quantize_weights_absmean(w)
+    packed_h, ws_h = layer.get_quantized_weights()
+    assert ws_h == ws and np.array_equal(packed_h.numpy(), orc.pack_2bit(qw))
+    out_ref, q_ref, s_ref, acc_ref = orc.bitlinear_forward(x, orc.pack_2bit(qw), 2560, ws)
+    assert np.array_equal(host(q), q_ref)
+    assert np.array_equal(host(a_scale), s_ref)
+    assert np.array_equal(host(acc), acc_ref)
+    assert np.array_equal(host(out), out_ref)
+    assert rel_err(host(out), out_ref) <= REL_TOL
+    # the non-debug call gives the same bits
+    assert np.array_equal(host(layer.forward(dev(x))), out_ref)
+
+
+def test_bitlinear_forward_shapes_bias_norm_and_layouts():
+    rng = np.random.default_rng(31)
+    k, n = 256, 80
+    w = synth_weights(rng, n, k)
+    qw, ws = orc.quantize_weights_absmean(w)
+    packed = orc.pack_2bit(qw)
+    bias = rng.standard_normal(n, dtype=f32)
+    g = rng.standard_normal(k, dtype=f32)
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n, use_bias=True), "t")
+    with pytest.raises(bh.BitLinearError) as ei:
+        layer.forward(dev(np.zeros((2, k), f32)))
+    assert ei.value.kind == "NotInitialized"
+    layer.update_weights(dev(w))
+    # bias starts at zero, like the reference's Tensor::zeros bias (layer.rs:127-133)
+    x = synth_activations(rng, 6, k)
+    ref0 = orc.bitlinear_forward(x, packed, n, ws)[0]
+    assert np.array_equal(host(layer.forward(dev(x))), ref0)
+    layer.update_bias(dev(bias))
+    ref = orc.bitlinear_forward(x, packed, n, ws, bias=bias)[0]
+    assert np.array_equal(host(layer.forward(dev(x))), ref)
+    # rank 3 input is flattened to [b*s, in] and reshaped back (forward.rs:182-207)
+    out3 = layer.forward(dev(x.reshape(2, 3, k)))
+    assert tuple(out3.shape) == (2, 3, n) and np.array_equal(host(out3).reshape(6, n), ref)
+    # fused RMSNorm + residual
+    res = rng.standard_normal((6, n), dtype=f32)
+    refn = orc.bitlinear_forward(x, packed, n, ws, g=g, eps=1e-5, bias=bias, residual=res)[0]
+    assert np.array_equal(host(layer.forward(dev(x), gamma=dev(g), residual=dev(res))), refn)
+    # [in, out] orientation (the GGUF-side convention) gives the same layer
+    layer_t = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "t_in_out")
+    layer_t.update_weights(dev(np.ascontiguousarray(w.T)), layout=bh.LAYOUT_IN_OUT)
+    p2, s2 = layer_t.get_quantized_weights()
+    assert np.array_equal(p2.numpy(), packed)
+    assert abs(s2 - float(ws)) <= 1e-7 * float(ws)  # the declared f64 summation order follows the given orientation
+    # pre-quantised weights (forward_with_quantized_weights)
+    layer_p = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "t_packed")
+    layer_p.set_quantized_weights(torch.from_numpy(packed), float(ws))
+    assert np.array_equal(host(layer_p.forward(dev(x))), ref0)
+
+
+def test_bitlinear_error_behaviour_matches_reference():
+    """forward.rs:304-371: wrong last dimension -> ShapeMismatch; rank other than 2/3 -> ShapeMismatch."""
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=4, out_features=3), "test_layer_shape")
+    layer.update_weights(torch.ones(3, 4))
+    out = layer.forward(torch.ones(2, 4, device="cuda"))
+    assert tuple(out.shape) == (2, 3)
+    with pytest.raises(bh.BitLinearError) as ei:
+        layer.forward(torch.ones(2, 5, device="cuda"))
+    assert ei.value.kind == "ShapeMismatch" and ei.value.expected == [2, 4] and ei.value.actual == [2, 5]
+    with pytest.raises(bh.BitLinearError) as ei:
+        layer.forward(torch.ones(4, device="cuda"))
+    assert ei.value.kind == "ShapeMismatch"
+    with pytest.raises(bh.BitLinearError) as ei:
+        layer.forward(torch.ones(2, 2, 2, 4, device="cuda"))
+    assert ei.value.kind == "ShapeMismatch"
+    with pytest.raises(bh.BitLinearError) as ei:
+        layer.update_weights(torch.ones(4, 3))
+    assert ei.value.kind == "ShapeMismatch" and ei.value.expected == [3, 4]
+    with pytest.raises(bh.BitLinearError) as ei:
+        layer.update_bias(torch.ones(3))
+    assert ei.value.kind == "InvalidConfig" and "Bias is not enabled" in str(ei.value)
+    with pytest.raises(bh.BitLinearError):
+        layer.forward_batch(torch.ones(4, device="cuda"))
+    # empty batch: nothing to do
+    assert tuple(layer.forward(torch.ones(0, 4, device="cuda")).shape) == (0, 3)
+
+
+# ---- L1: decoder layer and stack ----------------------------------------------------------------------------
+
+def build_decoder(rng, layers, hidden, ffn, qh, kvh, hd, max_tokens, eps=1e-5):
+    dec = bh.DecoderProjections(layers, hidden, ffn, qh, kvh, hd, eps=eps, max_tokens=max_tokens)
+    ref = []
+    for l in range(layers):
+        packed, scales = [], []
+        for p in range(7):
+            n, k = dec.proj_shape(p)
+            w = synth_weights(rng, n, k)
+            dec.projection(l, p).update_weights(dev(w))
+            qw, s = orc.quantize_weights_absmean(w)
+            packed.append(orc.pack_2bit(qw))
+            scales.append(s)
+        ga = (1 + 0.1 * rng.standard_normal(hidden, dtype=f32)).astype(f32)
+        gf = (1 + 0.1 * rng.standard_normal(hidden, dtype=f32)).astype(f32)
+        dec.set_norm(l, 0, torch.from_numpy(ga))
+        dec.set_norm(l, 1, torch.from_numpy(gf))
+        ref.append((packed, scales, ga, gf))
+    return dec, ref
+
+
+def oracle_stack(ref, x, hidden, ffn, qh, kvh, hd, eps=1e-5):
+    q = k = None
+    for packed, scales, ga, gf in ref:
+        x, q, k = orc.decoder_layer(x, packed, scales, hidden, ffn, qh, kvh, hd, ga, gf, eps)
+    return x, q, k
+
+
+@pytest.mark.parametrize("m", [1, 8])
+def test_decoder_layer_config2_bit_exact(m):
+    """BASELINE config 2: one decoder layer's seven projections at BitNet-2B shapes."""
+    rng = np.random.default_rng(0)
+    dec, ref = build_decoder(rng, 1, 2560, 6912, 20, 5, 128, max_tokens=8)
+    assert dec.weight_bytes() == 17_367_040
+    x = synth_activations(rng, m, 2560)
+    out, q, k = dec.decode(dev(x), want_qk=True)
+    x_ref, q_ref, k_ref = oracle_stack(ref, x, 2560, 6912, 20, 5, 128)
+    assert np.array_equal(host(q), q_ref) and np.array_equal(host(k), k_ref)
+    assert np.array_equal(host(out), x_ref)
+    assert rel_err(host(out), x_ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("layers", [2, 3])
+def test_decoder_stack_small_bit_exact(layers):
+    rng = np.random.default_rng(layers)
+    dims = (256, 512, 4, 2, 64)
+    dec, ref = build_decoder(rng, layers, *dims, max_tokens=4)
+    x = synth_activations(rng, 3, 256)
+    out = dec.decode(dev(x))
+    assert np.array_equal(host(out), oracle_stack(ref, x, *dims)[0])
+    with pytest.raises(bh.BitLinearError) as ei:
+        dec.decode(dev(synth_activations(rng, 5, 256)))
+    assert ei.value.kind == "ShapeMismatch"
