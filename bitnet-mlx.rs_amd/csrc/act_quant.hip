@@ -44,7 +44,7 @@ struct ActQuantParams {
 __device__ __forceinline__ float wave_sum_f32(float p)
 {
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) p = __fadd_rn(p, __shfl_xor(p, off, 64));
+    for (int off = 32; off >= 1; off >>= 1) p = f32_add(p, __shfl_xor(p, off, 64));
     return p;
 }
 
@@ -65,7 +65,7 @@ __device__ __forceinline__ int wave_sum_i32(int p)
 __device__ __forceinline__ float relu2_mul(float gate, float up)
 {
     float r = gate > 0.0f ? gate : 0.0f;
-    return __fmul_rn(up, __fmul_rn(r, r));
+    return f32_mul(up, f32_mul(r, r));
 }
 
 // Element i of the (virtual) input row `row` after the fused input transform.
@@ -113,7 +113,7 @@ __device__ __forceinline__ float4 load_chunk(const ActQuantParams &p, size_t row
 
 __device__ __forceinline__ int quant1(float y, float scale)
 {
-    float t = roundf(__fmul_rn(y, scale));
+    float t = roundf(f32_mul(y, scale));
     if (t != t) return 0;
     t = fminf(fmaxf(t, -128.0f), 127.0f);
     return (int)t;
@@ -152,28 +152,28 @@ __global__ __launch_bounds__(256) void act_quant_kernel(ActQuantParams p)
             ss = 0.0f;
             for (int i = 0; i < p.k; ++i) {
                 float e = load_elem<MODE>(p, row, i);
-                ss = __fadd_rn(ss, __fmul_rn(e, e));
+                ss = f32_add(ss, f32_mul(e, e));
             }
         } else {
             float part = 0.0f;
 #pragma unroll
             for (int i = 0; i < nloop; ++i) {
                 float4 e = chunk_at(i, lane + 64 * i);
-                part = __fadd_rn(part, __fmul_rn(e.x, e.x));
-                part = __fadd_rn(part, __fmul_rn(e.y, e.y));
-                part = __fadd_rn(part, __fmul_rn(e.z, e.z));
-                part = __fadd_rn(part, __fmul_rn(e.w, e.w));
+                part = f32_add(part, f32_mul(e.x, e.x));
+                part = f32_add(part, f32_mul(e.y, e.y));
+                part = f32_add(part, f32_mul(e.z, e.z));
+                part = f32_add(part, f32_mul(e.w, e.w));
             }
             ss = wave_sum_f32(part);
         }
-        rms = __fsqrt_rn(__fadd_rn(__fdiv_rn(ss, (float)p.k), p.eps));
+        rms = f32_sqrt(f32_add(f32_div(ss, (float)p.k), p.eps));
     }
 
     // normalised value of element `idx` whose raw value is e
     auto normed = [&](float e, int idx) -> float {
         if (!norm) return e;
         float g = idx < p.k ? p.gamma[idx] : 0.0f;
-        return __fmul_rn(__fdiv_rn(e, rms), g);
+        return f32_mul(f32_div(e, rms), g);
     };
 
     float amax = 0.0f;
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(ActQuantParams p)
         amax = fmaxf(amax, fmaxf(fmaxf(fabsf(e.x), fabsf(e.y)), fmaxf(fabsf(e.z), fabsf(e.w))));
     }
     amax = wave_max_f32(amax);
-    const float scale = amax > 0.0f ? __fdiv_rn(127.0f, amax) : 1.0f;
+    const float scale = amax > 0.0f ? f32_div(127.0f, amax) : 1.0f;
 
     int isum = 0;
 #pragma unroll

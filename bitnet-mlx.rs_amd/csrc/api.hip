@@ -457,6 +457,16 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
     return rc;
 }
 
+int bitnet_hip_bitlinear_matmul(bitnet_hip_bitlinear *layer, const int8_t *a, size_t m, const float *a_scale,
+                                const float *residual, int32_t *acc, float *out, void *stream)
+{
+    if (!layer) return fail(BITNET_HIP_NULL_POINTER, "bitlinear_matmul: layer is NULL");
+    std::shared_lock<std::shared_mutex> guard(layer->lock);
+    if (!layer->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "bitlinear_matmul: the layer has no weights yet");
+    return bitnet_hip_matmul_w2a8(layer->tiled, a, m, layer->out_features, layer->in_features, acc, layer->w_scale,
+                                  a_scale, layer->use_bias ? layer->bias : nullptr, residual, out, stream);
+}
+
 }  // extern "C"
 
 // ---------------------------------------------------------------------------------------------------
@@ -572,17 +582,22 @@ size_t bitnet_hip_decoder_weight_bytes(const bitnet_hip_decoder *dec)
     return total;
 }
 
-int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t m, float *x_out, float *q_last,
-                              float *k_last, void *stream)
+int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin, size_t layer_end,
+                                     const float *x_in, size_t m, float *x_out, float *q_last, float *k_last,
+                                     void *stream)
 {
     if (!dec || !x_in || !x_out) return fail(BITNET_HIP_NULL_POINTER, "decoder_decode: null argument");
-    if (m == 0) return BITNET_HIP_OK;
+    if (layer_begin > layer_end || layer_end > dec->layers)
+        return fail(BITNET_HIP_INVALID_CONFIG, "decoder_decode: layer range [%zu, %zu) outside [0, %zu)", layer_begin,
+                    layer_end, dec->layers);
+    if (m == 0 || layer_begin == layer_end) return BITNET_HIP_OK;
     if (m > dec->max_tokens) {
         size_t e[2] = {dec->max_tokens, dec->hidden}, a[2] = {m, dec->hidden};
         return fail_shape(e, 2, a, 2, "tokens per decode step exceed max_tokens");
     }
-    for (auto *p : dec->proj)
-        if (!p->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "decoder_decode: a projection has no weights yet");
+    for (size_t i = layer_begin * 7; i < layer_end * 7; ++i)
+        if (!dec->proj[i]->has_weights)
+            return fail(BITNET_HIP_NOT_INITIALIZED, "decoder_decode: a projection has no weights yet");
     hipStream_t s = as_stream(stream);
     const size_t H = dec->hidden, F = dec->ffn, KV = dec->kv_heads * dec->head_dim;
     const size_t group = dec->q_heads / dec->kv_heads;
@@ -598,12 +613,12 @@ int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t
                               dec->a_scale, nullptr, nullptr, s);
     };
     const float *x = x_in;
-    for (size_t l = 0; l < dec->layers; ++l) {
+    for (size_t l = layer_begin; l < layer_end; ++l) {
         bitnet_hip_bitlinear **P = &dec->proj[l * 7];
         const float *g_attn = dec->gamma + (l * 2) * H, *g_ffn = g_attn + H;
-        const bool last = l + 1 == dec->layers;
+        const bool last = l + 1 == layer_end;
         // hidden states alternate between x_out and the internal buffer so that the last block writes x_out
-        float *x2 = ((dec->layers - 1 - l) % 2 == 0) ? x_out : dec->ping;
+        float *x2 = ((layer_end - 1 - l) % 2 == 0) ? x_out : dec->ping;
         quant(x, nullptr, H, H, BITNET_HIP_INPUT_PLAIN, g_attn);
         mm(P[BITNET_HIP_PROJ_Q], nullptr, (last && q_last) ? q_last : dec->qb);
         mm(P[BITNET_HIP_PROJ_K], nullptr, (last && k_last) ? k_last : dec->kb);
@@ -618,6 +633,13 @@ int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t
         x = x2;
     }
     return rc;
+}
+
+int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t m, float *x_out, float *q_last,
+                              float *k_last, void *stream)
+{
+    if (!dec) return fail(BITNET_HIP_NULL_POINTER, "decoder_decode: null argument");
+    return bitnet_hip_decoder_decode_layers(dec, 0, dec->layers, x_in, m, x_out, q_last, k_last, stream);
 }
 
 }  // extern "C"

@@ -157,10 +157,10 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
             size_t o = (size_t)t * p.n + n;
             if (p.acc) p.acc[o] = total;
             if (p.out) {
-                float v = __fmul_rn((float)total, *p.w_scale);
-                v = __fdiv_rn(v, p.a_scale[t]);
-                if (p.bias) v = __fadd_rn(v, p.bias[n]);
-                if (p.residual) v = __fadd_rn(v, p.residual[o]);
+                float v = f32_mul((float)total, *p.w_scale);
+                v = f32_div(v, p.a_scale[t]);
+                if (p.bias) v = f32_add(v, p.bias[n]);
+                if (p.residual) v = f32_add(v, p.residual[o]);
                 p.out[o] = v;
             }
         }

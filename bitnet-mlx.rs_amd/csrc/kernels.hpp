@@ -2,6 +2,7 @@
 // these only pick a kernel variant and launch it.  All return a bitnet_hip_status.
 #pragma once
 #include "common.hpp"
+#include "ieee.hpp"
 
 namespace bitnet {
 

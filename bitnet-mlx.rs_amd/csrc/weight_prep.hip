@@ -79,7 +79,7 @@ __device__ __forceinline__ int ternarize_one(float w, int method, float s, float
     if (method == BITNET_HIP_TERNARY_ABSMEAN_ROUNDCLIP) {
         // RoundClip(w / s, -1, 1); s == 0 gives 0
         if (s == 0.0f) return 0;
-        float r = roundf(__fdiv_rn(w, s));
+        float r = roundf(f32_div(w, s));
         if (r != r) return 0;
         r = fminf(fmaxf(r, -1.0f), 1.0f);
         return (int)r;
@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256) void ternarize_pack_kernel(const float *w, siz
     size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= nbytes) return;
     const float s = *w_scale;
-    const float thr = __fmul_rn(factor, s);
+    const float thr = f32_mul(factor, s);
     unsigned byte = 0;
     for (int j = 0; j < 4; ++j) {
         size_t i = 4 * b + j;

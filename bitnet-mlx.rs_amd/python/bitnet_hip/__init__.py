@@ -102,6 +102,8 @@ def load_library() -> C.CDLL:
         "bitnet_hip_bitlinear_get_quantized": (i32, [vp, C.POINTER(f32), vp, sz]),
         "bitnet_hip_bitlinear_workspace_size": (sz, [vp, sz]),
         "bitnet_hip_bitlinear_forward": (i32, [vp, vp, C.POINTER(sz), i32, vp, f32, i32, vp, vp, vp, sz, vp, vp, vp, vp]),
+        "bitnet_hip_bitlinear_matmul": (i32, [vp, vp, sz, vp, vp, vp, vp, vp]),
+        "bitnet_hip_decoder_decode_layers": (i32, [vp, sz, sz, vp, sz, vp, vp, vp, vp]),
         "bitnet_hip_decoder_create": (i32, [sz, sz, sz, sz, sz, sz, f32, i32, sz, C.POINTER(vp)]),
         "bitnet_hip_decoder_destroy": (None, [vp]),
         "bitnet_hip_decoder_projection": (i32, [vp, sz, i32, C.POINTER(vp)]),
@@ -378,6 +380,21 @@ class BitLinear:
             return out, q, a_scale, acc
         return out
 
+    def matmul_quantized(self, a: torch.Tensor, a_scale: torch.Tensor, residual: Optional[torch.Tensor] = None,
+                         want_acc: bool = False, out: Optional[torch.Tensor] = None, stream=None):
+        """Contraction + epilogue on already-quantised activations (TernaryProcessor::ternary_matmul,
+        ternary_operations.rs:87-113, minus its quantiser).  a: [m, in] int8, a_scale: [m] f32."""
+        _dev(a, torch.int8, "a")
+        m = a.shape[0]
+        if a.shape[1] != self.config.in_features:
+            raise BitLinearError(SHAPE_MISMATCH, "activation width", [m, self.config.in_features], list(a.shape))
+        if out is None:
+            out = torch.empty((m, self.config.out_features), dtype=torch.float32, device=a.device)
+        acc = torch.empty((m, self.config.out_features), dtype=torch.int32, device=a.device) if want_acc else None
+        _check(load_library().bitnet_hip_bitlinear_matmul(self._h, _ptr(a), m, _ptr(a_scale), _ptr(residual), _ptr(acc),
+                                                          _ptr(out), _stream(stream)))
+        return (out, acc) if want_acc else out
+
     def forward_batch(self, x: torch.Tensor):
         """BitLinear::forward_batch (forward.rs:270-297): rank >= 2 required."""
         if x.dim() < 2:
@@ -428,13 +445,16 @@ class DecoderProjections:
     def weight_bytes(self) -> int:
         return load_library().bitnet_hip_decoder_weight_bytes(self._h)
 
-    def decode(self, x: torch.Tensor, out: Optional[torch.Tensor] = None, want_qk: bool = False, stream=None):
+    def decode(self, x: torch.Tensor, out: Optional[torch.Tensor] = None, want_qk: bool = False, stream=None,
+               layers: Optional[Sequence[int]] = None):
+        """One decode step through all blocks, or through blocks layers[0] .. layers[1]-1 only."""
         _dev(x, torch.float32, "x")
         m = x.shape[0]
         if out is None:
             out = torch.empty_like(x)
         q = torch.empty((m, self.hidden), dtype=torch.float32, device=x.device) if want_qk else None
         k = torch.empty((m, self.kv_dim), dtype=torch.float32, device=x.device) if want_qk else None
-        _check(load_library().bitnet_hip_decoder_decode(self._h, _ptr(x), m, _ptr(out), _ptr(q), _ptr(k),
-                                                        _stream(stream)))
+        lo, hi = (0, self.layers) if layers is None else layers
+        _check(load_library().bitnet_hip_decoder_decode_layers(self._h, lo, hi, _ptr(x), m, _ptr(out), _ptr(q), _ptr(k),
+                                                               _stream(stream)))
         return (out, q, k) if want_qk else out

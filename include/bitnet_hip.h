@@ -198,6 +198,13 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
                                  float *out, void *workspace, size_t workspace_bytes, int8_t *dbg_q,
                                  float *dbg_a_scale, int32_t *dbg_acc, void *stream);
 
+/* The contraction + epilogue of a layer on activations that are already quantised:
+ * TernaryProcessor::ternary_matmul (bitnet-inference/src/engine/ternary_operations.rs:87-113) /
+ * BitLinearForward::forward_with_quantized_weights (forward.rs:95-136) without the activation quantiser.
+ *   a [m, in] int8, a_scale [m] f32; acc [m, out] int32 and out [m, out] f32 may each be NULL (not both). */
+int bitnet_hip_bitlinear_matmul(bitnet_hip_bitlinear *layer, const int8_t *a, size_t m, const float *a_scale,
+                                const float *residual, int32_t *acc, float *out, void *stream);
+
 /* ---- decoder projections (seven BitLinear layers per block) ------------------------------------ */
 
 typedef struct bitnet_hip_decoder bitnet_hip_decoder; /* opaque */
@@ -231,6 +238,10 @@ size_t bitnet_hip_decoder_weight_bytes(const bitnet_hip_decoder *dec);
  * NULL) receive the last block's q [m, hidden] and k [m, kv_heads*head_dim] projections. */
 int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t m, float *x_out,
                               float *q_last, float *k_last, void *stream);
+/* The same for blocks layer_begin .. layer_end-1 only (x_in may equal x_out). */
+int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin, size_t layer_end,
+                                     const float *x_in, size_t m, float *x_out, float *q_last, float *k_last,
+                                     void *stream);
 
 #ifdef __cplusplus
 }
