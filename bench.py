@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the BitLinear W1.58A8 forward path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode pass (batch 1) through the seven BitLinear projections of one BitNet-b1.58-2B
+decoder layer (hidden 2560, FFN 6912, 20 query / 5 KV heads): fused RMSNorm + int8 quantisation before
+q/k/v and before gate/up, int8 quantisation before o and down, seven packed-ternary GEMVs with the scale
+epilogue.  Consecutive steps use the weights of consecutive layers of a 30-layer stack (521 MB of packed
+weights in total), so no step finds its weights in cache.  Inputs and weights are resident in HBM before
+the timed region.  value = packed-weight bytes streamed per second over the whole timed region.
+
+The line also carries: the roofline of the dominant kernel (the decode GEMV) from HIP-event timing of
+GEMV-only launches over the same 210 weight matrices; the prefill GEMM rate (M = 2048) at the two FFN
+shapes; and a CPU baseline (a C restatement of the reference's dequantise-to-f32 BitLinear forward)
+timed on this host's cores for a bounded sample.
+"""
+import argparse
+import json
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT / "bitnet-mlx.rs_amd" / "python"))
+sys.path.insert(0, str(ROOT))
+
+HIDDEN, FFN, Q_HEADS, KV_HEADS, HEAD_DIM, LAYERS = 2560, 6912, 20, 5, 128, 30
+LAYER_BYTES = 17_367_040  # sum of n*k/4 over q,k,v,o,gate,up,down
+HBM_PEAK_GBS = 8000.0
+INT8_PEAK_TOPS = 5000.0
+
+
+def build_stack(bh, torch, layers, max_tokens=1):
+    dec = bh.DecoderProjections(layers, HIDDEN, FFN, Q_HEADS, KV_HEADS, HEAD_DIM, eps=1e-5, max_tokens=max_tokens)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    for l in range(layers):
+        for p in range(7):
+            n, k = dec.proj_shape(p)
+            w = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+            dec.projection(l, p).update_weights(w)  # ternarised, packed and re-tiled on the GPU
+            del w
+    return dec, gen
+
+
+def time_events(torch, fn):
+    """Elapsed milliseconds of fn() measured with events on the stream the kernels are launched on."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop)
+
+
+def gemv_roofline(bh, torch, dec, gen, reps):
+    """GEMV-only launches over all 210 matrices, captured in a HIP graph so that host launch cost does not
+    starve the GPU; HIP events around the replays."""
+    a = {k: torch.randint(-127, 128, (1, k), generator=gen, device="cuda", dtype=torch.int8) for k in (HIDDEN, FFN)}
+    a_scale = torch.ones((1,), device="cuda", dtype=torch.float32)
+    outs = {n: torch.empty((1, n), device="cuda", dtype=torch.float32) for n in (HIDDEN, KV_HEADS * HEAD_DIM, FFN)}
+    projs = [(dec.projection(l, p), dec.proj_shape(p)) for l in range(dec.layers) for p in range(7)]
+
+    def launch_all():
+        for bl, (n, k) in projs:
+            bl.matmul_quantized(a[k], a_scale, out=outs[n])
+
+    launch_all()
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            launch_all()
+        graph.replay()
+        torch.cuda.synchronize()
+        ms = time_events(torch, lambda: [graph.replay() for _ in range(reps)])
+    launches = reps * len(projs)
+    total_bytes = reps * dec.weight_bytes()
+    avg_us = ms * 1e3 / launches
+    achieved = total_bytes / (ms * 1e-3) / 1e9
+    return {
+        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+        "kernel": "gemv_tiled_kernel<1>", "launches": launches, "avg_launch_us": round(avg_us, 3),
+        "bytes_per_launch": round(total_bytes / launches),
+        "how": "HIP events around graph replays of GEMV-only launches over 210 distinct weight matrices (521 MB)",
+    }
+
+
+def prefill_rates(bh, torch, dec, gen, reps):
+    m = 2048
+    res = {}
+    for name, p in (("2048x2560x6912", 4), ("2048x6912x2560", 6)):
+        n, k = dec.proj_shape(p)
+        bl = dec.projection(0, p)
+        a = torch.randint(-127, 128, (m, k), generator=gen, device="cuda", dtype=torch.int8)
+        a_scale = torch.ones((m,), device="cuda", dtype=torch.float32)
+        out = torch.empty((m, n), device="cuda", dtype=torch.float32)
+        bl.matmul_quantized(a, a_scale, out=out)
+        ms = time_events(torch, lambda: [bl.matmul_quantized(a, a_scale, out=out) for _ in range(reps)]) / reps
+        tops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+        res[name] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+        del a, out
+    return res
+
+
+def cpu_baseline(torch, dec, budget_s=15.0):
+    """The reference's BitLinear::forward on the host cores: per call, materialise q*scale as f32 [N,K], then an
+    f32 GEMV (bitnet-quant/src/bitlinear/forward.rs:153-258), for the seven projections of one layer."""
+    import numpy as np
+
+    from oracle import oracle as orc
+
+    cores = orc.cpu_threads()
+    orc.cpu_set_threads(cores)
+    mats = []
+    for p in range(7):
+        n, k = dec.proj_shape(p)
+        packed, scale = dec.projection(0, p).get_quantized_weights()
+        q = orc.unpack_2bit(packed.numpy(), n * k).reshape(n, k)
+        mats.append((q, np.float32(scale), np.empty(n * k, dtype=np.float32), np.empty((1, n), dtype=np.float32)))
+    rng = np.random.default_rng(0)
+    x = {k: rng.standard_normal((1, k), dtype=np.float32) for k in (HIDDEN, FFN)}
+
+    def one_layer():
+        for q, s, wf, out in mats:
+            orc.cpu_ref_f32_forward(x[q.shape[1]], q, s, wf, out)
+
+    one_layer()
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        one_layer()
+        reps += 1
+        if time.perf_counter() - t0 > budget_s or reps >= 200:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    return {
+        "value": round(LAYER_BYTES / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": f"{reps} passes over one layer's 7 projections at batch 1 (dequantise to f32 + f32 GEMV per call, "
+                  f"{orc.cpu_isa()}), {dt * 1e3:.2f} ms per layer",
+        "ms_per_step": round(dt * 1e3, 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=600)
+    ap.add_argument("--warmup", type=int, default=60)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip roofline / prefill / CPU legs (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the one-GPU BitLinear path; --gpus must be 1 (nothing here uses a second GPU)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import bitnet_hip as bh
+
+    bh.init(0)
+    dec, gen = build_stack(bh, torch, LAYERS)
+    x = torch.randn((1, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
+
+    def step(i):
+        l = i % LAYERS
+        dec.decode(x, out=x, layers=(l, l + 1))
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(args.steps):
+        step(args.warmup + i)
+    stop.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    event_ms = start.elapsed_time(stop)
+
+    value = args.steps * LAYER_BYTES / elapsed / 1e9
+    line = {
+        "metric": "BitLinear decode GB/s (% HBM peak) + prefill int8 TOPS (% MFMA peak)",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed * 1e3 / args.steps, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "i8", "data": "synthetic",
+        "config": {"workload": "configs[1]: one decoder layer's 7 decode projections at batch 1 "
+                               "(hidden 2560, ffn 6912, 20q/5kv heads), weights rotating over a 30-layer stack",
+                   "bytes_per_step": LAYER_BYTES, "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+                   "event_ms_per_step": round(event_ms / args.steps, 5), "device": bh.device_info()},
+    }
+    if not args.no_extras:
+        line["roofline"] = gemv_roofline(bh, torch, dec, gen, reps=5)
+        line["prefill"] = prefill_rates(bh, torch, dec, gen, reps=5)
+        if not args.no_cpu_baseline:
+            line["cpu_baseline"] = cpu_baseline(torch, dec)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
