@@ -13,7 +13,7 @@
 // gemv_tiled_kernel streams the re-tiled layout (weight_prep.hip).  A workgroup of four wavefronts owns
 // one block of 16 output rows; its wavefronts take the k-tiles round-robin, so all of a workgroup's
 // weight bytes are requested in the first few instructions.  Lane l of a wavefront loads the 16 bytes at
-// offset 16*l of a 1 KiB tile: row r = l mod 16, the 64 columns 64*(l/16) .. +63.  Activations sit in LDS
+// offset 16*l of a 1 KiB tile: row r = l mod 16, four groups of 16 columns.  Activations sit in LDS
 // (staged once per workgroup); the 16 lanes of a group read the same LDS address (a broadcast).
 // Partial sums are combined with two wavefront shuffles (the four lanes of a row), then across the four
 // wavefronts through LDS.  HBM traffic per call: n*k/4 weight bytes + k activation bytes per row block.
@@ -43,14 +43,15 @@ __device__ __forceinline__ int dot4(uint32_t a, uint32_t c, int acc)
     return __builtin_amdgcn_sdot4((int)a, (int)c, acc, false);
 }
 
-// 64 weights (one uint4 of a tile) against 64 activations (four uint4 from LDS).
+// 64 weights (one slot of a tile: dword t = 16 columns at 64t + 16kq) against their activations; ag
+// points at activation group kq of the tile, the groups of consecutive dwords are 4 apart.
 __device__ __forceinline__ int dot64(const uint4 &w4, const uint4 *ag, int acc)
 {
     const uint32_t ws[4] = {w4.x, w4.y, w4.z, w4.w};
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const uint32_t w = ws[t];
-        const uint4 a4 = ag[t];
+        const uint4 a4 = ag[4 * t];
         acc = dot4(a4.x, w & 0x03030303u, acc);
         acc = dot4(a4.y, (w >> 2) & 0x03030303u, acc);
         acc = dot4(a4.z, (w >> 4) & 0x03030303u, acc);
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
 #pragma unroll
     for (int t = 0; t < MB; ++t) acc[t] = 0;
 
-    const int kq = lane >> 4;  // which 64-column quarter of a tile this lane holds
+    const int kq = lane >> 4;  // lane group: columns 64t + 16kq .. +15 of each tile, t = 0..3
     for (int kt0 = wave; kt0 < p.kt_count; kt0 += 4 * GEMV_PREFETCH) {
         uint4 wnext[GEMV_PREFETCH];
 #pragma unroll
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
         for (int u = 0; u < GEMV_PREFETCH; ++u) {
             int kt = kt0 + 4 * u;
             if (kt < p.kt_count) {
-                const uint4 *ag = lds_a + kt * 16 + kq * 4;
+                const uint4 *ag = lds_a + kt * 16 + kq;
 #pragma unroll
                 for (int t = 0; t < MB; ++t) acc[t] = dot64(wbuf[u], ag + t * groups, acc[t]);
             }

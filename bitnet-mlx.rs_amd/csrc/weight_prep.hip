@@ -7,13 +7,15 @@
 // -1,0,+1,0 (bitnet-inference/src/engine/weight_conversion.rs:169-184).
 //
 // Re-tiled layout: the [n, k] matrix is cut into tiles of TILE_ROWS(16) rows x TILE_K(256) columns.  A
-// tile is 1 KiB = 64 slots of 16 bytes.  Slot s = kq*16 + r (kq = 0..3, r = 0..15) holds, for row r of the
-// tile, the 64 columns 64*kq .. 64*kq+63 as four dwords (dword t = columns 64*kq + 16t .. +15).  Inside a
-// dword the weight with column offset 4j + b sits at bits 2j + 8b, so that (dword >> 2j) & 0x03030303
-// yields the four code bytes of columns 4j..4j+3 in activation byte order.  Tiles are stored row-block
-// major: tile (rb, kt) starts at byte ((rb * k_tiles) + kt) * 1024.  A wavefront whose lane l loads slot
-// l reads one tile as a single contiguous 1 KiB burst; lanes l, l+16, l+32, l+48 share a row, which is
-// also the operand order of the 16x16x64 int8 MFMA (row/column = lane mod 16, k block = lane / 16).
+// tile is 1 KiB = 64 slots of 16 bytes.  Slot s = kq*16 + r (kq = 0..3, r = 0..15) belongs to row r of the
+// tile; its dword t (t = 0..3) holds the 16 columns 64*t + 16*kq .. +15.  Inside a dword the weight with
+// column offset 4j + b sits at bits 2j + 8b, so that (dword >> 2j) & 0x03030303 yields the four code
+// bytes of columns 4j..4j+3 in activation byte order.  Tiles are stored row-block major: tile (rb, kt)
+// starts at byte ((rb * k_tiles) + kt) * 1024.
+// Why this order: a wavefront whose lane l loads slot l reads one tile as a single contiguous 1 KiB
+// burst, and dword t of every lane is then exactly the B operand of the t-th 16x16x64 int8 MFMA over
+// the tile's columns 64t..64t+63 (operand row/column = lane mod 16, 16-column k block = lane / 16).
+// Lanes l, l+16, l+32, l+48 share a row, so the decode GEMV combines them with two shuffles.
 // Positions outside the matrix hold code 1 (weight 0) and code 3 is rewritten to code 1, so the
 // contraction kernels never see code 3.
 #include "kernels.hpp"
@@ -121,7 +123,7 @@ __global__ __launch_bounds__(256) void retile_kernel(const uint8_t *packed, size
     size_t tile = d >> 8;
     unsigned wd = (unsigned)(d & 255);
     unsigned slot = wd >> 2, t = wd & 3;
-    unsigned r = slot & 15, g = 4 * (slot >> 4) + t;
+    unsigned r = slot & 15, g = 4 * t + (slot >> 4);
     size_t rb = tile / kt_count, kt = tile % kt_count;
     size_t row = rb * TILE_ROWS + r;
     size_t kbase = kt * TILE_K + (size_t)g * 16;
@@ -153,7 +155,7 @@ __global__ __launch_bounds__(256) void untile_kernel(const uint32_t *tiled, size
         size_t row = e / k, kk = e % k;
         size_t tile = (row / TILE_ROWS) * kt_count + kk / TILE_K;
         unsigned g = (unsigned)((kk % TILE_K) / 16), c = (unsigned)(kk % 16);
-        unsigned wd = (((g >> 2) * 16 + (unsigned)(row % TILE_ROWS)) << 2) + (g & 3);
+        unsigned wd = (((g & 3) * 16 + (unsigned)(row % TILE_ROWS)) << 2) + (g >> 2);
         uint32_t word = tiled[tile * 256 + wd];
         byte |= ((word >> (2 * (c >> 2) + 8 * (c & 3))) & 3u) << (2 * j);
     }
