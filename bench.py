@@ -98,9 +98,10 @@ def prefill_rates(bh, torch, dec, gen, reps):
         bl = dec.projection(0, p)
         a = torch.randint(-127, 128, (m, k), generator=gen, device="cuda", dtype=torch.int8)
         a_scale = torch.ones((m,), device="cuda", dtype=torch.float32)
+        a_sum = a.to(torch.int32).sum(dim=1).to(torch.int32).contiguous()  # what the activation quantiser emits
         out = torch.empty((m, n), device="cuda", dtype=torch.float32)
-        bl.matmul_quantized(a, a_scale, out=out)
-        ms = time_events(torch, lambda: [bl.matmul_quantized(a, a_scale, out=out) for _ in range(reps)]) / reps
+        bl.matmul_quantized(a, a_scale, out=out, a_sum=a_sum)
+        ms = time_events(torch, lambda: [bl.matmul_quantized(a, a_scale, out=out, a_sum=a_sum) for _ in range(reps)]) / reps
         tops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
         res[name] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
         del a, out

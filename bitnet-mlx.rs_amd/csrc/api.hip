@@ -259,9 +259,9 @@ int bitnet_hip_gemv_w2a8_checked(const uint8_t *weights, size_t weights_len, con
     return bitnet_hip_gemv_w2a8(weights, activations, output, m, k, stream);
 }
 
-int bitnet_hip_matmul_w2a8(const uint8_t *tiled, const int8_t *a, size_t m, size_t n, size_t k, int32_t *acc,
-                           const float *w_scale, const float *a_scale, const float *bias, const float *residual,
-                           float *out, void *stream)
+int bitnet_hip_matmul_w2a8(const uint8_t *tiled, const int8_t *a, const int32_t *a_sum, size_t m, size_t n, size_t k,
+                           int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,
+                           const float *residual, float *out, void *stream)
 {
     if (m == 0 || n == 0) return BITNET_HIP_OK;
     if (!tiled || !a) return fail(BITNET_HIP_NULL_POINTER, "matmul_w2a8: null input buffer");
@@ -272,7 +272,7 @@ int bitnet_hip_matmul_w2a8(const uint8_t *tiled, const int8_t *a, size_t m, size
     if (n > 0x7fffffffu || k > 0x7fffffffu) return fail(BITNET_HIP_UNSUPPORTED, "matmul_w2a8: dimension too large");
     if (m <= (size_t)GEMV_MAX_M)
         return launch_gemv_tiled(tiled, a, m, n, k, acc, w_scale, a_scale, bias, residual, out, as_stream(stream));
-    return launch_gemm_tiled(tiled, a, m, n, k, acc, w_scale, a_scale, bias, residual, out, as_stream(stream));
+    return launch_gemm_tiled(tiled, a, a_sum, m, n, k, acc, w_scale, a_scale, bias, residual, out, as_stream(stream));
 }
 
 // ---- BitLinear layer object -------------------------------------------------------------------------
@@ -399,7 +399,7 @@ int bitnet_hip_bitlinear_get_quantized(bitnet_hip_bitlinear *layer, float *w_sca
 size_t bitnet_hip_bitlinear_workspace_size(const bitnet_hip_bitlinear *layer, size_t m)
 {
     if (!layer) return 0;
-    return align_up(m * layer->in_features, 256) + align_up(m * sizeof(float), 256) + 256;
+    return align_up(m * layer->in_features, 256) + 2 * align_up(m * sizeof(float), 256) + 256;
 }
 
 int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, const size_t *dims, int rank,
@@ -443,11 +443,12 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
     uintptr_t base = align_up(reinterpret_cast<uintptr_t>(ws), 256);
     int8_t *q = dbg_q ? dbg_q : reinterpret_cast<int8_t *>(base);
     float *a_scale = dbg_a_scale ? dbg_a_scale : reinterpret_cast<float *>(base + align_up(m * in, 256));
+    int32_t *a_sum = reinterpret_cast<int32_t *>(base + align_up(m * in, 256) + align_up(m * sizeof(float), 256));
 
     int rc = launch_act_quant(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, 1, gamma, eps, sum_order, q, a_scale,
-                              nullptr, nullptr, s);
+                              a_sum, nullptr, s);
     if (rc == BITNET_HIP_OK)
-        rc = bitnet_hip_matmul_w2a8(layer->tiled, q, m, nout, in, dbg_acc, layer->w_scale, a_scale,
+        rc = bitnet_hip_matmul_w2a8(layer->tiled, q, a_sum, m, nout, in, dbg_acc, layer->w_scale, a_scale,
                                     layer->use_bias ? layer->bias : nullptr, residual, out, stream);
     if (own_ws) {
         hipError_t e = hipFreeAsync(ws, s);
@@ -457,13 +458,13 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
     return rc;
 }
 
-int bitnet_hip_bitlinear_matmul(bitnet_hip_bitlinear *layer, const int8_t *a, size_t m, const float *a_scale,
-                                const float *residual, int32_t *acc, float *out, void *stream)
+int bitnet_hip_bitlinear_matmul(bitnet_hip_bitlinear *layer, const int8_t *a, const int32_t *a_sum, size_t m,
+                                const float *a_scale, const float *residual, int32_t *acc, float *out, void *stream)
 {
     if (!layer) return fail(BITNET_HIP_NULL_POINTER, "bitlinear_matmul: layer is NULL");
     std::shared_lock<std::shared_mutex> guard(layer->lock);
     if (!layer->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "bitlinear_matmul: the layer has no weights yet");
-    return bitnet_hip_matmul_w2a8(layer->tiled, a, m, layer->out_features, layer->in_features, acc, layer->w_scale,
+    return bitnet_hip_matmul_w2a8(layer->tiled, a, a_sum, m, layer->out_features, layer->in_features, acc, layer->w_scale,
                                   a_scale, layer->use_bias ? layer->bias : nullptr, residual, out, stream);
 }
 
@@ -481,13 +482,14 @@ struct bitnet_hip_decoder {
     // activation buffers, sized for max_tokens
     int8_t *a8 = nullptr;
     float *a_scale = nullptr;
+    int32_t *a_sum = nullptr;
     float *qb = nullptr, *kb = nullptr, *vb = nullptr, *x1 = nullptr, *gate = nullptr, *up = nullptr;
     float *ping = nullptr;
 
     ~bitnet_hip_decoder()
     {
         for (auto *p : proj) delete p;
-        void *bufs[] = {gamma, a8, a_scale, qb, kb, vb, x1, gate, up, ping};
+        void *bufs[] = {gamma, a8, a_scale, a_sum, qb, kb, vb, x1, gate, up, ping};
         for (void *b : bufs)
             if (b) (void)hipFree(b);
     }
@@ -529,6 +531,7 @@ int bitnet_hip_decoder_create(size_t layers, size_t hidden, size_t ffn, size_t q
     dev_alloc(&d->gamma, sizeof(float) * layers * 2 * hidden);
     dev_alloc(&d->a8, max_tokens * widest);
     dev_alloc(&d->a_scale, sizeof(float) * max_tokens);
+    dev_alloc(&d->a_sum, sizeof(int32_t) * max_tokens);
     dev_alloc(&d->qb, sizeof(float) * max_tokens * hidden);
     dev_alloc(&d->kb, sizeof(float) * max_tokens * kv_dim);
     dev_alloc(&d->vb, sizeof(float) * max_tokens * kv_dim);
@@ -604,13 +607,13 @@ int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin
     int rc = BITNET_HIP_OK;
     auto mm = [&](bitnet_hip_bitlinear *bl, const float *residual, float *out) {
         if (rc != BITNET_HIP_OK) return;
-        rc = bitnet_hip_matmul_w2a8(bl->tiled, dec->a8, m, bl->out_features, bl->in_features, nullptr, bl->w_scale,
+        rc = bitnet_hip_matmul_w2a8(bl->tiled, dec->a8, dec->a_sum, m, bl->out_features, bl->in_features, nullptr, bl->w_scale,
                                     dec->a_scale, nullptr, residual, out, stream);
     };
     auto quant = [&](const float *x, const float *x2, size_t ldx, size_t k, int mode, const float *gamma) {
         if (rc != BITNET_HIP_OK) return;
         rc = launch_act_quant(x, x2, ldx, m, k, mode, group, dec->head_dim, gamma, dec->eps, dec->sum_order, dec->a8,
-                              dec->a_scale, nullptr, nullptr, s);
+                              dec->a_scale, dec->a_sum, nullptr, s);
     };
     const float *x = x_in;
     for (size_t l = layer_begin; l < layer_end; ++l) {

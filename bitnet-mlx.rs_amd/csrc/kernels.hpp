@@ -39,8 +39,9 @@ int launch_gemv_tiled(const uint8_t *tiled, const int8_t *a, size_t m, size_t n,
                       float *out, hipStream_t stream);
 
 // gemm_w2a8.hip
-int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, size_t m, size_t n, size_t k, int32_t *acc,
-                      const float *w_scale, const float *a_scale, const float *bias, const float *residual,
-                      float *out, hipStream_t stream);
+// a_sum (sum_k a[t, k] per row, from the activation quantiser) may be NULL: the slower kernel then computes it
+int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_sum, size_t m, size_t n, size_t k,
+                      int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,
+                      const float *residual, float *out, hipStream_t stream);
 
 }  // namespace bitnet

@@ -93,7 +93,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_untile_weights": (i32, [vp, sz, sz, vp, vp]),
         "bitnet_hip_gemv_w2a8": (i32, [vp, vp, vp, sz, sz, vp]),
         "bitnet_hip_gemv_w2a8_checked": (i32, [vp, sz, vp, sz, vp, sz, sz, sz, vp]),
-        "bitnet_hip_matmul_w2a8": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp, vp, vp]),
+        "bitnet_hip_matmul_w2a8": (i32, [vp, vp, vp, sz, sz, sz, vp, vp, vp, vp, vp, vp, vp]),
         "bitnet_hip_bitlinear_create": (i32, [sz, sz, i32, C.POINTER(vp)]),
         "bitnet_hip_bitlinear_destroy": (None, [vp]),
         "bitnet_hip_bitlinear_set_weights_f32": (i32, [vp, vp, sz, sz, i32, i32, i32, f32, vp]),
@@ -102,7 +102,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_bitlinear_get_quantized": (i32, [vp, C.POINTER(f32), vp, sz]),
         "bitnet_hip_bitlinear_workspace_size": (sz, [vp, sz]),
         "bitnet_hip_bitlinear_forward": (i32, [vp, vp, C.POINTER(sz), i32, vp, f32, i32, vp, vp, vp, sz, vp, vp, vp, vp]),
-        "bitnet_hip_bitlinear_matmul": (i32, [vp, vp, sz, vp, vp, vp, vp, vp]),
+        "bitnet_hip_bitlinear_matmul": (i32, [vp, vp, vp, sz, vp, vp, vp, vp, vp]),
         "bitnet_hip_decoder_decode_layers": (i32, [vp, sz, sz, vp, sz, vp, vp, vp, vp]),
         "bitnet_hip_decoder_create": (i32, [sz, sz, sz, sz, sz, sz, f32, i32, sz, C.POINTER(vp)]),
         "bitnet_hip_decoder_destroy": (None, [vp]),
@@ -248,7 +248,8 @@ def untile_weights(tiled: torch.Tensor, n: int, k: int, stream=None) -> torch.Te
 
 def matmul_w2a8(tiled: torch.Tensor, a: torch.Tensor, n: int, w_scale: Optional[torch.Tensor] = None,
                 a_scale: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
-                residual: Optional[torch.Tensor] = None, want_acc: bool = True, want_out: bool = True, stream=None):
+                residual: Optional[torch.Tensor] = None, want_acc: bool = True, want_out: bool = True, stream=None,
+                a_sum: Optional[torch.Tensor] = None):
     """acc[m,n] (int32) and/or out[m,n] (f32) from re-tiled weights and int8 activations [m, k]."""
     _dev(tiled, torch.uint8, "tiled")
     _dev(a, torch.int8, "a")
@@ -257,7 +258,7 @@ def matmul_w2a8(tiled: torch.Tensor, a: torch.Tensor, n: int, w_scale: Optional[
         raise BitLinearError(SHAPE_MISMATCH, "tiled buffer too short", [tiled_size(n, k)], [tiled.numel()])
     acc = torch.empty((m, n), dtype=torch.int32, device=a.device) if want_acc else None
     out = torch.empty((m, n), dtype=torch.float32, device=a.device) if want_out else None
-    _check(load_library().bitnet_hip_matmul_w2a8(_ptr(tiled), _ptr(a), m, n, k, _ptr(acc), _ptr(w_scale), _ptr(a_scale),
+    _check(load_library().bitnet_hip_matmul_w2a8(_ptr(tiled), _ptr(a), _ptr(a_sum), m, n, k, _ptr(acc), _ptr(w_scale), _ptr(a_scale),
                                                  _ptr(bias), _ptr(residual), _ptr(out), _stream(stream)))
     return acc, out
 
@@ -381,7 +382,8 @@ class BitLinear:
         return out
 
     def matmul_quantized(self, a: torch.Tensor, a_scale: torch.Tensor, residual: Optional[torch.Tensor] = None,
-                         want_acc: bool = False, out: Optional[torch.Tensor] = None, stream=None):
+                         want_acc: bool = False, out: Optional[torch.Tensor] = None, stream=None,
+                         a_sum: Optional[torch.Tensor] = None):
         """Contraction + epilogue on already-quantised activations (TernaryProcessor::ternary_matmul,
         ternary_operations.rs:87-113, minus its quantiser).  a: [m, in] int8, a_scale: [m] f32."""
         _dev(a, torch.int8, "a")
@@ -391,7 +393,7 @@ class BitLinear:
         if out is None:
             out = torch.empty((m, self.config.out_features), dtype=torch.float32, device=a.device)
         acc = torch.empty((m, self.config.out_features), dtype=torch.int32, device=a.device) if want_acc else None
-        _check(load_library().bitnet_hip_bitlinear_matmul(self._h, _ptr(a), m, _ptr(a_scale), _ptr(residual), _ptr(acc),
+        _check(load_library().bitnet_hip_bitlinear_matmul(self._h, _ptr(a), _ptr(a_sum), m, _ptr(a_scale), _ptr(residual), _ptr(acc),
                                                           _ptr(out), _stream(stream)))
         return (out, acc) if want_acc else out
 

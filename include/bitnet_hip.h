@@ -117,8 +117,10 @@ int bitnet_hip_unpack_ternary_2bit(const uint8_t *packed, size_t count, int8_t *
 int bitnet_hip_quantize_weights(const float *w, size_t n, size_t k, int method, float threshold_factor,
                                 uint8_t *packed, float *w_scale, int8_t *q_i8, void *stream);
 
-/* Device layout the decode GEMV streams: tiles of 16 rows x 256 columns, 1 KiB each, stored
- * [row_block][k_tile][row][64 bytes]; rows/columns past n/k are zero weights; code 3 is rewritten to
+/* Device layout both contraction kernels stream: tiles of 16 rows x 256 columns, 1 KiB each, stored
+ * [row_block][k_tile]; inside a tile the 16 bytes at offset 16*(16*kq + r) hold row r's columns
+ * 64*t + 16*kq .. +15 in dword t (t = 0..3), bit-interleaved so that (dword >> 2j) & 0x03030303 is the code
+ * bytes of columns 4j..4j+3; rows/columns past n/k are zero weights; code 3 is rewritten to
  * code 1 (both decode to 0).  bitnet_hip_tiled_size gives the byte size for an [n, k] matrix.
  * retile/untile are inverse bijections on the n*k valid positions (up to the code 3 -> 1 rewrite). */
 size_t bitnet_hip_tiled_size(size_t n, size_t k);
@@ -148,10 +150,12 @@ int bitnet_hip_gemv_w2a8_checked(const uint8_t *weights, size_t weights_len, con
  *   (bitnet-quant/src/bitlinear/forward.rs:153-223) and TernaryProcessor::ternary_matmul
  *   (bitnet-inference/src/engine/ternary_operations.rs:87-113,283-338).
  *   Small m runs the HBM-bound decode GEMV, large m the int8 MFMA GEMM.
+ *   a_sum [m] int32 = sum over k of a[t, k], as bitnet_hip_quantize_activations_i8 returns it; may be NULL
+ *   (the kernels then compute it; the fastest GEMM kernel needs it supplied).
  *   acc / out may each be NULL (at least one must be given); out needs w_scale and a_scale. */
-int bitnet_hip_matmul_w2a8(const uint8_t *tiled, const int8_t *a, size_t m, size_t n, size_t k,
-                           int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,
-                           const float *residual, float *out, void *stream);
+int bitnet_hip_matmul_w2a8(const uint8_t *tiled, const int8_t *a, const int32_t *a_sum, size_t m, size_t n,
+                           size_t k, int32_t *acc, const float *w_scale, const float *a_scale,
+                           const float *bias, const float *residual, float *out, void *stream);
 
 /* ---- BitLinear layer object ------------------------------------------------------------------- */
 
@@ -201,9 +205,11 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
 /* The contraction + epilogue of a layer on activations that are already quantised:
  * TernaryProcessor::ternary_matmul (bitnet-inference/src/engine/ternary_operations.rs:87-113) /
  * BitLinearForward::forward_with_quantized_weights (forward.rs:95-136) without the activation quantiser.
- *   a [m, in] int8, a_scale [m] f32; acc [m, out] int32 and out [m, out] f32 may each be NULL (not both). */
-int bitnet_hip_bitlinear_matmul(bitnet_hip_bitlinear *layer, const int8_t *a, size_t m, const float *a_scale,
-                                const float *residual, int32_t *acc, float *out, void *stream);
+ *   a [m, in] int8, a_scale [m] f32, a_sum [m] int32 or NULL (see bitnet_hip_matmul_w2a8);
+ *   acc [m, out] int32 and out [m, out] f32 may each be NULL (not both). */
+int bitnet_hip_bitlinear_matmul(bitnet_hip_bitlinear *layer, const int8_t *a, const int32_t *a_sum, size_t m,
+                                const float *a_scale, const float *residual, int32_t *acc, float *out,
+                                void *stream);
 
 /* ---- decoder projections (seven BitLinear layers per block) ------------------------------------ */
 

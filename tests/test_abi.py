@@ -79,12 +79,12 @@ def test_null_and_config_validation_without_device():
     dummy = C.c_void_p(0x1000)
     assert lib.bitnet_hip_gemv_w2a8(None, None, None, 4, 4, None) == bh.NULL_POINTER
     assert lib.bitnet_hip_gemv_w2a8(dummy, dummy, dummy, 0, 4, None) == bh.OK  # nothing to do
-    assert lib.bitnet_hip_matmul_w2a8(None, dummy, 1, 1, 16, dummy, None, None, None, None, None, None) == bh.NULL_POINTER
-    assert lib.bitnet_hip_matmul_w2a8(dummy, dummy, 1, 1, 16, None, None, None, None, None, None, None) == bh.NULL_POINTER
+    assert lib.bitnet_hip_matmul_w2a8(None, dummy, None, 1, 1, 16, dummy, None, None, None, None, None, None) == bh.NULL_POINTER
+    assert lib.bitnet_hip_matmul_w2a8(dummy, dummy, None, 1, 1, 16, None, None, None, None, None, None, None) == bh.NULL_POINTER
     # out without scales
-    assert lib.bitnet_hip_matmul_w2a8(dummy, dummy, 1, 1, 16, None, None, None, None, None, dummy, None) == bh.NULL_POINTER
+    assert lib.bitnet_hip_matmul_w2a8(dummy, dummy, None, 1, 1, 16, None, None, None, None, None, dummy, None) == bh.NULL_POINTER
     # misaligned tiled buffer
-    assert lib.bitnet_hip_matmul_w2a8(C.c_void_p(0x1004), dummy, 1, 1, 16, dummy, None, None, None, None, None, None) == bh.INVALID_CONFIG
+    assert lib.bitnet_hip_matmul_w2a8(C.c_void_p(0x1004), dummy, None, 1, 1, 16, dummy, None, None, None, None, None, None) == bh.INVALID_CONFIG
     rc = lib.bitnet_hip_quantize_activations_i8(dummy, None, 16, 1, 16, 7, 1, 1, None, 1e-5, 1, dummy, dummy, None, None, None)
     assert rc == bh.INVALID_CONFIG and "input_mode" in _last_error()
     rc = lib.bitnet_hip_quantize_activations_i8(dummy, None, 16, 1, 16, 0, 1, 1, None, 1e-5, 5, dummy, dummy, None, None, None)

@@ -303,14 +303,17 @@ def test_batched_decode_sweep_bit_exact(m, n, k):
 
 
 @pytest.mark.parametrize("n,k", [(6912, 2560), (2560, 6912)])
-def test_prefill_gemm_full_size(n, k):
+@pytest.mark.parametrize("with_sum", [True, False], ids=["lds_direct_kernel", "register_staged_kernel"])
+def test_prefill_gemm_full_size(n, k, with_sum):
     """M = 2048 at the two prefill shapes: sampled rows bit-exact against the oracle, whole result through
-    order-free identities (column sums of acc against a one-row contraction of the summed activations)."""
+    order-free identities (column sums of acc against a one-row contraction of the summed activations).
+    Supplying the activation row sums selects the LDS-direct kernel, omitting them the register-staged one."""
     m = 2048
     rng = np.random.default_rng(n)
     packed, ws, a, a_scale = make_problem(rng, m, n, k, outliers=False)
     tiled = bh.retile_weights(dev(packed), n, k)
-    acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale))
+    a_sum = dev(a.astype(np.int32).sum(axis=1).astype(np.int32)) if with_sum else None
+    acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale), a_sum=a_sum)
     acc_h, out_h = host(acc), host(out)
     rows = np.sort(rng.choice(m, size=48, replace=False))
     acc_ref = orc.gemm_w2a8(packed, a[rows], n)
@@ -320,6 +323,42 @@ def test_prefill_gemm_full_size(n, k):
     w = orc.unpack_2bit(packed, n * k).reshape(n, k).astype(np.int64)
     assert np.array_equal(acc_h.astype(np.int64).sum(axis=0), w @ a.astype(np.int64).sum(axis=0))
     assert np.array_equal(out_h, orc.epilogue(acc_h, ws, a_scale))
+
+
+@pytest.mark.parametrize("m,n,k", [(96, 160, 512), (100, 33, 512), (257, 170, 768), (130, 6912, 2560), (300, 16, 256),
+                                   (128, 48, 300), (200, 200, 2561)])
+def test_gemm_ragged_shapes_both_kernels(m, n, k):
+    """Token counts, widths and depths that do not fill the MFMA tiles, with bias and residual; with row sums
+    (LDS-direct kernel where k allows it) and without."""
+    rng = np.random.default_rng(m + 10 * n + 100 * k)
+    packed, ws, a, a_scale = make_problem(rng, m, n, k, full_range=True)
+    tiled = bh.retile_weights(dev(packed), n, k)
+    bias = rng.standard_normal(n, dtype=f32)
+    res = rng.standard_normal((m, n), dtype=f32)
+    acc_ref = orc.gemm_w2a8(packed, a, n)
+    out_ref = orc.epilogue(acc_ref, ws, a_scale, bias, res)
+    for a_sum in (dev(a.astype(np.int32).sum(axis=1).astype(np.int32)), None):
+        acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale), dev(bias), dev(res),
+                                  a_sum=a_sum)
+        assert np.array_equal(host(acc), acc_ref)
+        assert np.array_equal(host(out), out_ref)
+
+
+def test_bitlinear_forward_prefill_uses_quantiser_row_sums():
+    """BitLinear.forward at a prefill token count: quantiser -> row sums -> LDS-direct GEMM, bit-exact."""
+    rng = np.random.default_rng(77)
+    m, k, n = 384, 2560, 640
+    w = synth_weights(rng, n, k)
+    x = synth_activations(rng, m, k, outliers=True)
+    g = (1 + 0.1 * rng.standard_normal(k, dtype=f32)).astype(f32)
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "prefill")
+    layer.update_weights(dev(w))
+    out, q, a_scale, acc = layer.forward(dev(x), gamma=dev(g), debug=True)
+    qw, ws = orc.quantize_weights_absmean(w)
+    out_ref, q_ref, s_ref, acc_ref = orc.bitlinear_forward(x, orc.pack_2bit(qw), n, ws, g=g, eps=1e-5)
+    assert np.array_equal(host(q), q_ref) and np.array_equal(host(a_scale), s_ref)
+    assert np.array_equal(host(acc), acc_ref)
+    assert np.array_equal(host(out), out_ref)
 
 
 # ---- L1: BitLinear object ----------------------------------------------------------------------------------
