@@ -92,6 +92,77 @@ struct bitnet_hip_bitlinear {
     }
 };
 
+namespace {
+
+// Runs `count` projections that share one input row block [m, k].  At decode token counts the quantiser runs
+// inside the GEMV launch (up to GEMV_MAX_PROJ projections per launch); otherwise the stand-alone quantiser
+// fills q / a_scale / a_sum (scratch the caller provides) and the GEMV or GEMM kernels consume them.
+// residual / out / acc are per-projection arrays (entries of residual and acc may be null, and so may the arrays).
+int run_projections(bitnet_hip_bitlinear *const *layers, int count, const float *x, const float *x2, size_t ldx,
+                    size_t m, int input_mode, size_t gqa_group, size_t head_dim, const float *gamma, float eps,
+                    int sum_order, const float *const *residual, float *const *out, int32_t *const *acc, int8_t *q,
+                    float *a_scale, int32_t *a_sum, bool want_quant_outputs, hipStream_t s)
+{
+    const size_t k = layers[0]->in_features;
+    auto proj_of = [&](int j) {
+        bitnet_hip_bitlinear *bl = layers[j];
+        GemvProj pj = {bl->tiled, bl->w_scale, bl->use_bias ? bl->bias : nullptr, residual ? residual[j] : nullptr,
+                       out[j], acc ? acc[j] : nullptr, bl->out_features};
+        return pj;
+    };
+    if (gemv_fused_supported(x, x2, ldx, m, k, input_mode, head_dim, gamma)) {
+        for (int j0 = 0; j0 < count; j0 += GEMV_MAX_PROJ) {
+            GemvProj pjs[GEMV_MAX_PROJ];
+            const int nj = count - j0 < GEMV_MAX_PROJ ? count - j0 : GEMV_MAX_PROJ;
+            for (int j = 0; j < nj; ++j) pjs[j] = proj_of(j0 + j);
+            const bool first = j0 == 0 && want_quant_outputs;
+            int rc = launch_gemv_fused(pjs, nj, x, x2, ldx, m, k, input_mode, gqa_group, head_dim, gamma, eps, sum_order,
+                                       first ? q : nullptr, first ? a_scale : nullptr, first ? a_sum : nullptr, s);
+            if (rc != BITNET_HIP_OK) return rc;
+        }
+        return BITNET_HIP_OK;
+    }
+    if (!q || !a_scale || !a_sum) return fail(BITNET_HIP_MEMORY_ERROR, "projection: no scratch for the quantised activations");
+    int rc = launch_act_quant(x, x2, ldx, m, k, input_mode, gqa_group, head_dim, gamma, eps, sum_order, q, a_scale, a_sum,
+                              nullptr, s);
+    if (rc != BITNET_HIP_OK) return rc;
+    if (m <= (size_t)GEMV_MAX_M) {
+        for (int j0 = 0; j0 < count; j0 += GEMV_MAX_PROJ) {
+            GemvProj pjs[GEMV_MAX_PROJ];
+            const int nj = count - j0 < GEMV_MAX_PROJ ? count - j0 : GEMV_MAX_PROJ;
+            for (int j = 0; j < nj; ++j) pjs[j] = proj_of(j0 + j);
+            rc = launch_gemv_tiled(pjs, nj, q, a_scale, m, k, s);
+            if (rc != BITNET_HIP_OK) return rc;
+        }
+        return BITNET_HIP_OK;
+    }
+    for (int j = 0; j < count; ++j) {
+        GemvProj pj = proj_of(j);
+        rc = launch_gemm_tiled(pj.tiled, q, a_sum, m, pj.n, k, pj.acc, pj.w_scale, a_scale, pj.bias, pj.residual, pj.out, s);
+        if (rc != BITNET_HIP_OK) return rc;
+    }
+    return BITNET_HIP_OK;
+}
+
+// Scratch for the quantised activations of m rows of width k: q [m*k] int8, a_scale [m] f32, a_sum [m] int32.
+struct QuantScratch {
+    int8_t *q;
+    float *a_scale;
+    int32_t *a_sum;
+};
+size_t quant_scratch_bytes(size_t m, size_t k) { return align_up(m * k, 256) + 2 * align_up(m * sizeof(float), 256) + 256; }
+QuantScratch carve_scratch(void *ws, size_t m, size_t k)
+{
+    uintptr_t base = align_up(reinterpret_cast<uintptr_t>(ws), 256);
+    QuantScratch sc;
+    sc.q = reinterpret_cast<int8_t *>(base);
+    sc.a_scale = reinterpret_cast<float *>(base + align_up(m * k, 256));
+    sc.a_sum = reinterpret_cast<int32_t *>(base + align_up(m * k, 256) + align_up(m * sizeof(float), 256));
+    return sc;
+}
+
+}  // namespace
+
 extern "C" {
 
 const char *bitnet_hip_last_error(void) { return error_record().msg; }
@@ -147,7 +218,7 @@ int bitnet_hip_quantize_activations_i8(const float *x, const float *x2, size_t l
     if (m == 0 || k == 0) return BITNET_HIP_OK;
     if (!x || !q || !a_scale) return fail(BITNET_HIP_NULL_POINTER, "quantize_activations_i8: x, q and a_scale are required");
     if (k > 0x7fffffffu) return fail(BITNET_HIP_UNSUPPORTED, "quantize_activations_i8: k=%zu too large", k);
-    if (sum_order != BITNET_HIP_SUM_SEQUENTIAL && sum_order != BITNET_HIP_SUM_WAVE64)
+    if (sum_order != BITNET_HIP_SUM_SEQUENTIAL && sum_order != BITNET_HIP_SUM_BLOCK256)
         return fail(BITNET_HIP_INVALID_CONFIG, "quantize_activations_i8: unknown sum_order %d", sum_order);
     size_t src_cols = k;
     switch (input_mode) {
@@ -270,8 +341,10 @@ int bitnet_hip_matmul_w2a8(const uint8_t *tiled, const int8_t *a, const int32_t 
     if (reinterpret_cast<uintptr_t>(tiled) % 16)
         return fail(BITNET_HIP_INVALID_CONFIG, "matmul_w2a8: tiled weights must be 16-byte aligned");
     if (n > 0x7fffffffu || k > 0x7fffffffu) return fail(BITNET_HIP_UNSUPPORTED, "matmul_w2a8: dimension too large");
-    if (m <= (size_t)GEMV_MAX_M)
-        return launch_gemv_tiled(tiled, a, m, n, k, acc, w_scale, a_scale, bias, residual, out, as_stream(stream));
+    if (m <= (size_t)GEMV_MAX_M) {
+        GemvProj pj = {tiled, w_scale, bias, residual, out, acc, n};
+        return launch_gemv_tiled(&pj, 1, a, a_scale, m, k, as_stream(stream));
+    }
     return launch_gemm_tiled(tiled, a, a_sum, m, n, k, acc, w_scale, a_scale, bias, residual, out, as_stream(stream));
 }
 
@@ -399,7 +472,7 @@ int bitnet_hip_bitlinear_get_quantized(bitnet_hip_bitlinear *layer, float *w_sca
 size_t bitnet_hip_bitlinear_workspace_size(const bitnet_hip_bitlinear *layer, size_t m)
 {
     if (!layer) return 0;
-    return align_up(m * layer->in_features, 256) + 2 * align_up(m * sizeof(float), 256) + 256;
+    return quant_scratch_bytes(m, layer->in_features);
 }
 
 int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, const size_t *dims, int rank,
@@ -408,7 +481,7 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
                                  int32_t *dbg_acc, void *stream)
 {
     if (!layer) return fail(BITNET_HIP_NULL_POINTER, "forward: layer is NULL");
-    const size_t in = layer->in_features, nout = layer->out_features;
+    const size_t in = layer->in_features;
     // shape rules of BitLinearForward::forward (forward.rs:60-76) and quantized_matmul (:179-214)
     if (rank <= 0 || !dims) {
         size_t e[2] = {1, in};
@@ -430,30 +503,79 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
     if (!layer->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "forward: the layer has no weights yet");
 
     hipStream_t s = as_stream(stream);
+    const bool debug = dbg_q || dbg_a_scale || dbg_acc;
+    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma);
     void *ws = workspace;
     bool own_ws = false;
-    const size_t need = bitnet_hip_bitlinear_workspace_size(layer, m);
-    if (!ws) {
-        hipError_t e = hipMallocAsync(&ws, need, s);
-        if (e != hipSuccess) return fail(BITNET_HIP_MEMORY_ERROR, "forward: hipMallocAsync(%zu) failed: %s", need, hipGetErrorString(e));
-        own_ws = true;
-    } else if (workspace_bytes < need) {
-        return fail(BITNET_HIP_MEMORY_ERROR, "forward: workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    QuantScratch sc = {dbg_q, dbg_a_scale, nullptr};
+    if (!fused || debug) {  // the fused decode launch needs no scratch unless the caller wants q / a_scale back
+        const size_t need = quant_scratch_bytes(m, in);
+        if (!ws) {
+            hipError_t e = hipMallocAsync(&ws, need, s);
+            if (e != hipSuccess) return fail(BITNET_HIP_MEMORY_ERROR, "forward: hipMallocAsync(%zu) failed: %s", need, hipGetErrorString(e));
+            own_ws = true;
+        } else if (workspace_bytes < need) {
+            return fail(BITNET_HIP_MEMORY_ERROR, "forward: workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+        }
+        sc = carve_scratch(ws, m, in);
+        if (dbg_q) sc.q = dbg_q;
+        if (dbg_a_scale) sc.a_scale = dbg_a_scale;
     }
-    uintptr_t base = align_up(reinterpret_cast<uintptr_t>(ws), 256);
-    int8_t *q = dbg_q ? dbg_q : reinterpret_cast<int8_t *>(base);
-    float *a_scale = dbg_a_scale ? dbg_a_scale : reinterpret_cast<float *>(base + align_up(m * in, 256));
-    int32_t *a_sum = reinterpret_cast<int32_t *>(base + align_up(m * in, 256) + align_up(m * sizeof(float), 256));
-
-    int rc = launch_act_quant(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, 1, gamma, eps, sum_order, q, a_scale,
-                              a_sum, nullptr, s);
-    if (rc == BITNET_HIP_OK)
-        rc = bitnet_hip_matmul_w2a8(layer->tiled, q, a_sum, m, nout, in, dbg_acc, layer->w_scale, a_scale,
-                                    layer->use_bias ? layer->bias : nullptr, residual, out, stream);
+    bitnet_hip_bitlinear *layers[1] = {layer};
+    const float *res[1] = {residual};
+    float *outs[1] = {out};
+    int32_t *accs[1] = {dbg_acc};
+    int rc = run_projections(layers, 1, x, nullptr, in, m, BITNET_HIP_INPUT_PLAIN, 1, 1, gamma, eps, sum_order, res, outs,
+                             accs, sc.q, sc.a_scale, sc.a_sum, debug, s);
     if (own_ws) {
         hipError_t e = hipFreeAsync(ws, s);
         if (rc == BITNET_HIP_OK && e != hipSuccess)
             rc = fail(BITNET_HIP_MEMORY_ERROR, "forward: hipFreeAsync failed: %s", hipGetErrorString(e));
+    }
+    return rc;
+}
+
+int bitnet_hip_bitlinear_forward_multi(bitnet_hip_bitlinear *const *layers, size_t count, const float *x, size_t m,
+                                       const float *gamma, float eps, int sum_order, float *const *outs, void *workspace,
+                                       size_t workspace_bytes, void *stream)
+{
+    if (!layers || !outs) return fail(BITNET_HIP_NULL_POINTER, "forward_multi: null argument");
+    if (count == 0 || m == 0) return BITNET_HIP_OK;
+    if (count > 16) return fail(BITNET_HIP_INVALID_CONFIG, "forward_multi: at most 16 layers per call, got %zu", count);
+    if (!x) return fail(BITNET_HIP_NULL_POINTER, "forward_multi: x is NULL");
+    std::vector<std::shared_lock<std::shared_mutex>> guards;
+    for (size_t j = 0; j < count; ++j) {
+        if (!layers[j] || !outs[j]) return fail(BITNET_HIP_NULL_POINTER, "forward_multi: layer or output %zu is NULL", j);
+        if (layers[j]->in_features != layers[0]->in_features) {
+            size_t e[2] = {m, layers[0]->in_features}, a[2] = {m, layers[j]->in_features};
+            return fail_shape(e, 2, a, 2, "layers of one forward_multi call must share in_features");
+        }
+        guards.emplace_back(layers[j]->lock);
+        if (!layers[j]->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "forward_multi: layer %zu has no weights yet", j);
+    }
+    const size_t in = layers[0]->in_features;
+    hipStream_t s = as_stream(stream);
+    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma);
+    void *ws = workspace;
+    bool own_ws = false;
+    QuantScratch sc = {nullptr, nullptr, nullptr};
+    if (!fused) {
+        const size_t need = quant_scratch_bytes(m, in);
+        if (!ws) {
+            hipError_t e = hipMallocAsync(&ws, need, s);
+            if (e != hipSuccess) return fail(BITNET_HIP_MEMORY_ERROR, "forward_multi: hipMallocAsync(%zu) failed: %s", need, hipGetErrorString(e));
+            own_ws = true;
+        } else if (workspace_bytes < need) {
+            return fail(BITNET_HIP_MEMORY_ERROR, "forward_multi: workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+        }
+        sc = carve_scratch(ws, m, in);
+    }
+    int rc = run_projections(layers, (int)count, x, nullptr, in, m, BITNET_HIP_INPUT_PLAIN, 1, 1, gamma, eps, sum_order,
+                             nullptr, outs, nullptr, sc.q, sc.a_scale, sc.a_sum, false, s);
+    if (own_ws) {
+        hipError_t e = hipFreeAsync(ws, s);
+        if (rc == BITNET_HIP_OK && e != hipSuccess)
+            rc = fail(BITNET_HIP_MEMORY_ERROR, "forward_multi: hipFreeAsync failed: %s", hipGetErrorString(e));
     }
     return rc;
 }
@@ -476,7 +598,7 @@ int bitnet_hip_bitlinear_matmul(bitnet_hip_bitlinear *layer, const int8_t *a, co
 struct bitnet_hip_decoder {
     size_t layers = 0, hidden = 0, ffn = 0, q_heads = 0, kv_heads = 0, head_dim = 0, max_tokens = 0;
     float eps = 1e-5f;
-    int sum_order = BITNET_HIP_SUM_WAVE64;
+    int sum_order = BITNET_HIP_SUM_BLOCK256;
     std::vector<bitnet_hip_bitlinear *> proj;  // layers * 7
     float *gamma = nullptr;                    // [layers][2][hidden]
     // activation buffers, sized for max_tokens
@@ -605,15 +727,13 @@ int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin
     const size_t H = dec->hidden, F = dec->ffn, KV = dec->kv_heads * dec->head_dim;
     const size_t group = dec->q_heads / dec->kv_heads;
     int rc = BITNET_HIP_OK;
-    auto mm = [&](bitnet_hip_bitlinear *bl, const float *residual, float *out) {
+    // one launch group: `count` projections reading the same (transformed) input
+    auto run = [&](bitnet_hip_bitlinear *const *layers, int count, const float *x, const float *x2, size_t ldx, int mode,
+                   const float *gamma, const float *res0, float *const *outs) {
         if (rc != BITNET_HIP_OK) return;
-        rc = bitnet_hip_matmul_w2a8(bl->tiled, dec->a8, dec->a_sum, m, bl->out_features, bl->in_features, nullptr, bl->w_scale,
-                                    dec->a_scale, nullptr, residual, out, stream);
-    };
-    auto quant = [&](const float *x, const float *x2, size_t ldx, size_t k, int mode, const float *gamma) {
-        if (rc != BITNET_HIP_OK) return;
-        rc = launch_act_quant(x, x2, ldx, m, k, mode, group, dec->head_dim, gamma, dec->eps, dec->sum_order, dec->a8,
-                              dec->a_scale, dec->a_sum, nullptr, s);
+        const float *res[GEMV_MAX_PROJ] = {res0, nullptr, nullptr};
+        rc = run_projections(layers, count, x, x2, ldx, m, mode, group, dec->head_dim, gamma, dec->eps, dec->sum_order, res,
+                             outs, nullptr, dec->a8, dec->a_scale, dec->a_sum, false, s);
     };
     const float *x = x_in;
     for (size_t l = layer_begin; l < layer_end; ++l) {
@@ -622,17 +742,14 @@ int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin
         const bool last = l + 1 == layer_end;
         // hidden states alternate between x_out and the internal buffer so that the last block writes x_out
         float *x2 = ((layer_end - 1 - l) % 2 == 0) ? x_out : dec->ping;
-        quant(x, nullptr, H, H, BITNET_HIP_INPUT_PLAIN, g_attn);
-        mm(P[BITNET_HIP_PROJ_Q], nullptr, (last && q_last) ? q_last : dec->qb);
-        mm(P[BITNET_HIP_PROJ_K], nullptr, (last && k_last) ? k_last : dec->kb);
-        mm(P[BITNET_HIP_PROJ_V], nullptr, dec->vb);
-        quant(dec->vb, nullptr, KV, H, BITNET_HIP_INPUT_GQA_BROADCAST, nullptr);
-        mm(P[BITNET_HIP_PROJ_O], x, dec->x1);
-        quant(dec->x1, nullptr, H, H, BITNET_HIP_INPUT_PLAIN, g_ffn);
-        mm(P[BITNET_HIP_PROJ_GATE], nullptr, dec->gate);
-        mm(P[BITNET_HIP_PROJ_UP], nullptr, dec->up);
-        quant(dec->gate, dec->up, F, F, BITNET_HIP_INPUT_RELU2_MUL, nullptr);
-        mm(P[BITNET_HIP_PROJ_DOWN], dec->x1, x2);
+        float *qkv_out[3] = {(last && q_last) ? q_last : dec->qb, (last && k_last) ? k_last : dec->kb, dec->vb};
+        run(&P[BITNET_HIP_PROJ_Q], 3, x, nullptr, H, BITNET_HIP_INPUT_PLAIN, g_attn, nullptr, qkv_out);
+        float *o_out[1] = {dec->x1};
+        run(&P[BITNET_HIP_PROJ_O], 1, dec->vb, nullptr, KV, BITNET_HIP_INPUT_GQA_BROADCAST, nullptr, x, o_out);
+        float *gu_out[2] = {dec->gate, dec->up};
+        run(&P[BITNET_HIP_PROJ_GATE], 2, dec->x1, nullptr, H, BITNET_HIP_INPUT_PLAIN, g_ffn, nullptr, gu_out);
+        float *d_out[1] = {x2};
+        run(&P[BITNET_HIP_PROJ_DOWN], 1, dec->gate, dec->up, F, BITNET_HIP_INPUT_RELU2_MUL, nullptr, dec->x1, d_out);
         x = x2;
     }
     return rc;

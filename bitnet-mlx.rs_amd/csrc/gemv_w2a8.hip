@@ -13,27 +13,52 @@
 // gemv_tiled_kernel streams the re-tiled layout (weight_prep.hip).  A workgroup of four wavefronts owns
 // one block of 16 output rows; its wavefronts take the k-tiles round-robin, so all of a workgroup's
 // weight bytes are requested in the first few instructions.  Lane l of a wavefront loads the 16 bytes at
-// offset 16*l of a 1 KiB tile: row r = l mod 16, four groups of 16 columns.  Activations sit in LDS
-// (staged once per workgroup); the 16 lanes of a group read the same LDS address (a broadcast).
-// Partial sums are combined with two wavefront shuffles (the four lanes of a row), then across the four
-// wavefronts through LDS.  HBM traffic per call: n*k/4 weight bytes + k activation bytes per row block.
+// offset 16*l of a 1 KiB tile: row r = l mod 16, four groups of 16 columns.  Activations sit in LDS; the 16
+// lanes of a group read the same LDS address (a broadcast).  Partial sums are combined with two wavefront
+// shuffles (the four lanes of a row), then across the four wavefronts through LDS.
+//
+// Two more things are folded into the same launch, because at one token the cost of a decode step is the
+// number of dependent launches, not bytes:
+//   * the activation quantiser: with MODE >= 0 the workgroup reads the f32 row itself, runs RMSNorm +
+//     absmax + int8 rounding (rowquant.hpp, the same code and summation order as the stand-alone
+//     quantiser) and writes the int8 row straight into LDS.  The weight tiles are requested first, so
+//     their HBM latency overlaps this prologue.
+//   * up to three projections that share the input row (q, k, v or gate, up): the grid is the
+//     concatenation of their row blocks.
+// HBM traffic per call: n*k/4 weight bytes; the input row (K or 4K bytes per workgroup) comes from L2.
 #include "kernels.hpp"
+#include "rowquant.hpp"
 
 namespace bitnet {
 
 namespace {
 
-struct GemvParams {
+constexpr int MODE_PREQUANT = -1;
+constexpr int FUSED_NCH = 7;  // 16-byte f32 chunks per thread kept in registers: K <= 7168
+
+struct GemvProjDev {
     const uint8_t *w;
-    const int8_t *a;
-    int32_t *acc;
     const float *w_scale;
-    const float *a_scale;
     const float *bias;
     const float *residual;
     float *out;
-    int m;  // tokens in this launch (<= MB)
+    int32_t *acc;
     int n;
+    int rb_end;  // row blocks of projections 0..this one, cumulative
+};
+
+struct GemvParams {
+    GemvProjDev proj[GEMV_MAX_PROJ];
+    int nproj;
+    // MODE_PREQUANT: activations already int8
+    const int8_t *a;
+    const float *a_scale;
+    // MODE >= 0: f32 input, quantised in the prologue
+    RowSource src;
+    int8_t *q_out;        // optional copies of what the prologue produced (written by workgroup 0)
+    float *a_scale_out;
+    int32_t *a_sum_out;
+    int m;  // tokens in this launch (<= MB)
     int k;
     int kt_count;
 };
@@ -62,16 +87,26 @@ __device__ __forceinline__ int dot64(const uint4 &w4, const uint4 *ag, int acc)
 
 constexpr int GEMV_PREFETCH = 4;  // tiles in flight per wavefront
 
-template <int MB>
+template <int MB, int MODE>
 __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
 {
-    extern __shared__ uint4 lds_a[];  // [MB][groups]: activations, 16 per uint4, zero past K / past m
+    extern __shared__ uint4 lds_a[];  // [MB][groups]: int8 activations, 16 per uint4, zero past K / past m
     __shared__ int red[4][TILE_ROWS][MB];
-    __shared__ int asum[MB];
+    __shared__ float red_f[MB][2][4];
+    __shared__ int red_i[MB][4];
+    __shared__ float scale_s[MB];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int groups = p.kt_count * 16;
-    const uint4 *tiles = reinterpret_cast<const uint4 *>(p.w) + (size_t)blockIdx.x * p.kt_count * 64;
+
+    // which projection, which of its row blocks
+    int pj = 0;
+#pragma unroll
+    for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
+        if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
+    const GemvProjDev &P = p.proj[pj];
+    const int rb = (int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0);
+    const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + (size_t)rb * p.kt_count * 64;
 
     // Request the first batch of weight tiles before anything else.
     uint4 wbuf[GEMV_PREFETCH];
@@ -81,37 +116,109 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
         wbuf[u] = kt < p.kt_count ? tiles[(size_t)kt * 64 + lane] : make_uint4(0, 0, 0, 0);
     }
 
-    // Stage activations; every thread also accumulates sum_k a[t, k] for the code offset.
-    if (tid < MB) asum[tid] = 0;
-    __syncthreads();
-    const bool vec_ok = (p.k % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0);
+    if constexpr (MODE == MODE_PREQUANT) {
+        // Stage the int8 activations; every thread also accumulates sum_k a[t, k] for the code offset.
+        const bool vec_ok = (p.k % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0);
 #pragma unroll
-    for (int t = 0; t < MB; ++t) {
-        int local = 0;
-        for (int g = tid; g < groups; g += 256) {
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (t < p.m) {
-                const int8_t *src = p.a + (size_t)t * p.k + 16 * (size_t)g;
-                if (vec_ok) {
-                    if (16 * g < p.k) v = *reinterpret_cast<const uint4 *>(src);
+        for (int t = 0; t < MB; ++t) {
+            int local = 0;
+            for (int g = tid; g < groups; g += 256) {
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (t < p.m) {
+                    const int8_t *srcp = p.a + (size_t)t * p.k + 16 * (size_t)g;
+                    if (vec_ok) {
+                        if (16 * g < p.k) v = *reinterpret_cast<const uint4 *>(srcp);
+                    } else {
+                        uint32_t d[4] = {0, 0, 0, 0};
+                        for (int j = 0; j < 16; ++j)
+                            if (16 * g + j < p.k) d[j >> 2] |= (uint32_t)(uint8_t)srcp[j] << (8 * (j & 3));
+                        v = make_uint4(d[0], d[1], d[2], d[3]);
+                    }
+                }
+                lds_a[t * groups + g] = v;
+                local = dot4(v.x, 0x01010101u, local);
+                local = dot4(v.y, 0x01010101u, local);
+                local = dot4(v.z, 0x01010101u, local);
+                local = dot4(v.w, 0x01010101u, local);
+            }
+            local = wave_sum_i32(local);
+            if (lane == 0) red_i[t][wave] = local;
+            if (tid == 0) scale_s[t] = (t < p.m && p.a_scale) ? p.a_scale[t] : 1.0f;
+        }
+    } else {
+        // Quantise the f32 input row(s) here: thread tid is virtual lane tid of the declared summation order.
+        const RowSource &src = p.src;
+        const int chunks = p.k >> 2;  // the host takes this path only when K % 4 == 0
+        const int lds_words = groups * 4;
+        uint32_t *lds_w = reinterpret_cast<uint32_t *>(lds_a);
+        const bool norm = src.gamma != nullptr;
+#pragma unroll
+        for (int t = 0; t < MB; ++t) {
+            if (t >= p.m) {  // uniform
+                for (int c = tid; c < lds_words; c += 256) lds_w[t * lds_words + c] = 0;
+                if (lane == 0) red_i[t][wave] = 0;
+                if (tid == 0) scale_s[t] = 1.0f;
+                continue;
+            }
+            float4 v[FUSED_NCH];
+#pragma unroll
+            for (int i = 0; i < FUSED_NCH; ++i) {
+                int c = tid + 256 * i;
+                v[i] = c < chunks ? load_chunk<MODE, true>(src, (size_t)t, c) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            float rms = 1.0f;
+            if (norm) {
+                float ss;
+                if (src.sum_order == BITNET_HIP_SUM_SEQUENTIAL) {
+                    ss = sum_squares_sequential<MODE>(src, (size_t)t);
                 } else {
-                    uint32_t d[4] = {0, 0, 0, 0};
-                    for (int j = 0; j < 16; ++j)
-                        if (16 * g + j < p.k) d[j >> 2] |= (uint32_t)(uint8_t)src[j] << (8 * (j & 3));
-                    v = make_uint4(d[0], d[1], d[2], d[3]);
+                    float part = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < FUSED_NCH; ++i) part = sum_squares4(part, v[i]);
+                    part = wave_sum_f32(part);
+                    if (lane == 0) red_f[t][0][wave] = part;
+                    __syncthreads();
+                    ss = f32_add(f32_add(f32_add(red_f[t][0][0], red_f[t][0][1]), red_f[t][0][2]), red_f[t][0][3]);
+                }
+                rms = rms_from_ss(ss, p.k, src.eps);
+            }
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < FUSED_NCH; ++i) {
+                int c = tid + 256 * i;
+                if (norm && c < chunks) v[i] = normalize4(v[i], rms, load_gamma_chunk(src, c, true));
+                amax = absmax4(amax, v[i]);
+            }
+            amax = wave_max_f32(amax);
+            if (lane == 0) red_f[t][1][wave] = amax;
+            __syncthreads();
+            amax = fmaxf(fmaxf(red_f[t][1][0], red_f[t][1][1]), fmaxf(red_f[t][1][2], red_f[t][1][3]));
+            const float scale = scale_from_absmax(amax);
+            int isum = 0;
+#pragma unroll
+            for (int i = 0; i < FUSED_NCH; ++i) {
+                int c = tid + 256 * i;
+                if (c < chunks) {
+                    uint32_t packed = quant4_packed(v[i], scale, &isum);
+                    lds_w[t * lds_words + c] = packed;
+                    if (p.q_out && blockIdx.x == 0) reinterpret_cast<uint32_t *>(p.q_out)[(size_t)t * chunks + c] = packed;
+                } else if (c < lds_words) {
+                    lds_w[t * lds_words + c] = 0;
                 }
             }
-            lds_a[t * groups + g] = v;
-            local = dot4(v.x, 0x01010101u, local);
-            local = dot4(v.y, 0x01010101u, local);
-            local = dot4(v.z, 0x01010101u, local);
-            local = dot4(v.w, 0x01010101u, local);
+            isum = wave_sum_i32(isum);
+            if (lane == 0) red_i[t][wave] = isum;
+            if (tid == 0) scale_s[t] = scale;
         }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) local += __shfl_xor(local, off, 64);
-        if (lane == 0) atomicAdd(&asum[t], local);
     }
     __syncthreads();
+
+    if constexpr (MODE != MODE_PREQUANT) {
+        if (blockIdx.x == 0 && tid < MB && tid < p.m) {
+            if (p.a_scale_out) p.a_scale_out[tid] = scale_s[tid];
+            if (p.a_sum_out) p.a_sum_out[tid] = red_i[tid][0] + red_i[tid][1] + red_i[tid][2] + red_i[tid][3];
+        }
+    }
 
     int acc[MB];
 #pragma unroll
@@ -138,7 +245,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
         for (int u = 0; u < GEMV_PREFETCH; ++u) wbuf[u] = wnext[u];
     }
 
-    // the four lanes l, l+16, l+32, l+48 hold the four column quarters of row l mod 16
+    // the four lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
 #pragma unroll
     for (int t = 0; t < MB; ++t) {
         acc[t] += __shfl_xor(acc[t], 16, 64);
@@ -152,17 +259,18 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
 
     if (tid < TILE_ROWS * MB) {
         const int r = tid / MB, t = tid % MB;
-        const int n = blockIdx.x * TILE_ROWS + r;
-        if (n < p.n && t < p.m) {
-            int total = red[0][r][t] + red[1][r][t] + red[2][r][t] + red[3][r][t] - asum[t];
-            size_t o = (size_t)t * p.n + n;
-            if (p.acc) p.acc[o] = total;
-            if (p.out) {
-                float v = f32_mul((float)total, *p.w_scale);
-                v = f32_div(v, p.a_scale[t]);
-                if (p.bias) v = f32_add(v, p.bias[n]);
-                if (p.residual) v = f32_add(v, p.residual[o]);
-                p.out[o] = v;
+        const int n = rb * TILE_ROWS + r;
+        if (n < P.n && t < p.m) {
+            const int asum = red_i[t][0] + red_i[t][1] + red_i[t][2] + red_i[t][3];
+            int total = red[0][r][t] + red[1][r][t] + red[2][r][t] + red[3][r][t] - asum;
+            size_t o = (size_t)t * P.n + n;
+            if (P.acc) P.acc[o] = total;
+            if (P.out) {
+                float v = f32_mul((float)total, *P.w_scale);
+                v = f32_div(v, scale_s[t]);
+                if (P.bias) v = f32_add(v, P.bias[n]);
+                if (P.residual) v = f32_add(v, P.residual[o]);
+                P.out[o] = v;
             }
         }
     }
@@ -205,21 +313,58 @@ __global__ __launch_bounds__(256) void gemv_rowmajor_kernel(const uint8_t *packe
             }
         }
     }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    acc = wave_sum_i32(acc);
     if (lane == 0) out[row] = acc;
 }
 
-template <int MB>
-int launch_tiled_mb(const GemvParams &p, hipStream_t stream)
+template <int MB, int MODE>
+int launch_mb_mode(const GemvParams &p, hipStream_t stream)
 {
     size_t lds = (size_t)MB * p.kt_count * 16 * sizeof(uint4);
-    if (lds > 60 * 1024)
-        return fail(BITNET_HIP_UNSUPPORTED, "decode GEMV: %d tokens x k=%d need %zu bytes of LDS", MB, p.k, lds);
-    dim3 grid((unsigned)row_blocks((size_t)p.n));
-    hipLaunchKernelGGL((gemv_tiled_kernel<MB>), grid, dim3(256), lds, stream, p);
+    dim3 grid((unsigned)p.proj[p.nproj - 1].rb_end);
+    hipLaunchKernelGGL((gemv_tiled_kernel<MB, MODE>), grid, dim3(256), lds, stream, p);
     BITNET_HIP_CHECK_LAUNCH("gemv_tiled_kernel");
     return BITNET_HIP_OK;
+}
+
+template <int MODE>
+int launch_mode(const GemvParams &p, int mb, hipStream_t stream)
+{
+    switch (mb) {
+        case 8: return launch_mb_mode<8, MODE>(p, stream);
+        case 4: return launch_mb_mode<4, MODE>(p, stream);
+        case 2: return launch_mb_mode<2, MODE>(p, stream);
+        default: return launch_mb_mode<1, MODE>(p, stream);
+    }
+}
+
+// rows per launch that fit the 60 KB LDS budget
+int rows_per_launch(size_t m, size_t k)
+{
+    const size_t row_lds = k_tiles(k) * 16 * sizeof(uint4);
+    int mb = m > 4 ? 8 : (m > 2 ? 4 : (m > 1 ? 2 : 1));
+    while (mb > 1 && mb * row_lds > 60 * 1024) mb >>= 1;
+    return mb;
+}
+
+int fill_projs(GemvParams &p, const GemvProj *projs, int nproj, size_t t0, size_t k)
+{
+    int rb_end = 0;
+    for (int j = 0; j < nproj; ++j) {
+        const GemvProj &s = projs[j];
+        GemvProjDev &d = p.proj[j];
+        d.w = s.tiled; d.w_scale = s.w_scale; d.bias = s.bias; d.n = (int)s.n;
+        d.residual = s.residual ? s.residual + t0 * s.n : nullptr;
+        d.out = s.out ? s.out + t0 * s.n : nullptr;
+        d.acc = s.acc ? s.acc + t0 * s.n : nullptr;
+        rb_end += (int)row_blocks(s.n);
+        d.rb_end = rb_end;
+    }
+    for (int j = nproj; j < GEMV_MAX_PROJ; ++j) p.proj[j] = p.proj[nproj - 1];
+    p.nproj = nproj;
+    p.k = (int)k;
+    p.kt_count = (int)k_tiles(k);
+    return rb_end;
 }
 
 }  // namespace
@@ -234,36 +379,55 @@ int launch_gemv_rowmajor(const uint8_t *packed, const int8_t *a, int32_t *out, s
     return BITNET_HIP_OK;
 }
 
-int launch_gemv_tiled(const uint8_t *tiled, const int8_t *a, size_t m, size_t n, size_t k, int32_t *acc,
-                      const float *w_scale, const float *a_scale, const float *bias, const float *residual,
-                      float *out, hipStream_t stream)
+int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const float *a_scale, size_t m, size_t k,
+                      hipStream_t stream)
 {
-    if (m == 0 || n == 0) return BITNET_HIP_OK;
-    GemvParams p;
-    p.w = tiled; p.a = a; p.acc = acc; p.w_scale = w_scale; p.a_scale = a_scale; p.bias = bias;
-    p.residual = residual; p.out = out; p.m = (int)m; p.n = (int)n; p.k = (int)k; p.kt_count = (int)k_tiles(k);
-    // LDS holds MB activation rows; fall back to fewer rows per launch for very long rows.
-    const size_t row_lds = (size_t)p.kt_count * 16 * sizeof(uint4);
-    int mb = m >= 8 ? 8 : (m >= 4 ? 4 : (m >= 2 ? 2 : 1));
-    while (mb > 1 && mb * row_lds > 60 * 1024) mb >>= 1;
+    if (m == 0 || nproj <= 0) return BITNET_HIP_OK;
+    if (k_tiles(k) * 16 * sizeof(uint4) > 60 * 1024)
+        return fail(BITNET_HIP_UNSUPPORTED, "decode GEMV: k=%zu does not fit the LDS activation buffer", k);
+    const int mb = rows_per_launch(m, k);
     for (size_t t0 = 0; t0 < m; t0 += (size_t)mb) {
-        GemvParams q = p;
-        q.m = (int)((m - t0) < (size_t)mb ? (m - t0) : (size_t)mb);
-        q.a = a + t0 * k;
-        if (acc) q.acc = acc + t0 * n;
-        if (out) q.out = out + t0 * n;
-        if (a_scale) q.a_scale = a_scale + t0;
-        if (residual) q.residual = residual + t0 * n;
-        int rc;
-        switch (mb) {
-            case 8: rc = launch_tiled_mb<8>(q, stream); break;
-            case 4: rc = launch_tiled_mb<4>(q, stream); break;
-            case 2: rc = launch_tiled_mb<2>(q, stream); break;
-            default: rc = launch_tiled_mb<1>(q, stream); break;
-        }
+        GemvParams p = {};
+        if (fill_projs(p, projs, nproj, t0, k) == 0) return BITNET_HIP_OK;
+        p.m = (int)((m - t0) < (size_t)mb ? (m - t0) : (size_t)mb);
+        p.a = a + t0 * k;
+        p.a_scale = a_scale ? a_scale + t0 : nullptr;
+        int rc = launch_mode<MODE_PREQUANT>(p, mb, stream);
         if (rc != BITNET_HIP_OK) return rc;
     }
     return BITNET_HIP_OK;
+}
+
+bool gemv_fused_supported(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
+                          size_t head_dim, const float *gamma)
+{
+    auto al16 = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+    if (m == 0 || m > (size_t)GEMV_MAX_M) return false;
+    if (k % 4 != 0 || ldx % 4 != 0 || k > (size_t)FUSED_NCH * 1024) return false;
+    if (!al16(x) || (x2 && !al16(x2)) || (gamma && !al16(gamma))) return false;
+    if (input_mode == BITNET_HIP_INPUT_GQA_BROADCAST && head_dim % 4 != 0) return false;
+    if ((size_t)rows_per_launch(m, k) < m) return false;  // one launch must hold every row
+    return k_tiles(k) * 16 * sizeof(uint4) <= 60 * 1024;
+}
+
+int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const float *x2, size_t ldx, size_t m,
+                      size_t k, int input_mode, size_t gqa_group, size_t head_dim, const float *gamma, float eps,
+                      int sum_order, int8_t *q_out, float *a_scale_out, int32_t *a_sum_out, hipStream_t stream)
+{
+    if (m == 0 || nproj <= 0) return BITNET_HIP_OK;
+    GemvParams p = {};
+    if (fill_projs(p, projs, nproj, 0, k) == 0) return BITNET_HIP_OK;
+    p.m = (int)m;
+    p.src.x = x; p.src.x2 = x2; p.src.gamma = gamma; p.src.ldx = ldx; p.src.k = (int)k;
+    p.src.head_dim = (int)(head_dim ? head_dim : 1); p.src.gqa_group = (int)(gqa_group ? gqa_group : 1);
+    p.src.sum_order = sum_order; p.src.eps = eps;
+    p.q_out = q_out; p.a_scale_out = a_scale_out; p.a_sum_out = a_sum_out;
+    const int mb = rows_per_launch(m, k);
+    switch (input_mode) {
+        case BITNET_HIP_INPUT_PLAIN: return launch_mode<BITNET_HIP_INPUT_PLAIN>(p, mb, stream);
+        case BITNET_HIP_INPUT_RELU2_MUL: return launch_mode<BITNET_HIP_INPUT_RELU2_MUL>(p, mb, stream);
+        default: return launch_mode<BITNET_HIP_INPUT_GQA_BROADCAST>(p, mb, stream);
+    }
 }
 
 }  // namespace bitnet

@@ -32,11 +32,29 @@ int launch_untile(const uint8_t *tiled, size_t n, size_t k, uint8_t *packed, hip
 // gemv_w2a8.hip
 int launch_gemv_rowmajor(const uint8_t *packed, const int8_t *a, int32_t *out, size_t n, size_t k,
                          hipStream_t stream);
-// m <= GEMV_MAX_M tokens per launch
-constexpr int GEMV_MAX_M = 8;
-int launch_gemv_tiled(const uint8_t *tiled, const int8_t *a, size_t m, size_t n, size_t k, int32_t *acc,
-                      const float *w_scale, const float *a_scale, const float *bias, const float *residual,
-                      float *out, hipStream_t stream);
+constexpr int GEMV_MAX_M = 8;     // token rows one decode-GEMV launch can hold
+constexpr int GEMV_MAX_PROJ = 3;  // projections sharing one input row per launch (q,k,v / gate,up)
+// One projection of a decode-GEMV launch: re-tiled weights [n, k], its scale, optional bias [n] and
+// residual [m, n]; out [m, n] f32 and acc [m, n] int32 are each optional.
+struct GemvProj {
+    const uint8_t *tiled;
+    const float *w_scale;
+    const float *bias;
+    const float *residual;
+    float *out;
+    int32_t *acc;
+    size_t n;
+};
+// activations already int8 ([m, k], a_scale [m]); any m (launched in groups of up to GEMV_MAX_M rows)
+int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const float *a_scale, size_t m, size_t k,
+                      hipStream_t stream);
+// f32 input quantised inside the GEMV launch; only where gemv_fused_supported() says so.  q_out / a_scale_out /
+// a_sum_out (each optional) receive the quantiser's results.
+bool gemv_fused_supported(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
+                          size_t head_dim, const float *gamma);
+int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const float *x2, size_t ldx, size_t m,
+                      size_t k, int input_mode, size_t gqa_group, size_t head_dim, const float *gamma, float eps,
+                      int sum_order, int8_t *q_out, float *a_scale_out, int32_t *a_sum_out, hipStream_t stream);
 
 // gemm_w2a8.hip
 // a_sum (sum_k a[t, k] per row, from the activation quantiser) may be NULL: the slower kernel then computes it

@@ -1,0 +1,180 @@
+// Device-side pieces of the fused RMSNorm + per-token absmax int8 quantiser, shared by the stand-alone
+// quantiser kernels (act_quant.hip) and by the decode GEMV, which quantises its input row itself
+// (gemv_w2a8.hip).  Every caller produces the same bits for the same row.
+//
+// Arithmetic (each f32 step one IEEE operation):
+//   ss      = sum_k x[k]*x[k]                      bitnet-inference/src/engine/inference_integration.rs:476
+//   rms     = sqrt(ss / K + eps)                   :477
+//   y[k]    = (x[k] / rms) * gamma[k]              :481
+//   absmax  = max_k |y[k]|                         bitnet-inference/src/engine/ternary_operations.rs:143-145
+//   a_scale = absmax > 0 ? 127 / absmax : 1        :147-151
+//   q[k]    = clamp(round(y[k] * a_scale),-128,127) :158-161  (round = half away from zero)
+//
+// Order of the f32 sum of squares, the only order-dependent step (BITNET_HIP_SUM_BLOCK256):
+//   the row is cut into chunks of 4 consecutive elements; chunk c belongs to virtual lane c mod 256; a lane
+//   adds the squares of its chunks in ascending chunk order and, inside a chunk, ascending element order,
+//   starting from +0; the 256 partials form 4 groups of 64 consecutive lanes, each combined by the butterfly
+//   p[l] += p[l ^ off], off = 32,16,8,4,2,1; the four group sums are added as ((s0 + s1) + s2) + s3.
+//   A 256-thread workgroup maps thread = virtual lane; a single wavefront keeps 4 partials per lane
+//   (virtual lanes l, l+64, l+128, l+192).  Elements past K count as 0.
+// BITNET_HIP_SUM_SEQUENTIAL is the reference's literal running sum over k ascending.
+#pragma once
+#include "common.hpp"
+#include "ieee.hpp"
+
+namespace bitnet {
+
+struct RowSource {
+    const float *x;      // [m, ldx]
+    const float *x2;     // second operand of RELU2_MUL
+    const float *gamma;  // RMSNorm weight or nullptr
+    size_t ldx;
+    int k;
+    int head_dim;
+    int gqa_group;
+    int sum_order;
+    float eps;
+};
+
+__device__ __forceinline__ float wave_sum_f32(float p)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) p = f32_add(p, __shfl_xor(p, off, 64));
+    return p;
+}
+
+__device__ __forceinline__ float wave_max_f32(float p)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) p = fmaxf(p, __shfl_xor(p, off, 64));
+    return p;
+}
+
+__device__ __forceinline__ int wave_sum_i32(int p)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) p += __shfl_xor(p, off, 64);
+    return p;
+}
+
+__device__ __forceinline__ float relu2_mul(float gate, float up)
+{
+    float r = gate > 0.0f ? gate : 0.0f;
+    return f32_mul(up, f32_mul(r, r));
+}
+
+// Element i of the (virtual) input row after the fused input transform.
+template <int MODE>
+__device__ __forceinline__ float load_elem(const RowSource &p, size_t row, int i)
+{
+    if constexpr (MODE == BITNET_HIP_INPUT_PLAIN) {
+        return p.x[row * p.ldx + i];
+    } else if constexpr (MODE == BITNET_HIP_INPUT_RELU2_MUL) {
+        return relu2_mul(p.x[row * p.ldx + i], p.x2[row * p.ldx + i]);
+    } else {
+        int h = i / p.head_dim, d = i - h * p.head_dim;
+        return p.x[row * p.ldx + (size_t)(h / p.gqa_group) * p.head_dim + d];
+    }
+}
+
+// Chunk c (elements 4c .. 4c+3).  VEC: 16-byte loads, all four elements inside the row.
+template <int MODE, bool VEC>
+__device__ __forceinline__ float4 load_chunk(const RowSource &p, size_t row, int c)
+{
+    if constexpr (VEC) {
+        if constexpr (MODE == BITNET_HIP_INPUT_PLAIN) {
+            return *reinterpret_cast<const float4 *>(p.x + row * p.ldx + 4 * (size_t)c);
+        } else if constexpr (MODE == BITNET_HIP_INPUT_RELU2_MUL) {
+            float4 g = *reinterpret_cast<const float4 *>(p.x + row * p.ldx + 4 * (size_t)c);
+            float4 u = *reinterpret_cast<const float4 *>(p.x2 + row * p.ldx + 4 * (size_t)c);
+            return make_float4(relu2_mul(g.x, u.x), relu2_mul(g.y, u.y), relu2_mul(g.z, u.z),
+                               relu2_mul(g.w, u.w));
+        } else {
+            int i = 4 * c;
+            int h = i / p.head_dim, d = i - h * p.head_dim;
+            return *reinterpret_cast<const float4 *>(p.x + row * p.ldx +
+                                                     (size_t)(h / p.gqa_group) * p.head_dim + d);
+        }
+    } else {
+        float4 v;
+        int i = 4 * c;
+        v.x = i + 0 < p.k ? load_elem<MODE>(p, row, i + 0) : 0.0f;
+        v.y = i + 1 < p.k ? load_elem<MODE>(p, row, i + 1) : 0.0f;
+        v.z = i + 2 < p.k ? load_elem<MODE>(p, row, i + 2) : 0.0f;
+        v.w = i + 3 < p.k ? load_elem<MODE>(p, row, i + 3) : 0.0f;
+        return v;
+    }
+}
+
+__device__ __forceinline__ float4 load_gamma_chunk(const RowSource &p, int c, bool vec)
+{
+    if (vec) return *reinterpret_cast<const float4 *>(p.gamma + 4 * (size_t)c);
+    float4 g;
+    int i = 4 * c;
+    g.x = i + 0 < p.k ? p.gamma[i + 0] : 0.0f;
+    g.y = i + 1 < p.k ? p.gamma[i + 1] : 0.0f;
+    g.z = i + 2 < p.k ? p.gamma[i + 2] : 0.0f;
+    g.w = i + 3 < p.k ? p.gamma[i + 3] : 0.0f;
+    return g;
+}
+
+__device__ __forceinline__ float sum_squares4(float part, const float4 &e)
+{
+    part = f32_add(part, f32_mul(e.x, e.x));
+    part = f32_add(part, f32_mul(e.y, e.y));
+    part = f32_add(part, f32_mul(e.z, e.z));
+    part = f32_add(part, f32_mul(e.w, e.w));
+    return part;
+}
+
+// The reference's literal order: every lane runs the same chain over the whole row.
+template <int MODE>
+__device__ __forceinline__ float sum_squares_sequential(const RowSource &p, size_t row)
+{
+    float ss = 0.0f;
+    for (int i = 0; i < p.k; ++i) {
+        float e = load_elem<MODE>(p, row, i);
+        ss = f32_add(ss, f32_mul(e, e));
+    }
+    return ss;
+}
+
+__device__ __forceinline__ float rms_from_ss(float ss, int k, float eps)
+{
+    return f32_sqrt(f32_add(f32_div(ss, (float)k), eps));
+}
+
+__device__ __forceinline__ float4 normalize4(const float4 &e, float rms, const float4 &g)
+{
+    return make_float4(f32_mul(f32_div(e.x, rms), g.x), f32_mul(f32_div(e.y, rms), g.y),
+                       f32_mul(f32_div(e.z, rms), g.z), f32_mul(f32_div(e.w, rms), g.w));
+}
+
+__device__ __forceinline__ float absmax4(float amax, const float4 &e)
+{
+    return fmaxf(amax, fmaxf(fmaxf(fabsf(e.x), fabsf(e.y)), fmaxf(fabsf(e.z), fabsf(e.w))));
+}
+
+__device__ __forceinline__ float scale_from_absmax(float amax)
+{
+    return amax > 0.0f ? f32_div(127.0f, amax) : 1.0f;
+}
+
+__device__ __forceinline__ int quant1(float y, float scale)
+{
+    float t = roundf(f32_mul(y, scale));
+    if (t != t) return 0;  // NaN quantises to 0, as Rust's `as i8` does
+    t = fminf(fmaxf(t, -128.0f), 127.0f);
+    return (int)t;
+}
+
+// Four quantised values of a chunk packed little-endian (byte j = element j); *sum += their sum.
+__device__ __forceinline__ uint32_t quant4_packed(const float4 &e, float scale, int *sum)
+{
+    int q0 = quant1(e.x, scale), q1 = quant1(e.y, scale), q2 = quant1(e.z, scale), q3 = quant1(e.w, scale);
+    *sum += q0 + q1 + q2 + q3;
+    return (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) |
+           ((uint32_t)(q3 & 0xff) << 24);
+}
+
+}  // namespace bitnet

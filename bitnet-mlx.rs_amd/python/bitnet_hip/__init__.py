@@ -36,7 +36,7 @@ NULL_POINTER = 8
 UNSUPPORTED = 9
 
 SUM_SEQUENTIAL = 0
-SUM_WAVE64 = 1
+SUM_BLOCK256 = 1
 LAYOUT_OUT_IN = 0
 LAYOUT_IN_OUT = 1
 TERNARY_ABSMEAN_ROUNDCLIP = 0
@@ -102,6 +102,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_bitlinear_get_quantized": (i32, [vp, C.POINTER(f32), vp, sz]),
         "bitnet_hip_bitlinear_workspace_size": (sz, [vp, sz]),
         "bitnet_hip_bitlinear_forward": (i32, [vp, vp, C.POINTER(sz), i32, vp, f32, i32, vp, vp, vp, sz, vp, vp, vp, vp]),
+        "bitnet_hip_bitlinear_forward_multi": (i32, [C.POINTER(vp), sz, vp, sz, vp, f32, i32, C.POINTER(vp), vp, sz, vp]),
         "bitnet_hip_bitlinear_matmul": (i32, [vp, vp, vp, sz, vp, vp, vp, vp, vp]),
         "bitnet_hip_decoder_decode_layers": (i32, [vp, sz, sz, vp, sz, vp, vp, vp, vp]),
         "bitnet_hip_decoder_create": (i32, [sz, sz, sz, sz, sz, sz, f32, i32, sz, C.POINTER(vp)]),
@@ -175,7 +176,7 @@ def device_info():
 # ---- raw operators ------------------------------------------------------------------------------
 
 def quantize_activations_i8(x: torch.Tensor, gamma: Optional[torch.Tensor] = None, eps: float = 1e-5,
-                            sum_order: int = SUM_WAVE64, x2: Optional[torch.Tensor] = None,
+                            sum_order: int = SUM_BLOCK256, x2: Optional[torch.Tensor] = None,
                             input_mode: int = INPUT_PLAIN, gqa_group: int = 1, head_dim: int = 1,
                             want_sum: bool = False, want_y: bool = False, stream=None):
     """Fused RMSNorm (if gamma) + per-token absmax int8 quantisation of a [m, k] f32 matrix."""
@@ -306,7 +307,7 @@ class BitLinearConfig:
     ternary_method: int = TERNARY_ABSMEAN_ROUNDCLIP
     threshold_factor: float = 0.5
     rms_norm_eps: float = 1e-5
-    sum_order: int = SUM_WAVE64
+    sum_order: int = SUM_BLOCK256
 
 
 class BitLinear:
@@ -405,11 +406,29 @@ class BitLinear:
         return self.forward(x)
 
 
+def forward_multi(layers: Sequence["BitLinear"], x: torch.Tensor, gamma: Optional[torch.Tensor] = None, stream=None):
+    """Several BitLinear layers on one input [m, in] (q/k/v, gate/up): one activation quantisation, shared launches."""
+    _dev(x, torch.float32, "input")
+    if x.dim() != 2:
+        raise BitLinearError(SHAPE_MISMATCH, "forward_multi takes a [m, in] input", [1, layers[0].config.in_features],
+                             list(x.shape))
+    m = x.shape[0]
+    outs = [torch.empty((m, l.config.out_features), dtype=torch.float32, device=x.device) for l in layers]
+    if x.shape[1] != layers[0].config.in_features:
+        raise BitLinearError(SHAPE_MISMATCH, "last input dimension", [m, layers[0].config.in_features], list(x.shape))
+    hs = (C.c_void_p * len(layers))(*[l._h for l in layers])
+    os_ = (C.c_void_p * len(layers))(*[o.data_ptr() for o in outs])
+    cfg = layers[0].config
+    _check(load_library().bitnet_hip_bitlinear_forward_multi(hs, len(layers), _ptr(x), m, _ptr(gamma), cfg.rms_norm_eps,
+                                                             cfg.sum_order, os_, None, 0, _stream(stream)))
+    return outs
+
+
 class DecoderProjections:
     """The seven BitLinear projections of a stack of decoder blocks at decode time."""
 
     def __init__(self, layers: int, hidden: int = 2560, ffn: int = 6912, q_heads: int = 20, kv_heads: int = 5,
-                 head_dim: int = 128, eps: float = 1e-5, sum_order: int = SUM_WAVE64, max_tokens: int = 8):
+                 head_dim: int = 128, eps: float = 1e-5, sum_order: int = SUM_BLOCK256, max_tokens: int = 8):
         lib = load_library()
         h = C.c_void_p()
         _check(lib.bitnet_hip_decoder_create(layers, hidden, ffn, q_heads, kv_heads, head_dim, eps, sum_order,

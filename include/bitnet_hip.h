@@ -41,7 +41,8 @@ typedef enum bitnet_hip_status {
 /* Order of the f32 sum of squares inside RMSNorm. */
 #define BITNET_HIP_SUM_SEQUENTIAL 0 /* one running sum, k ascending: the literal order of
                                        bitnet-inference/src/engine/inference_integration.rs:476 (slow) */
-#define BITNET_HIP_SUM_WAVE64 1     /* 64 lane-strided partials + xor butterfly (default, one wavefront pass) */
+#define BITNET_HIP_SUM_BLOCK256 1   /* 256 lane-strided partials, four 64-lane xor butterflies, then
+                                       ((s0+s1)+s2)+s3 (default; one wavefront or one workgroup pass) */
 
 /* Weight matrix orientation handed to set_weights. */
 #define BITNET_HIP_LAYOUT_OUT_IN 0 /* [out_features, in_features], bitnet-quant/src/bitlinear/layer.rs:86,122 */
@@ -201,6 +202,16 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
                                  const float *gamma, float eps, int sum_order, const float *residual,
                                  float *out, void *workspace, size_t workspace_bytes, int8_t *dbg_q,
                                  float *dbg_a_scale, int32_t *dbg_acc, void *stream);
+
+/* Several layers applied to the same input x [m, in] (q, k, v of an attention block; gate, up of an FFN):
+ * MultiHeadAttention::forward runs q_proj/k_proj/v_proj on one input
+ * (bitnet-inference/src/engine/transformer_layers.rs:470-475), FeedForwardNetwork::forward up_proj/gate_proj
+ * (:605-611).  The input is quantised once; at decode token counts up to three layers share one kernel
+ * launch.  outs[j] is [m, out_features of layers[j]].  All layers must have the same in_features
+ * (else SHAPE_MISMATCH).  workspace as for bitnet_hip_bitlinear_forward (sized for layers[0]). */
+int bitnet_hip_bitlinear_forward_multi(bitnet_hip_bitlinear *const *layers, size_t count, const float *x, size_t m,
+                                       const float *gamma, float eps, int sum_order, float *const *outs,
+                                       void *workspace, size_t workspace_bytes, void *stream);
 
 /* The contraction + epilogue of a layer on activations that are already quantised:
  * TernaryProcessor::ternary_matmul (bitnet-inference/src/engine/ternary_operations.rs:87-113) /

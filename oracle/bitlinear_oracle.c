@@ -19,7 +19,7 @@
  *                                        the reference holds no exact-value vector for it
  *   orc_rmsnorm                          the reference holds NO fixture: pinned by closed forms (constant
  *                                        rows, one-hot rows), scale equivariance and an f64 bound; the
- *                                        bits of the ORC_SUM_WAVE64 order are a declaration of this build
+ *                                        bits of the ORC_SUM_BLOCK256 order are a declaration of this build
  *   orc_epilogue                         two IEEE f32 operations; closed form
  *   orc_quantize_weights_reference       PARITY UNPINNED for the f32 statistics: the reference computes
  *                                        mean/sum with candle-core 0.8 (third party, not vendored), whose
@@ -33,7 +33,7 @@
 #include <string.h>
 
 #define ORC_SUM_SEQUENTIAL 0 /* literal order of the reference: one running f32 sum, k ascending   */
-#define ORC_SUM_WAVE64 1     /* declared order the HIP kernel follows: 64 strided partials + butterfly */
+#define ORC_SUM_BLOCK256 1   /* declared order the HIP kernels follow: 256 strided partials, 4 butterflies */
 
 /* ------------------------------------------------------------------------------------------------
  * R1  RMSNorm.   reference: bitnet-inference/src/engine/inference_integration.rs:449-493
@@ -44,11 +44,12 @@
 
 /* Sum of squares of one row in the requested order.
  *
- * ORC_SUM_WAVE64: the row is cut into chunks of 4 consecutive elements; chunk c belongs to lane
- * c mod 64; a lane adds the squares of its chunks in ascending chunk order and, inside a chunk, in
- * ascending element order, starting from +0.  Elements past K count as 0.  The 64 partials are then
- * combined by a butterfly: for off = 32,16,8,4,2,1: p[l] = p[l] + p[l ^ off].  IEEE addition is
- * commutative, so all lanes end with the same value; lane 0's is returned. */
+ * ORC_SUM_BLOCK256: the row is cut into chunks of 4 consecutive elements; chunk c belongs to lane
+ * c mod 256; a lane adds the squares of its chunks in ascending chunk order and, inside a chunk, in
+ * ascending element order, starting from +0.  Elements past K count as 0.  The 256 partials form 4
+ * groups of 64 consecutive lanes; each group is combined by a butterfly: for off = 32,16,8,4,2,1:
+ * p[l] = p[l] + p[l ^ off] (IEEE addition is commutative, so every lane of a group ends with the same
+ * value).  The four group sums are added as ((s0 + s1) + s2) + s3. */
 float orc_sum_squares(const float *x, size_t k, int order)
 {
     if (order == ORC_SUM_SEQUENTIAL) {
@@ -59,11 +60,11 @@ float orc_sum_squares(const float *x, size_t k, int order)
         }
         return s;
     }
-    float p[64], t[64];
-    for (int l = 0; l < 64; ++l) p[l] = 0.0f;
+    float p[256], t[256];
+    for (int l = 0; l < 256; ++l) p[l] = 0.0f;
     size_t chunks = (k + 3) / 4;
     for (size_t c = 0; c < chunks; ++c) {
-        int l = (int)(c % 64);
+        int l = (int)(c % 256);
         for (size_t j = 0; j < 4; ++j) {
             size_t i = 4 * c + j;
             float v = i < k ? x[i] : 0.0f;
@@ -72,10 +73,13 @@ float orc_sum_squares(const float *x, size_t k, int order)
         }
     }
     for (int off = 32; off >= 1; off >>= 1) {
-        for (int l = 0; l < 64; ++l) t[l] = p[l] + p[l ^ off];
+        for (int l = 0; l < 256; ++l) t[l] = p[l] + p[l ^ off]; /* l ^ off stays inside l's group of 64 */
         memcpy(p, t, sizeof p);
     }
-    return p[0];
+    float s = p[0] + p[64];
+    s = s + p[128];
+    s = s + p[192];
+    return s;
 }
 
 void orc_rmsnorm(const float *x, const float *g, float eps, size_t m, size_t k, int order, float *y)

@@ -15,7 +15,7 @@ _DIR = Path(__file__).resolve().parent
 LIB_PATH = _DIR / "libbitnet_oracle.so"
 
 SUM_SEQUENTIAL = 0
-SUM_WAVE64 = 1
+SUM_BLOCK256 = 1
 
 _lib = None
 
@@ -53,12 +53,12 @@ def _sz(v):
     return C.c_size_t(int(v))
 
 
-def sum_squares(x, order=SUM_WAVE64) -> np.float32:
+def sum_squares(x, order=SUM_BLOCK256) -> np.float32:
     x = _f32(x).reshape(-1)
     return np.float32(lib().orc_sum_squares(_p(x), _sz(x.size), C.c_int(order)))
 
 
-def rmsnorm(x, g, eps, order=SUM_WAVE64):
+def rmsnorm(x, g, eps, order=SUM_BLOCK256):
     x = _f32(x)
     g = _f32(g)
     m, k = x.shape
@@ -86,7 +86,7 @@ def fake_quantize_activations(x):
     return out
 
 
-def rmsnorm_quantize_i8(x, g, eps, order=SUM_WAVE64):
+def rmsnorm_quantize_i8(x, g, eps, order=SUM_BLOCK256):
     x = _f32(x)
     g = None if g is None else _f32(g)
     m, k = x.shape
@@ -201,7 +201,7 @@ def epilogue(acc, w_scale, a_scale, bias=None, residual=None):
     return out
 
 
-def bitlinear_forward(x, packed, n_out, w_scale, g=None, eps=1e-5, order=SUM_WAVE64, bias=None, residual=None):
+def bitlinear_forward(x, packed, n_out, w_scale, g=None, eps=1e-5, order=SUM_BLOCK256, bias=None, residual=None):
     """Returns (out f32 [m,n], q int8 [m,k], a_scale f32 [m], acc int32 [m,n])."""
     x = _f32(x)
     m, k = x.shape
@@ -234,7 +234,7 @@ def gqa_broadcast_v(v, q_heads, kv_heads, head_dim):
 
 
 def decoder_layer(x, weights, w_scales, hidden, ffn, q_heads, kv_heads, head_dim, g_attn, g_ffn, eps=1e-5,
-                  order=SUM_WAVE64):
+                  order=SUM_BLOCK256):
     """weights: 7 flat-packed u8 arrays (q,k,v,o,gate,up,down); returns (x_out, q, k)."""
     x = _f32(x)
     m = x.shape[0]

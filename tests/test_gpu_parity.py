@@ -113,19 +113,20 @@ def test_quantize_weights_reference_vectors():
 # ---- R1 + A1 -------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("m,k", [(1, 2560), (4, 2560), (3, 6912), (2, 1024), (5, 4096), (2, 8192), (2, 12000),
-                                 (3, 7), (2, 257), (1, 4), (9, 64)])
+                                 (3, 7), (2, 257), (1, 4), (9, 64), (33, 2560), (40, 6912), (35, 1028), (34, 20000),
+                                 (2, 20000), (3, 16384), (33, 5)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_activation_quant_bit_exact(m, k, norm):
     rng = np.random.default_rng(m * 100003 + k)
     x = synth_activations(rng, m, k, outliers=True)
     g = rng.standard_normal(k, dtype=f32) if norm else None
     q, s, asum, y = bh.quantize_activations_i8(dev(x), dev(g) if norm else None, eps=1e-5, want_sum=True, want_y=norm)
-    q_ref, s_ref, rs_ref = orc.rmsnorm_quantize_i8(x, g, 1e-5, orc.SUM_WAVE64)
+    q_ref, s_ref, rs_ref = orc.rmsnorm_quantize_i8(x, g, 1e-5, orc.SUM_BLOCK256)
     assert np.array_equal(host(s), s_ref)
     assert np.array_equal(host(q), q_ref)
     assert np.array_equal(host(asum), rs_ref)
     if norm:
-        assert np.array_equal(host(y), orc.rmsnorm(x, g, 1e-5, orc.SUM_WAVE64))
+        assert np.array_equal(host(y), orc.rmsnorm(x, g, 1e-5, orc.SUM_BLOCK256))
 
 
 @pytest.mark.parametrize("k", [2560, 300])
@@ -421,6 +422,56 @@ def test_bitlinear_forward_shapes_bias_norm_and_layouts():
     layer_p = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "t_packed")
     layer_p.set_quantized_weights(torch.from_numpy(packed), float(ws))
     assert np.array_equal(host(layer_p.forward(dev(x))), ref0)
+
+
+@pytest.mark.parametrize("m", [1, 3, 8, 20, 200])
+def test_forward_multi_matches_single_forwards(m):
+    """q/k/v-style: several layers on one input give exactly what each layer gives alone, and what the oracle gives."""
+    rng = np.random.default_rng(40 + m)
+    k = 2560
+    ns = [2560, 640, 640, 96]
+    g = (1 + 0.1 * rng.standard_normal(k, dtype=f32)).astype(f32)
+    x = synth_activations(rng, m, k, outliers=True)
+    layers, refs = [], []
+    for i, n in enumerate(ns):
+        w = synth_weights(rng, n, k)
+        layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), f"multi{i}")
+        layer.update_weights(dev(w))
+        layers.append(layer)
+        qw, ws = orc.quantize_weights_absmean(w)
+        refs.append(orc.bitlinear_forward(x, orc.pack_2bit(qw), n, ws, g=g, eps=1e-5)[0])
+    outs = bh.forward_multi(layers, dev(x), gamma=dev(g))
+    for layer, out, ref in zip(layers, outs, refs):
+        assert np.array_equal(host(out), ref)
+        assert np.array_equal(host(layer.forward(dev(x), gamma=dev(g))), ref)
+    other = bh.BitLinear(bh.BitLinearConfig(in_features=k + 4, out_features=8), "other")
+    other.update_weights(torch.ones(8, k + 4))
+    with pytest.raises(bh.BitLinearError) as ei:
+        bh.forward_multi([layers[0], other], dev(x))
+    assert ei.value.kind == "ShapeMismatch"
+
+
+@pytest.mark.parametrize("m", [1, 2, 5, 8])
+def test_bitlinear_forward_decode_debug_outputs(m):
+    """At decode token counts the quantiser runs inside the GEMV launch; its int8 row, scale and the int32
+    accumulators are still observable and bit-exact, with and without RMSNorm, at both FFN widths."""
+    rng = np.random.default_rng(50 + m)
+    for k, n, norm in [(2560, 640, True), (6912, 2560, False), (1024, 48, True)]:
+        w = synth_weights(rng, n, k)
+        x = synth_activations(rng, m, k, outliers=True)
+        g = (1 + 0.1 * rng.standard_normal(k, dtype=f32)).astype(f32) if norm else None
+        layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "dbg")
+        layer.update_weights(dev(w))
+        out, q, a_scale, acc = layer.forward(dev(x), gamma=dev(g) if norm else None, debug=True)
+        qw, ws = orc.quantize_weights_absmean(w)
+        out_ref, q_ref, s_ref, acc_ref = orc.bitlinear_forward(x, orc.pack_2bit(qw), n, ws, g=g, eps=1e-5)
+        assert np.array_equal(host(q), q_ref) and np.array_equal(host(a_scale), s_ref)
+        assert np.array_equal(host(acc), acc_ref) and np.array_equal(host(out), out_ref)
+    # the reference's literal summation order inside the fused launch
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=1024, out_features=48, sum_order=bh.SUM_SEQUENTIAL), "seq")
+    layer.update_weights(dev(w))
+    out_ref = orc.bitlinear_forward(x, orc.pack_2bit(qw), n, ws, g=g, eps=1e-5, order=orc.SUM_SEQUENTIAL)[0]
+    assert np.array_equal(host(layer.forward(dev(x), gamma=dev(g))), out_ref)
 
 
 def test_bitlinear_error_behaviour_matches_reference():

@@ -259,19 +259,19 @@ def test_activation_quant_invariants_and_numpy_model(outliers):
 
 # ---- R1: RMSNorm --------------------------------------------------------------------------------------
 
-def np_wave64_sum_squares(x):
-    """Independent numpy model of the declared 64-lane order (f32 arithmetic step by step)."""
+def np_block256_sum_squares(x):
+    """Independent numpy model of the declared 256-lane order (f32 arithmetic step by step)."""
     x = np.asarray(x, dtype=f32)
     k = x.size
-    pad = (-k) % 256
-    xp = np.concatenate([x, np.zeros(pad, dtype=f32)]).reshape(-1, 64, 4)  # [round, lane, elem]
-    p = np.zeros(64, dtype=f32)
+    pad = (-k) % 1024
+    xp = np.concatenate([x, np.zeros(pad, dtype=f32)]).reshape(-1, 256, 4)  # [round, lane, elem]
+    p = np.zeros(256, dtype=f32)
     for rnd in range(xp.shape[0]):
         for j in range(4):
             p = (p + xp[rnd, :, j] * xp[rnd, :, j]).astype(f32)
     for off in (32, 16, 8, 4, 2, 1):
-        p = (p + p[np.arange(64) ^ off]).astype(f32)
-    return p[0]
+        p = (p + p[np.arange(256) ^ off]).astype(f32)
+    return f32(f32(f32(p[0] + p[64]) + p[128]) + p[192])
 
 
 def np_seq_sum_squares(x):
@@ -281,14 +281,14 @@ def np_seq_sum_squares(x):
     return s
 
 
-@pytest.mark.parametrize("k", [1, 3, 4, 255, 256, 257, 2560, 6912])
+@pytest.mark.parametrize("k", [1, 3, 4, 255, 256, 257, 1023, 1024, 1025, 2560, 6912])
 def test_sum_squares_orders_match_models(k):
     rng = np.random.default_rng(k)
     x = rng.standard_normal(k, dtype=f32)
-    assert orc.sum_squares(x, orc.SUM_WAVE64) == np_wave64_sum_squares(x)
+    assert orc.sum_squares(x, orc.SUM_BLOCK256) == np_block256_sum_squares(x)
     assert orc.sum_squares(x, orc.SUM_SEQUENTIAL) == np_seq_sum_squares(x)
     exact = float((x.astype(np.float64) ** 2).sum())
-    for order in (orc.SUM_WAVE64, orc.SUM_SEQUENTIAL):
+    for order in (orc.SUM_BLOCK256, orc.SUM_SEQUENTIAL):
         assert abs(float(orc.sum_squares(x, order)) - exact) <= 1e-5 * exact
 
 
@@ -298,11 +298,11 @@ def test_sum_squares_order_is_observable():
     differs = 0
     for _ in range(32):
         x = rng.standard_normal(2560, dtype=f32)
-        differs += orc.sum_squares(x, orc.SUM_WAVE64) != orc.sum_squares(x, orc.SUM_SEQUENTIAL)
+        differs += orc.sum_squares(x, orc.SUM_BLOCK256) != orc.sum_squares(x, orc.SUM_SEQUENTIAL)
     assert differs > 0
 
 
-@pytest.mark.parametrize("order", [orc.SUM_SEQUENTIAL, orc.SUM_WAVE64])
+@pytest.mark.parametrize("order", [orc.SUM_SEQUENTIAL, orc.SUM_BLOCK256])
 def test_rmsnorm_closed_forms(order):
     k = 2560
     g = np.ones(k, dtype=f32)
@@ -326,7 +326,7 @@ def test_rmsnorm_closed_forms(order):
     assert np.array_equal(orc.rmsnorm(x, g2, 0.0, order), orc.rmsnorm(x * f32(4.0), g2, 0.0, order))
 
 
-@pytest.mark.parametrize("order", [orc.SUM_SEQUENTIAL, orc.SUM_WAVE64])
+@pytest.mark.parametrize("order", [orc.SUM_SEQUENTIAL, orc.SUM_BLOCK256])
 def test_rmsnorm_f64_bound(order):
     rng = np.random.default_rng(7)
     x = rng.standard_normal((8, 2560), dtype=f32) * f32(3.0)
