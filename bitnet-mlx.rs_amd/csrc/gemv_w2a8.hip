@@ -160,11 +160,13 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
                 if (tid == 0) scale_s[t] = 1.0f;
                 continue;
             }
-            float4 v[FUSED_NCH];
+            float4 v[FUSED_NCH], gm[FUSED_NCH];
 #pragma unroll
             for (int i = 0; i < FUSED_NCH; ++i) {
                 int c = tid + 256 * i;
                 v[i] = c < chunks ? load_chunk<MODE, true>(src, (size_t)t, c) : make_float4(0.f, 0.f, 0.f, 0.f);
+                // the RMSNorm weights are requested together with the row, not after the first reduction
+                gm[i] = (norm && c < chunks) ? load_gamma_chunk(src, c, true) : make_float4(0.f, 0.f, 0.f, 0.f);
             }
             float rms = 1.0f;
             if (norm) {
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
 #pragma unroll
             for (int i = 0; i < FUSED_NCH; ++i) {
                 int c = tid + 256 * i;
-                if (norm && c < chunks) v[i] = normalize4(v[i], rms, load_gamma_chunk(src, c, true));
+                if (norm && c < chunks) v[i] = normalize4(v[i], rms, gm[i]);
                 amax = absmax4(amax, v[i]);
             }
             amax = wave_max_f32(amax);

@@ -1,0 +1,292 @@
+// C++ host-side mirror of the reference's Rust types for the BitLinear path, over the C ABI
+// (include/bitnet_hip.h).  Header only.  Names, fields and error behaviour follow the reference so that
+// call sites translate line by line:
+//
+//   bitnet::BitLinearError            bitnet-quant/src/bitlinear/error.rs:10-84 (variant + message; ShapeMismatch
+//                                     carries expected / actual)
+//   bitnet::BitLinearConfig           bitnet-quant/src/bitlinear/layer.rs:20-75
+//   bitnet::BitLinear                 bitnet-quant/src/bitlinear/layer.rs:82-109,113-179,299-352 and the
+//                                     BitLinearForward trait, bitnet-quant/src/bitlinear/forward.rs:14-51
+//   bitnet::TernaryProcessor          bitnet-inference/src/engine/ternary_operations.rs:56-172
+//   bitnet::BitLinearLayer            bitnet-inference/src/engine/transformer_layers.rs:68-202
+//   bitnet::FeedForwardNetwork        bitnet-inference/src/engine/transformer_layers.rs:553-623
+//
+// Rust returns Result<T, E>; here every fallible call returns a Result<T> holding either the value or the
+// error.  Nothing throws and nothing aborts.  Tensors are dense row-major f32 buffers in device memory
+// (DeviceTensor owns its allocation, like the fresh Tensor the reference's forward returns).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <memory>
+#include <optional>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../include/bitnet_hip.h"
+
+namespace bitnet {
+
+struct BitLinearError {
+    enum Kind { ShapeMismatch = 1, ConfigError, DeviceError, MemoryError, QuantizationError, NotInitialized,
+                KernelError, NullPointer, Unsupported };
+    Kind kind;
+    std::string message;
+    std::vector<size_t> expected, actual;  // ShapeMismatch only
+};
+
+template <class T>
+class Result {
+public:
+    Result(T v) : value_(std::move(v)) {}
+    Result(BitLinearError e) : error_(std::move(e)) {}
+    bool is_ok() const { return value_.has_value(); }
+    bool is_err() const { return !is_ok(); }
+    T &unwrap() { return *value_; }
+    const BitLinearError &unwrap_err() const { return *error_; }
+
+private:
+    std::optional<T> value_;
+    std::optional<BitLinearError> error_;
+};
+struct Unit {};
+
+inline BitLinearError last_error(int status)
+{
+    BitLinearError e{static_cast<BitLinearError::Kind>(status), bitnet_hip_last_error(), {}, {}};
+    if (status == BITNET_HIP_SHAPE_MISMATCH) {
+        size_t ex[4], ac[4];
+        int ar = 0;
+        int er = bitnet_hip_last_shape_mismatch(ex, ac, &ar);
+        e.expected.assign(ex, ex + er);
+        e.actual.assign(ac, ac + ar);
+    }
+    return e;
+}
+
+// Dense f32 tensor in device memory.
+class DeviceTensor {
+public:
+    DeviceTensor() = default;
+    static Result<DeviceTensor> zeros(std::vector<size_t> dims)
+    {
+        DeviceTensor t;
+        t.dims_ = std::move(dims);
+        size_t n = t.elem_count();
+        float *p = nullptr;
+        if (hipMalloc(reinterpret_cast<void **>(&p), (n ? n : 1) * sizeof(float)) != hipSuccess)
+            return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
+        (void)hipMemset(p, 0, n * sizeof(float));
+        t.data_.reset(p, [](float *q) { (void)hipFree(q); });
+        return t;
+    }
+    static Result<DeviceTensor> from_vec(const std::vector<float> &host, std::vector<size_t> dims)
+    {
+        auto r = zeros(std::move(dims));
+        if (r.is_err()) return r;
+        if (r.unwrap().elem_count() != host.size())
+            return BitLinearError{BitLinearError::ShapeMismatch, "from_vec: element count", {r.unwrap().elem_count()}, {host.size()}};
+        (void)hipMemcpy(r.unwrap().data(), host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice);
+        return r;
+    }
+    std::vector<float> to_vec() const
+    {
+        std::vector<float> h(elem_count());
+        (void)hipDeviceSynchronize();
+        (void)hipMemcpy(h.data(), data_.get(), h.size() * sizeof(float), hipMemcpyDeviceToHost);
+        return h;
+    }
+    const std::vector<size_t> &dims() const { return dims_; }
+    size_t elem_count() const
+    {
+        size_t n = 1;
+        for (size_t d : dims_) n *= d;
+        return n;
+    }
+    float *data() const { return data_.get(); }
+
+private:
+    std::vector<size_t> dims_;
+    std::shared_ptr<float> data_;
+};
+
+struct BitLinearConfig {
+    size_t in_features = 512;
+    size_t out_features = 512;
+    bool use_bias = false;  // BitNet standard is bias-free
+    int ternary_method = BITNET_HIP_TERNARY_ABSMEAN_ROUNDCLIP;
+    float threshold_factor = 0.5f;
+    float rms_norm_eps = 1e-5f;
+    int sum_order = BITNET_HIP_SUM_BLOCK256;
+};
+
+class BitLinear {
+public:
+    // BitLinear::new(config, layer_name)
+    static Result<std::shared_ptr<BitLinear>> create(const BitLinearConfig &config, std::string layer_name)
+    {
+        bitnet_hip_bitlinear *h = nullptr;
+        int rc = bitnet_hip_bitlinear_create(config.in_features, config.out_features, config.use_bias, &h);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return std::shared_ptr<BitLinear>(new BitLinear(config, std::move(layer_name), h));
+    }
+    ~BitLinear() { bitnet_hip_bitlinear_destroy(handle_); }
+    BitLinear(const BitLinear &) = delete;
+    BitLinear &operator=(const BitLinear &) = delete;
+
+    const BitLinearConfig &config() const { return config_; }
+    const std::string &layer_name() const { return layer_name_; }
+    bitnet_hip_bitlinear *handle() const { return handle_; }
+
+    // update_weights: latent f32 [out_features, in_features] in host memory
+    Result<Unit> update_weights(const std::vector<float> &w, size_t rows, size_t cols)
+    {
+        int rc = bitnet_hip_bitlinear_set_weights_f32(handle_, w.data(), rows, cols, BITNET_HIP_LAYOUT_OUT_IN, 0,
+                                                      config_.ternary_method, config_.threshold_factor, nullptr);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return Unit{};
+    }
+    Result<Unit> update_bias(const std::vector<float> &b)
+    {
+        int rc = bitnet_hip_bitlinear_set_bias(handle_, b.data(), b.size(), 0, nullptr);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return Unit{};
+    }
+    // BitLinearForward::forward: [.., in_features] -> [.., out_features]
+    Result<DeviceTensor> forward(const DeviceTensor &input, const float *gamma = nullptr, hipStream_t stream = nullptr) const
+    {
+        std::vector<size_t> out_dims = input.dims();
+        if (!out_dims.empty()) out_dims.back() = config_.out_features;
+        auto out = DeviceTensor::zeros(out_dims.empty() ? std::vector<size_t>{config_.out_features} : out_dims);
+        if (out.is_err()) return out;
+        int rc = bitnet_hip_bitlinear_forward(handle_, input.data(), input.dims().data(), (int)input.dims().size(), gamma,
+                                              config_.rms_norm_eps, config_.sum_order, nullptr, out.unwrap().data(),
+                                              nullptr, 0, nullptr, nullptr, nullptr, stream);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return out;
+    }
+    Result<DeviceTensor> forward_batch(const DeviceTensor &inputs) const
+    {
+        if (inputs.dims().size() < 2)
+            return BitLinearError{BitLinearError::ShapeMismatch, "forward_batch needs at least 2 dimensions",
+                                  {1, 1, config_.in_features}, inputs.dims()};
+        return forward(inputs);
+    }
+
+private:
+    BitLinear(BitLinearConfig c, std::string n, bitnet_hip_bitlinear *h) : config_(c), layer_name_(std::move(n)), handle_(h) {}
+    BitLinearConfig config_;
+    std::string layer_name_;
+    bitnet_hip_bitlinear *handle_;
+};
+
+// TernaryProcessor: per-token int8 absmax quantisation and the ternary matmul on top of it.
+struct QuantizedActivations {
+    int8_t *values = nullptr;   // [m, k] device
+    float *scales = nullptr;    // [m] device (127 / absmax)
+    int32_t *row_sums = nullptr;
+    size_t m = 0, k = 0;
+    ~QuantizedActivations()
+    {
+        if (values) (void)hipFree(values);
+        if (scales) (void)hipFree(scales);
+        if (row_sums) (void)hipFree(row_sums);
+    }
+};
+
+class TernaryProcessor {
+public:
+    // quantize_activations: input [m, k] (rank 1 is one token)
+    Result<std::shared_ptr<QuantizedActivations>> quantize_activations(const DeviceTensor &input, hipStream_t stream = nullptr)
+    {
+        auto q = std::make_shared<QuantizedActivations>();
+        q->k = input.dims().empty() ? 0 : input.dims().back();
+        q->m = q->k ? input.elem_count() / q->k : 0;
+        if (hipMalloc(reinterpret_cast<void **>(&q->values), q->m * q->k + 1) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&q->scales), (q->m + 1) * sizeof(float)) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&q->row_sums), (q->m + 1) * sizeof(int32_t)) != hipSuccess)
+            return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
+        int rc = bitnet_hip_quantize_activations_i8(input.data(), nullptr, q->k, q->m, q->k, BITNET_HIP_INPUT_PLAIN, 1, 1,
+                                                    nullptr, 0.0f, BITNET_HIP_SUM_BLOCK256, q->values, q->scales,
+                                                    q->row_sums, nullptr, stream);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        ++activations_quantized;
+        return q;
+    }
+    // ternary_matmul(weights, input, output): output [m, out] = input [m, in] through the layer's ternary weights
+    Result<Unit> ternary_matmul(const BitLinear &weights, const DeviceTensor &input, DeviceTensor &output, hipStream_t stream = nullptr)
+    {
+        const size_t in = weights.config().in_features, outf = weights.config().out_features;
+        if (input.dims().size() != 2 || input.dims()[1] != in)
+            return BitLinearError{BitLinearError::ShapeMismatch, "ternary_matmul input", {input.dims().empty() ? 1 : input.dims()[0], in}, input.dims()};
+        if (output.dims().size() != 2 || output.dims()[0] != input.dims()[0] || output.dims()[1] != outf)
+            return BitLinearError{BitLinearError::ShapeMismatch, "ternary_matmul output", {input.dims()[0], outf}, output.dims()};
+        auto q = quantize_activations(input, stream);
+        if (q.is_err()) return q.unwrap_err();
+        int rc = bitnet_hip_bitlinear_matmul(weights.handle(), q.unwrap()->values, q.unwrap()->row_sums, q.unwrap()->m,
+                                             q.unwrap()->scales, nullptr, nullptr, output.data(), stream);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        (void)hipStreamSynchronize(stream);  // the quantised activations are released on return
+        ++ternary_multiplications;
+        return Unit{};
+    }
+    uint64_t ternary_multiplications = 0, activations_quantized = 0;  // TernaryStats
+};
+
+// BitLinearLayer::forward handles rank 2 and rank 3 inputs (transformer_layers.rs:119-201).
+class BitLinearLayer {
+public:
+    static Result<std::shared_ptr<BitLinearLayer>> create(size_t in_features, size_t out_features, bool use_bias, std::string name)
+    {
+        BitLinearConfig c;
+        c.in_features = in_features; c.out_features = out_features; c.use_bias = use_bias;
+        auto l = BitLinear::create(c, std::move(name));
+        if (l.is_err()) return l.unwrap_err();
+        auto p = std::shared_ptr<BitLinearLayer>(new BitLinearLayer());
+        p->in_features = in_features; p->out_features = out_features; p->layer = l.unwrap();
+        return p;
+    }
+    Result<DeviceTensor> forward(const DeviceTensor &input) const { return layer->forward(input); }
+    size_t in_features = 0, out_features = 0;
+    std::shared_ptr<BitLinear> layer;
+};
+
+// FeedForwardNetwork::forward: down( up(x) * relu(gate(x))^2 ) (transformer_layers.rs:603-623).  gate and up
+// share one activation quantisation; the ReLU^2 gating is fused into the quantiser in front of down.
+class FeedForwardNetwork {
+public:
+    std::shared_ptr<BitLinear> up_proj, gate_proj, down_proj;
+    Result<DeviceTensor> forward(const DeviceTensor &input, hipStream_t stream = nullptr) const
+    {
+        const size_t hidden = up_proj->config().in_features, ffn = up_proj->config().out_features;
+        if (input.dims().size() != 2 || input.dims()[1] != hidden)
+            return BitLinearError{BitLinearError::ShapeMismatch, "ffn input", {1, hidden}, input.dims()};
+        const size_t m = input.dims()[0];
+        auto gate = DeviceTensor::zeros({m, ffn}), up = DeviceTensor::zeros({m, ffn}), out = DeviceTensor::zeros({m, hidden});
+        if (gate.is_err() || up.is_err() || out.is_err()) return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
+        bitnet_hip_bitlinear *layers[2] = {gate_proj->handle(), up_proj->handle()};
+        float *outs[2] = {gate.unwrap().data(), up.unwrap().data()};
+        int rc = bitnet_hip_bitlinear_forward_multi(layers, 2, input.data(), m, nullptr, 0.0f, BITNET_HIP_SUM_BLOCK256, outs,
+                                                    nullptr, 0, stream);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        TernaryProcessor tp;
+        QuantizedActivations q;
+        q.m = m; q.k = ffn;
+        if (hipMalloc(reinterpret_cast<void **>(&q.values), m * ffn) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&q.scales), m * sizeof(float)) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&q.row_sums), m * sizeof(int32_t)) != hipSuccess)
+            return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
+        rc = bitnet_hip_quantize_activations_i8(gate.unwrap().data(), up.unwrap().data(), ffn, m, ffn, BITNET_HIP_INPUT_RELU2_MUL,
+                                                1, 1, nullptr, 0.0f, BITNET_HIP_SUM_BLOCK256, q.values, q.scales, q.row_sums,
+                                                nullptr, stream);
+        if (rc == BITNET_HIP_OK)
+            rc = bitnet_hip_bitlinear_matmul(down_proj->handle(), q.values, q.row_sums, m, q.scales, nullptr, nullptr,
+                                             out.unwrap().data(), stream);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        (void)hipStreamSynchronize(stream);
+        return out;
+    }
+};
+
+}  // namespace bitnet

@@ -1,0 +1,103 @@
+//! Raw `extern "C"` declarations of include/bitnet_hip.h, one per exported symbol, same order.
+//! Device pointers are plain raw pointers owned by the caller; `stream` is a `hipStream_t`.
+#![allow(non_camel_case_types)]
+use std::os::raw::{c_char, c_int, c_void};
+
+#[repr(C)]
+pub struct bitnet_hip_bitlinear {
+    _private: [u8; 0],
+}
+#[repr(C)]
+pub struct bitnet_hip_decoder {
+    _private: [u8; 0],
+}
+
+pub const BITNET_HIP_OK: c_int = 0;
+pub const BITNET_HIP_SHAPE_MISMATCH: c_int = 1;
+pub const BITNET_HIP_INVALID_CONFIG: c_int = 2;
+pub const BITNET_HIP_DEVICE_ERROR: c_int = 3;
+pub const BITNET_HIP_MEMORY_ERROR: c_int = 4;
+pub const BITNET_HIP_QUANTIZATION_ERROR: c_int = 5;
+pub const BITNET_HIP_NOT_INITIALIZED: c_int = 6;
+pub const BITNET_HIP_KERNEL_ERROR: c_int = 7;
+pub const BITNET_HIP_NULL_POINTER: c_int = 8;
+pub const BITNET_HIP_UNSUPPORTED: c_int = 9;
+
+pub const BITNET_HIP_SUM_SEQUENTIAL: c_int = 0;
+pub const BITNET_HIP_SUM_BLOCK256: c_int = 1;
+pub const BITNET_HIP_LAYOUT_OUT_IN: c_int = 0;
+pub const BITNET_HIP_LAYOUT_IN_OUT: c_int = 1;
+pub const BITNET_HIP_TERNARY_ABSMEAN_ROUNDCLIP: c_int = 0;
+pub const BITNET_HIP_TERNARY_MEAN_THRESHOLD: c_int = 1;
+pub const BITNET_HIP_INPUT_PLAIN: c_int = 0;
+pub const BITNET_HIP_INPUT_RELU2_MUL: c_int = 1;
+pub const BITNET_HIP_INPUT_GQA_BROADCAST: c_int = 2;
+
+extern "C" {
+    pub fn bitnet_hip_last_error() -> *const c_char;
+    pub fn bitnet_hip_last_shape_mismatch(expected: *mut usize, actual: *mut usize, actual_rank: *mut c_int) -> c_int;
+    pub fn bitnet_hip_init(device: c_int) -> c_int;
+    pub fn bitnet_hip_device_info(arch_name: *mut c_char, arch_name_len: usize, compute_units: *mut c_int,
+                                  clock_mhz: *mut c_int, total_mem_bytes: *mut usize) -> c_int;
+    pub fn bitnet_hip_quantize_activations_i8(x: *const f32, x2: *const f32, ldx: usize, m: usize, k: usize,
+                                              input_mode: c_int, gqa_group: usize, head_dim: usize, gamma: *const f32,
+                                              eps: f32, sum_order: c_int, q: *mut i8, a_scale: *mut f32,
+                                              a_sum: *mut i32, y_f32: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_packed_size(count: usize) -> usize;
+    pub fn bitnet_hip_pack_ternary_2bit(q: *const i8, count: usize, packed: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_unpack_ternary_2bit(packed: *const u8, count: usize, q: *mut i8, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_quantize_weights(w: *const f32, n: usize, k: usize, method: c_int, threshold_factor: f32,
+                                       packed: *mut u8, w_scale: *mut f32, q_i8: *mut i8, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_tiled_size(n: usize, k: usize) -> usize;
+    pub fn bitnet_hip_retile_weights(packed: *const u8, n: usize, k: usize, layout: c_int, tiled: *mut u8,
+                                     stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_untile_weights(tiled: *const u8, n: usize, k: usize, packed: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_gemv_w2a8(weights: *const u8, activations: *const i8, output: *mut i32, m: usize, k: usize,
+                                stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_gemv_w2a8_checked(weights: *const u8, weights_len: usize, activations: *const i8,
+                                        activations_len: usize, output: *mut i32, output_len: usize, m: usize,
+                                        k: usize, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_matmul_w2a8(tiled: *const u8, a: *const i8, a_sum: *const i32, m: usize, n: usize, k: usize,
+                                  acc: *mut i32, w_scale: *const f32, a_scale: *const f32, bias: *const f32,
+                                  residual: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_bitlinear_create(in_features: usize, out_features: usize, use_bias: c_int,
+                                       layer: *mut *mut bitnet_hip_bitlinear) -> c_int;
+    pub fn bitnet_hip_bitlinear_destroy(layer: *mut bitnet_hip_bitlinear);
+    pub fn bitnet_hip_bitlinear_set_weights_f32(layer: *mut bitnet_hip_bitlinear, w: *const f32, rows: usize,
+                                                cols: usize, layout: c_int, on_device: c_int, method: c_int,
+                                                threshold_factor: f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_bitlinear_set_weights_packed(layer: *mut bitnet_hip_bitlinear, packed: *const u8,
+                                                   packed_len: usize, w_scale: f32, on_device: c_int,
+                                                   stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_bitlinear_set_bias(layer: *mut bitnet_hip_bitlinear, bias: *const f32, len: usize,
+                                         on_device: c_int, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_bitlinear_get_quantized(layer: *mut bitnet_hip_bitlinear, w_scale: *mut f32, packed: *mut u8,
+                                              packed_len: usize) -> c_int;
+    pub fn bitnet_hip_bitlinear_workspace_size(layer: *const bitnet_hip_bitlinear, m: usize) -> usize;
+    pub fn bitnet_hip_bitlinear_forward(layer: *mut bitnet_hip_bitlinear, x: *const f32, dims: *const usize,
+                                        rank: c_int, gamma: *const f32, eps: f32, sum_order: c_int,
+                                        residual: *const f32, out: *mut f32, workspace: *mut c_void,
+                                        workspace_bytes: usize, dbg_q: *mut i8, dbg_a_scale: *mut f32,
+                                        dbg_acc: *mut i32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_bitlinear_forward_multi(layers: *const *mut bitnet_hip_bitlinear, count: usize, x: *const f32,
+                                              m: usize, gamma: *const f32, eps: f32, sum_order: c_int,
+                                              outs: *const *mut f32, workspace: *mut c_void, workspace_bytes: usize,
+                                              stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_bitlinear_matmul(layer: *mut bitnet_hip_bitlinear, a: *const i8, a_sum: *const i32, m: usize,
+                                       a_scale: *const f32, residual: *const f32, acc: *mut i32, out: *mut f32,
+                                       stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_decoder_create(layers: usize, hidden: usize, ffn: usize, q_heads: usize, kv_heads: usize,
+                                     head_dim: usize, eps: f32, sum_order: c_int, max_tokens: usize,
+                                     dec: *mut *mut bitnet_hip_decoder) -> c_int;
+    pub fn bitnet_hip_decoder_destroy(dec: *mut bitnet_hip_decoder);
+    pub fn bitnet_hip_decoder_projection(dec: *mut bitnet_hip_decoder, layer: usize, proj: c_int,
+                                         out: *mut *mut bitnet_hip_bitlinear) -> c_int;
+    pub fn bitnet_hip_decoder_set_norm(dec: *mut bitnet_hip_decoder, layer: usize, which: c_int, gamma: *const f32,
+                                       on_device: c_int, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_decoder_weight_bytes(dec: *const bitnet_hip_decoder) -> usize;
+    pub fn bitnet_hip_decoder_decode(dec: *mut bitnet_hip_decoder, x_in: *const f32, m: usize, x_out: *mut f32,
+                                     q_last: *mut f32, k_last: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_decoder_decode_layers(dec: *mut bitnet_hip_decoder, layer_begin: usize, layer_end: usize,
+                                            x_in: *const f32, m: usize, x_out: *mut f32, q_last: *mut f32,
+                                            k_last: *mut f32, stream: *mut c_void) -> c_int;
+}

@@ -555,3 +555,18 @@ def test_decoder_stack_small_bit_exact(layers):
     with pytest.raises(bh.BitLinearError) as ei:
         dec.decode(dev(synth_activations(rng, 5, 256)))
     assert ei.value.kind == "ShapeMismatch"
+
+
+# ---- C++ host mirror -----------------------------------------------------------------------------------------
+
+def test_cpp_host_mirror_selftest():
+    """bitnet-mlx.rs_amd/host/bitlinear.hpp (the C++ stand-in for the Rust types) against the reference's own
+    BitLinear forward tests and against the other routes through the library."""
+    import subprocess
+    from pathlib import Path
+
+    exe = Path(bh.LIB_PATH).parents[1] / "bin" / "host_selftest"
+    assert exe.exists(), "build first: make -C bitnet-mlx.rs_amd"
+    proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "all passed" in proc.stdout
