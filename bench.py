@@ -10,10 +10,13 @@ epilogue.  Consecutive steps use the weights of consecutive layers of a 30-layer
 weights in total), so no step finds its weights in cache.  Inputs and weights are resident in HBM before
 the timed region.  value = packed-weight bytes streamed per second over the whole timed region.
 
-The line also carries: the roofline of the dominant kernel (the decode GEMV) from HIP-event timing of
-GEMV-only launches over the same 210 weight matrices; the prefill GEMM rate (M = 2048) at the two FFN
-shapes; and a CPU baseline (a C restatement of the reference's dequantise-to-f32 BitLinear forward)
-timed on this host's cores for a bounded sample.
+The timed region contains one kernel family only, the decode GEMV with the activation quantiser fused into
+its prologue (four launches per step: q+k+v, o, gate+up, down), so the roofline of the dominant kernel comes
+straight from the HIP events around the timed region: achieved = packed-weight bytes per launch / average
+launch duration.  The line also carries the GEMV alone on pre-quantised activations (graph replays over the
+same 210 matrices), the prefill GEMM rate (M = 2048) at the two FFN shapes, and a CPU baseline (a C
+restatement of the reference's dequantise-to-f32 BitLinear forward) timed on this host's cores for a bounded
+sample.
 """
 import argparse
 import json
@@ -55,9 +58,32 @@ def time_events(torch, fn):
     return start.elapsed_time(stop)
 
 
-def gemv_roofline(bh, torch, dec, gen, reps):
-    """GEMV-only launches over all 210 matrices, captured in a HIP graph so that host launch cost does not
-    starve the GPU; HIP events around the replays."""
+LAUNCHES_PER_STEP = 4  # q+k+v | o | gate+up | down, each one gemv_tiled_kernel<1, MODE> launch
+# HBM bytes per launch of that kernel from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (two runs of this
+# script with --no-extras --calibration-copy), each scaled by what the same counter reads for the plain
+# 256 MiB copy: FETCH_SIZE reads 0.5 KiB per KiB fetched (factor 2.0), WRITE_SIZE 1.0 (factor 1.0).
+# Summary: profiles/decode_layer_b1_gemv_hbm_traffic.md
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_778_957
+
+
+def decode_roofline(event_ms, steps):
+    launches = steps * LAUNCHES_PER_STEP
+    total_bytes = steps * LAYER_BYTES
+    achieved = total_bytes / (event_ms * 1e-3) / 1e9
+    return {
+        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
+        "kernel": "gemv_tiled_kernel<1, MODE> (decode GEMV, activation quantiser in the prologue)",
+        "launches": launches, "avg_launch_us": round(event_ms * 1e3 / launches, 3),
+        "bytes_per_launch": LAYER_BYTES // LAUNCHES_PER_STEP,
+        "how": "HIP events on the launch stream around the timed region, which holds only this kernel "
+               "(4 launches per step, back to back); algorithmic bytes = packed weights n*k/4",
+    }
+
+
+def gemv_only(bh, torch, dec, gen, reps):
+    """The GEMV alone on pre-quantised int8 activations: one launch per projection over all 210 matrices,
+    captured in a HIP graph so that host launch cost does not starve the GPU; HIP events around the replays."""
     a = {k: torch.randint(-127, 128, (1, k), generator=gen, device="cuda", dtype=torch.int8) for k in (HIDDEN, FFN)}
     a_scale = torch.ones((1,), device="cuda", dtype=torch.float32)
     outs = {n: torch.empty((1, n), device="cuda", dtype=torch.float32) for n in (HIDDEN, KV_HEADS * HEAD_DIM, FFN)}
@@ -79,15 +105,8 @@ def gemv_roofline(bh, torch, dec, gen, reps):
         ms = time_events(torch, lambda: [graph.replay() for _ in range(reps)])
     launches = reps * len(projs)
     total_bytes = reps * dec.weight_bytes()
-    avg_us = ms * 1e3 / launches
-    achieved = total_bytes / (ms * 1e-3) / 1e9
-    return {
-        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-        "kernel": "gemv_tiled_kernel<1>", "launches": launches, "avg_launch_us": round(avg_us, 3),
-        "bytes_per_launch": round(total_bytes / launches),
-        "how": "HIP events around graph replays of GEMV-only launches over 210 distinct weight matrices (521 MB)",
-    }
+    return {"kernel": "gemv_tiled_kernel<1, -1>", "launches": launches, "avg_launch_us": round(ms * 1e3 / launches, 3),
+            "bytes_per_launch": round(total_bytes / launches), "gbs": round(total_bytes / (ms * 1e-3) / 1e9, 1)}
 
 
 def prefill_rates(bh, torch, dec, gen, reps):
@@ -154,6 +173,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=60)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip roofline / prefill / CPU legs (profiling runs)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the one-GPU BitLinear path; --gpus must be 1 (nothing here uses a second GPU)",
@@ -171,6 +193,13 @@ def main():
     def step(i):
         l = i % LAYERS
         dec.decode(x, out=x, layers=(l, l + 1))
+
+    if args.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for i in range(args.warmup):
         step(i)
@@ -196,8 +225,9 @@ def main():
                    "bytes_per_step": LAYER_BYTES, "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
                    "event_ms_per_step": round(event_ms / args.steps, 5), "device": bh.device_info()},
     }
+    line["roofline"] = decode_roofline(event_ms, args.steps)
     if not args.no_extras:
-        line["roofline"] = gemv_roofline(bh, torch, dec, gen, reps=5)
+        line["gemv_only"] = gemv_only(bh, torch, dec, gen, reps=5)
         line["prefill"] = prefill_rates(bh, torch, dec, gen, reps=5)
         if not args.no_cpu_baseline:
             line["cpu_baseline"] = cpu_baseline(torch, dec)
