@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void act_quant_wave_kernel(ActQuantParams p)
         else return c < chunks ? load_chunk<MODE, VEC>(src, row, c) : zero4;
     };
 
-    float rms = 1.0f;
+    RowDivisor rdiv = {1.0f, 1.0f, false};
     const bool norm = src.gamma != nullptr;
     if (norm) {
         float ss;
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256) void act_quant_wave_kernel(ActQuantParams p)
             ss = f32_add(f32_add(f32_add(wave_sum_f32(part[0]), wave_sum_f32(part[1])), wave_sum_f32(part[2])),
                          wave_sum_f32(part[3]));
         }
-        rms = rms_from_ss(ss, k, src.eps);
+        rdiv = make_row_divisor(rms_from_ss(ss, k, src.eps));
     }
 
     float amax = 0.0f;
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void act_quant_wave_kernel(ActQuantParams p)
     for (int i = 0; i < nloop; ++i) {
         int c = lane + 64 * i;
         float4 e = chunk_at(i, c);
-        if (norm && c < chunks) e = normalize4(e, rms, load_gamma_chunk(src, c, VEC));
+        if (norm && c < chunks) e = normalize4(e, rdiv, load_gamma_chunk(src, c, VEC));
         if constexpr (NCH > 0) v[i] = e;
         amax = absmax4(amax, e);
     }
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void act_quant_wave_kernel(ActQuantParams p)
             e = v[i];
         } else {
             e = load_chunk<MODE, VEC>(src, row, c);
-            if (norm) e = normalize4(e, rms, load_gamma_chunk(src, c, VEC));
+            if (norm) e = normalize4(e, rdiv, load_gamma_chunk(src, c, VEC));
         }
         size_t base = row * (size_t)k + 4 * (size_t)c;
         if constexpr (VEC) {
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void act_quant_block_kernel(ActQuantParams p)
         else return c < chunks ? load_chunk<MODE, VEC>(src, row, c) : zero4;
     };
 
-    float rms = 1.0f;
+    RowDivisor rdiv = {1.0f, 1.0f, false};
     const bool norm = src.gamma != nullptr;
     if (norm) {
         float ss;
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256) void act_quant_block_kernel(ActQuantParams p)
             __syncthreads();
             ss = f32_add(f32_add(f32_add(red_f[0][0], red_f[0][1]), red_f[0][2]), red_f[0][3]);
         }
-        rms = rms_from_ss(ss, k, src.eps);
+        rdiv = make_row_divisor(rms_from_ss(ss, k, src.eps));
     }
 
     float amax = 0.0f;
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void act_quant_block_kernel(ActQuantParams p)
     for (int i = 0; i < nloop; ++i) {
         int c = tid + 256 * i;
         float4 e = chunk_at(i, c);
-        if (norm && c < chunks) e = normalize4(e, rms, load_gamma_chunk(src, c, VEC));
+        if (norm && c < chunks) e = normalize4(e, rdiv, load_gamma_chunk(src, c, VEC));
         if constexpr (NCH > 0) v[i] = e;
         amax = absmax4(amax, e);
     }
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(256) void act_quant_block_kernel(ActQuantParams p)
             e = v[i];
         } else {
             e = load_chunk<MODE, VEC>(src, row, c);
-            if (norm) e = normalize4(e, rms, load_gamma_chunk(src, c, VEC));
+            if (norm) e = normalize4(e, rdiv, load_gamma_chunk(src, c, VEC));
         }
         size_t base = row * (size_t)k + 4 * (size_t)c;
         if constexpr (VEC) {

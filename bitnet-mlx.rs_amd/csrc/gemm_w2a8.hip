@@ -54,18 +54,6 @@ struct GemmParams {
     int tiles_m, tiles_n;
 };
 
-// x / d for a divisor that is the same for a whole output row.  recip must be the correctly rounded 1/d.
-// q0 = RN(x*recip) is within one ulp of x/d; the remainder x - d*q0 is then exact in one FMA and the
-// corrected quotient RN(q0 + rem*recip) is the correctly rounded x/d (Markstein's division step; the only
-// exception, a divisor whose significand is all ones, cannot flip more than the last bit).  Three
-// operations per element instead of the full IEEE division sequence, with the same result.
-__device__ __forceinline__ float div_by_row_invariant(float x, float d, float recip)
-{
-    const float q0 = x * recip;
-    const float rem = __builtin_fmaf(-q0, d, x);
-    return __builtin_fmaf(rem, recip, q0);
-}
-
 constexpr int STAGE_K = 256;              // columns per pipeline stage = one weight tile
 constexpr int LDS_PITCH = STAGE_K + 16;   // bytes per activation row in LDS
 
@@ -215,6 +203,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p)
 
     // ---- epilogue ----
     const float ws = p.out ? *p.w_scale : 0.0f;
+    const unsigned ws_expo = (__builtin_bit_cast(unsigned, ws) >> 23) & 0xffu;
+    const bool ws_fast = ws > 0.0f && ws_expo > 64u && ws_expo < 160u;
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
 #pragma unroll
@@ -225,6 +215,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p)
             const int rs = lds_rowsum[lrow];
             const float as = p.out ? p.a_scale[row] : 1.0f;
             const float as_recip = f32_div(1.0f, as);
+            // the short division needs a well-behaved divisor (per row) and dividends in range: float(total) * ws
+            // is zero or has ws's exponent plus at most 24, so one check on ws covers them.  The choice is made
+            // per wavefront so that the usual case runs no plain division at all.
+            const bool row_fast = ws_fast && invariant_divisor_ok(as);
+            const bool wave_fast = __builtin_amdgcn_ballot_w64(!row_fast) == 0;
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 const int col = n0 + wn * WTN + j * 16 + lr;
@@ -233,7 +228,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p)
                 const size_t o = (size_t)row * p.n + col;
                 if (p.acc) p.acc[o] = total;
                 if (p.out) {
-                    float v = div_by_row_invariant(f32_mul((float)total, ws), as, as_recip);
+                    const float scaled = f32_mul((float)total, ws);
+                    float v = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
                     if (p.bias) v = f32_add(v, p.bias[col]);
                     if (p.residual) v = f32_add(v, p.residual[o]);
                     p.out[o] = v;
@@ -385,6 +381,8 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_kernel(GemmParams p)
     }
 
     const float ws = p.out ? *p.w_scale : 0.0f;
+    const unsigned ws_expo = (__builtin_bit_cast(unsigned, ws) >> 23) & 0xffu;
+    const bool ws_fast = ws > 0.0f && ws_expo > 64u && ws_expo < 160u;
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
 #pragma unroll
@@ -394,6 +392,11 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_kernel(GemmParams p)
             const int rs = p.a_sum[row];
             const float as = p.out ? p.a_scale[row] : 1.0f;
             const float as_recip = f32_div(1.0f, as);
+            // the short division needs a well-behaved divisor (per row) and dividends in range: float(total) * ws
+            // is zero or has ws's exponent plus at most 24, so one check on ws covers them.  The choice is made
+            // per wavefront so that the usual case runs no plain division at all.
+            const bool row_fast = ws_fast && invariant_divisor_ok(as);
+            const bool wave_fast = __builtin_amdgcn_ballot_w64(!row_fast) == 0;
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 const int col = n0 + wn * WTN + j * 16 + lr;
@@ -402,7 +405,8 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_kernel(GemmParams p)
                 const size_t o = (size_t)row * p.n + col;
                 if (p.acc) p.acc[o] = total;
                 if (p.out) {
-                    float v = div_by_row_invariant(f32_mul((float)total, ws), as, as_recip);
+                    const float scaled = f32_mul((float)total, ws);
+                    float v = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
                     if (p.bias) v = f32_add(v, p.bias[col]);
                     if (p.residual) v = f32_add(v, p.residual[o]);
                     p.out[o] = v;

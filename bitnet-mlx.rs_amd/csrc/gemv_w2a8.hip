@@ -108,7 +108,20 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
     const int rb = (int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0);
     const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + (size_t)rb * p.kt_count * 64;
 
-    // Request the first batch of weight tiles before anything else.
+    // Loads retire in issue order, so what the prologue waits for first is requested first: the f32 input row
+    // of token 0 and the RMSNorm weights (L2 hits), then the first batch of weight tiles (HBM), whose latency
+    // the quantiser prologue then hides.
+    float4 v0[MODE == MODE_PREQUANT ? 1 : FUSED_NCH], gm[MODE == MODE_PREQUANT ? 1 : FUSED_NCH];
+    if constexpr (MODE != MODE_PREQUANT) {
+        const int chunks = p.k >> 2;
+        const bool norm = p.src.gamma != nullptr;
+#pragma unroll
+        for (int i = 0; i < FUSED_NCH; ++i) {
+            int c = tid + 256 * i;
+            v0[i] = c < chunks ? load_chunk<MODE, true>(p.src, 0, c) : make_float4(0.f, 0.f, 0.f, 0.f);
+            gm[i] = (norm && c < chunks) ? load_gamma_chunk(p.src, c, true) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
     uint4 wbuf[GEMV_PREFETCH];
 #pragma unroll
     for (int u = 0; u < GEMV_PREFETCH; ++u) {
@@ -160,15 +173,14 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
                 if (tid == 0) scale_s[t] = 1.0f;
                 continue;
             }
-            float4 v[FUSED_NCH], gm[FUSED_NCH];
+            float4 v[FUSED_NCH];
 #pragma unroll
             for (int i = 0; i < FUSED_NCH; ++i) {
                 int c = tid + 256 * i;
-                v[i] = c < chunks ? load_chunk<MODE, true>(src, (size_t)t, c) : make_float4(0.f, 0.f, 0.f, 0.f);
-                // the RMSNorm weights are requested together with the row, not after the first reduction
-                gm[i] = (norm && c < chunks) ? load_gamma_chunk(src, c, true) : make_float4(0.f, 0.f, 0.f, 0.f);
+                if (t == 0) v[i] = v0[i];
+                else v[i] = c < chunks ? load_chunk<MODE, true>(src, (size_t)t, c) : make_float4(0.f, 0.f, 0.f, 0.f);
             }
-            float rms = 1.0f;
+            RowDivisor rdiv = {1.0f, 1.0f, false};
             if (norm) {
                 float ss;
                 if (src.sum_order == BITNET_HIP_SUM_SEQUENTIAL) {
@@ -182,13 +194,13 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
                     __syncthreads();
                     ss = f32_add(f32_add(f32_add(red_f[t][0][0], red_f[t][0][1]), red_f[t][0][2]), red_f[t][0][3]);
                 }
-                rms = rms_from_ss(ss, p.k, src.eps);
+                rdiv = make_row_divisor(rms_from_ss(ss, p.k, src.eps));
             }
             float amax = 0.0f;
 #pragma unroll
             for (int i = 0; i < FUSED_NCH; ++i) {
                 int c = tid + 256 * i;
-                if (norm && c < chunks) v[i] = normalize4(v[i], rms, gm[i]);
+                if (norm && c < chunks) v[i] = normalize4(v[i], rdiv, gm[i]);
                 amax = absmax4(amax, v[i]);
             }
             amax = wave_max_f32(amax);

@@ -14,7 +14,10 @@
 //   the row is cut into chunks of 4 consecutive elements; chunk c belongs to virtual lane c mod 256; a lane
 //   adds the squares of its chunks in ascending chunk order and, inside a chunk, ascending element order,
 //   starting from +0; the 256 partials form 4 groups of 64 consecutive lanes, each combined by the butterfly
-//   p[l] += p[l ^ off], off = 32,16,8,4,2,1; the four group sums are added as ((s0 + s1) + s2) + s3.
+//   p[l] += p[l ^ off], off = 1,2,4,8,16,32; the four group sums are added as ((s0 + s1) + s2) + s3.
+//   (After the step with offset `off` all lanes of an aligned group of 2*off lanes hold the same value, so a
+//   step may fetch its operand from ANY lane of the partner group: the kernels use DPP quad permutes and row
+//   mirrors for offsets 1..8, a swizzle for 16 and a shuffle for 32.)
 //   A 256-thread workgroup maps thread = virtual lane; a single wavefront keeps 4 partials per lane
 //   (virtual lanes l, l+64, l+128, l+192).  Elements past K count as 0.
 // BITNET_HIP_SUM_SEQUENTIAL is the reference's literal running sum over k ascending.
@@ -36,26 +39,33 @@ struct RowSource {
     float eps;
 };
 
-__device__ __forceinline__ float wave_sum_f32(float p)
+// Lane exchanges of the butterfly.  CTRL is a DPP control word: 0xB1 = quad_perm[1,0,3,2] (l ^ 1),
+// 0x4E = quad_perm[2,3,0,1] (l ^ 2), 0x141 = row_half_mirror (a lane of the other quad of the same 8),
+// 0x140 = row_mirror (a lane of the other half of the same 16).
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v)
 {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) p = f32_add(p, __shfl_xor(p, off, 64));
-    return p;
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
 }
+__device__ __forceinline__ int xchg16_i32(int v) { return __builtin_amdgcn_ds_swizzle(v, (0x10 << 10) | 0x1f); }  // l ^ 16
+__device__ __forceinline__ int xchg32_i32(int v) { return __shfl_xor(v, 32, 64); }                                 // l ^ 32
 
-__device__ __forceinline__ float wave_max_f32(float p)
-{
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) p = fmaxf(p, __shfl_xor(p, off, 64));
-    return p;
-}
-
-__device__ __forceinline__ int wave_sum_i32(int p)
-{
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) p += __shfl_xor(p, off, 64);
-    return p;
-}
+#define BITNET_WAVE_REDUCE(TYPE, NAME, COMBINE)                                                    \
+    __device__ __forceinline__ TYPE NAME(TYPE p)                                                   \
+    {                                                                                              \
+        auto step = [](TYPE a, int other_bits) { TYPE b = __builtin_bit_cast(TYPE, other_bits); return COMBINE; }; \
+        p = step(p, dpp_i32<0xB1>(__builtin_bit_cast(int, p)));                                    \
+        p = step(p, dpp_i32<0x4E>(__builtin_bit_cast(int, p)));                                    \
+        p = step(p, dpp_i32<0x141>(__builtin_bit_cast(int, p)));                                   \
+        p = step(p, dpp_i32<0x140>(__builtin_bit_cast(int, p)));                                   \
+        p = step(p, xchg16_i32(__builtin_bit_cast(int, p)));                                       \
+        p = step(p, xchg32_i32(__builtin_bit_cast(int, p)));                                       \
+        return p;                                                                                  \
+    }
+BITNET_WAVE_REDUCE(float, wave_sum_f32, f32_add(a, b))
+BITNET_WAVE_REDUCE(float, wave_max_f32, fmaxf(a, b))
+BITNET_WAVE_REDUCE(int, wave_sum_i32, a + b)
+#undef BITNET_WAVE_REDUCE
 
 __device__ __forceinline__ float relu2_mul(float gate, float up)
 {
@@ -144,10 +154,32 @@ __device__ __forceinline__ float rms_from_ss(float ss, int k, float eps)
     return f32_sqrt(f32_add(f32_div(ss, (float)k), eps));
 }
 
-__device__ __forceinline__ float4 normalize4(const float4 &e, float rms, const float4 &g)
+// (x / rms) * g for the four elements of a chunk.  The divisor is the same for the whole row, so the division
+// uses div_by_invariant (ieee.hpp), which returns the same bits as x / rms.
+struct RowDivisor {
+    float d, recip;
+    bool fast;
+};
+__device__ __forceinline__ RowDivisor make_row_divisor(float rms)
 {
-    return make_float4(f32_mul(f32_div(e.x, rms), g.x), f32_mul(f32_div(e.y, rms), g.y),
-                       f32_mul(f32_div(e.z, rms), g.z), f32_mul(f32_div(e.w, rms), g.w));
+    RowDivisor r;
+    r.d = rms;
+    r.recip = f32_div(1.0f, rms);
+    r.fast = invariant_divisor_ok(rms);
+    return r;
+}
+__device__ __forceinline__ float4 normalize4(const float4 &e, const RowDivisor &r, const float4 &g)
+{
+    // the short division when the divisor and, in every lane of the wavefront, all four dividends allow it
+    const bool lane_ok = dividend_ok(e.x) && dividend_ok(e.y) && dividend_ok(e.z) && dividend_ok(e.w);
+    float4 q;
+    if (r.fast && __builtin_amdgcn_ballot_w64(!lane_ok) == 0) {
+        q = make_float4(div_by_invariant_unchecked(e.x, r.d, r.recip), div_by_invariant_unchecked(e.y, r.d, r.recip),
+                        div_by_invariant_unchecked(e.z, r.d, r.recip), div_by_invariant_unchecked(e.w, r.d, r.recip));
+    } else {
+        q = make_float4(f32_div(e.x, r.d), f32_div(e.y, r.d), f32_div(e.z, r.d), f32_div(e.w, r.d));
+    }
+    return make_float4(f32_mul(q.x, g.x), f32_mul(q.y, g.y), f32_mul(q.z, g.z), f32_mul(q.w, g.w));
 }
 
 __device__ __forceinline__ float absmax4(float amax, const float4 &e)
@@ -162,10 +194,10 @@ __device__ __forceinline__ float scale_from_absmax(float amax)
 
 __device__ __forceinline__ int quant1(float y, float scale)
 {
-    float t = roundf(f32_mul(y, scale));
-    if (t != t) return 0;  // NaN quantises to 0, as Rust's `as i8` does
-    t = fminf(fmaxf(t, -128.0f), 127.0f);
-    return (int)t;
+    // round half away from zero, then a saturating conversion (NaN converts to 0, as Rust's `as i8` does),
+    // then the clamp to [-128, 127] on the integer
+    const int q = __float2int_rz(roundf(f32_mul(y, scale)));
+    return min(max(q, -128), 127);
 }
 
 // Four quantised values of a chunk packed little-endian (byte j = element j); *sum += their sum.

@@ -47,7 +47,7 @@
  * ORC_SUM_BLOCK256: the row is cut into chunks of 4 consecutive elements; chunk c belongs to lane
  * c mod 256; a lane adds the squares of its chunks in ascending chunk order and, inside a chunk, in
  * ascending element order, starting from +0.  Elements past K count as 0.  The 256 partials form 4
- * groups of 64 consecutive lanes; each group is combined by a butterfly: for off = 32,16,8,4,2,1:
+ * groups of 64 consecutive lanes; each group is combined by a butterfly: for off = 1,2,4,8,16,32:
  * p[l] = p[l] + p[l ^ off] (IEEE addition is commutative, so every lane of a group ends with the same
  * value).  The four group sums are added as ((s0 + s1) + s2) + s3. */
 float orc_sum_squares(const float *x, size_t k, int order)
@@ -72,7 +72,7 @@ float orc_sum_squares(const float *x, size_t k, int order)
             p[l] = p[l] + sq;
         }
     }
-    for (int off = 32; off >= 1; off >>= 1) {
+    for (int off = 1; off <= 32; off <<= 1) {
         for (int l = 0; l < 256; ++l) t[l] = p[l] + p[l ^ off]; /* l ^ off stays inside l's group of 64 */
         memcpy(p, t, sizeof p);
     }

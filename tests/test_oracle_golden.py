@@ -269,7 +269,7 @@ def np_block256_sum_squares(x):
     for rnd in range(xp.shape[0]):
         for j in range(4):
             p = (p + xp[rnd, :, j] * xp[rnd, :, j]).astype(f32)
-    for off in (32, 16, 8, 4, 2, 1):
+    for off in (1, 2, 4, 8, 16, 32):
         p = (p + p[np.arange(256) ^ off]).astype(f32)
     return f32(f32(f32(p[0] + p[64]) + p[128]) + p[192])
 
