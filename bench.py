@@ -127,6 +127,36 @@ def prefill_rates(bh, torch, dec, gen, reps):
     return res
 
 
+def stack_latency(bh, torch, dec, gen, reps=20):
+    """configs[4]: per-token decode latency through all 30 layers' projections, batch 1 and batch 8, and
+    configs[2]: the gate / down projections at M in {1, 4, 16, 64} tokens (activations with 1 % x20 outliers)."""
+    out = {}
+    big = bh.DecoderProjections(dec.layers, HIDDEN, FFN, Q_HEADS, KV_HEADS, HEAD_DIM, eps=1e-5, max_tokens=8)
+    for l in range(dec.layers):
+        for p in range(7):
+            packed, scale = dec.projection(l, p).get_quantized_weights()
+            big.projection(l, p).set_quantized_weights(packed.cuda(), scale)
+    for m in (1, 8):
+        x = torch.randn((m, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
+        y = torch.empty_like(x)
+        big.decode(x, out=y)
+        ms = time_events(torch, lambda: [big.decode(x, out=y) for _ in range(reps)]) / reps
+        out[f"stack30_batch{m}"] = {"us_per_token_step": round(ms * 1e3, 1),
+                                    "gbs_packed_weights": round(dec.weight_bytes() / (ms * 1e-3) / 1e9, 1)}
+    del big
+    for name, p in (("gate_2560x6912", 4), ("down_6912x2560", 6)):
+        n, k = dec.proj_shape(p)
+        bl = dec.projection(0, p)
+        for m in (1, 4, 16, 64):
+            x = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32)
+            mask = torch.rand((m, k), generator=gen, device="cuda") < 0.01
+            x = torch.where(mask, x * 20.0, x).contiguous()
+            bl.forward(x)
+            ms = time_events(torch, lambda: [bl.forward(x) for _ in range(50)]) / 50
+            out[f"{name}_m{m}"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1)}
+    return out
+
+
 def cpu_baseline(torch, dec, budget_s=15.0):
     """The reference's BitLinear::forward on the host cores: per call, materialise q*scale as f32 [N,K], then an
     f32 GEMV (bitnet-quant/src/bitlinear/forward.rs:153-258), for the seven projections of one layer."""
@@ -229,6 +259,7 @@ def main():
     if not args.no_extras:
         line["gemv_only"] = gemv_only(bh, torch, dec, gen, reps=5)
         line["prefill"] = prefill_rates(bh, torch, dec, gen, reps=5)
+        line["other_configs"] = stack_latency(bh, torch, dec, gen)
         if not args.no_cpu_baseline:
             line["cpu_baseline"] = cpu_baseline(torch, dec)
     print(json.dumps(line))

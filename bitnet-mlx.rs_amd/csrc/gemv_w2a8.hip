@@ -26,6 +26,12 @@
 //   * up to three projections that share the input row (q, k, v or gate, up): the grid is the
 //     concatenation of their row blocks.
 // HBM traffic per call: n*k/4 weight bytes; the input row (K or 4K bytes per workgroup) comes from L2.
+//
+// gemv_mfma_kernel is the same weight-streaming scheme for 2..16 token rows: the 16 x 16 x 64 int8 MFMA takes
+// the place of the dot-product chain (its A operand is 16 token rows x 64 columns, loaded straight from the
+// int8 activation matrix, which stays in L2; its B operand is a decoded weight dword, exactly as in the
+// prefill GEMM), so up to 16 tokens cost what one costs in weight traffic and instructions.  A workgroup
+// owns RB adjacent 16-row blocks so that the activation matrix is re-read by fewer workgroups.
 #include "kernels.hpp"
 #include "rowquant.hpp"
 
@@ -290,6 +296,158 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
     }
 }
 
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+struct GemvMfmaParams {
+    GemvProjDev proj[GEMV_MAX_PROJ];  // rb_end counts groups of RB row blocks
+    int nproj;
+    const int8_t *a;       // [m, k] int8
+    const float *a_scale;  // [m]
+    int m;                 // 1..16
+    int k;
+    int kt_count;
+};
+
+template <int RB>
+__global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
+{
+    __shared__ int red[3][RB][64][4];  // partial accumulators of wavefronts 1..3
+    __shared__ int red_sum[4][16];     // per wavefront: sum_k a[t, k] over its k-tiles
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
+
+    int pj = 0;
+#pragma unroll
+    for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
+        if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
+    const GemvProjDev &P = p.proj[pj];
+    const int grp = (int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0);
+    const int rb0 = grp * RB;
+    const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
+    const uint4 *wbase = reinterpret_cast<const uint4 *>(P.w) + lane;
+
+    // A operand of this lane: token row lr, the 16 columns 64t + 16lg of each k-tile (rows past m read as zero)
+    const bool row_ok = lr < p.m;
+    const bool a_vec = (p.k % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0);
+    const int8_t *arow = p.a + (size_t)(row_ok ? lr : 0) * p.k + lg * 16;
+    auto load_a = [&](int kt, int t) -> v4i {
+        v4i v = (v4i){0, 0, 0, 0};
+        const int col = kt * TILE_K + t * 64 + lg * 16;
+        if (row_ok && col < p.k) {
+            const int8_t *src = arow + kt * TILE_K + t * 64;
+            if (a_vec) {
+                v = *reinterpret_cast<const v4i *>(src);
+            } else {
+                int d[4] = {0, 0, 0, 0};
+                for (int j = 0; j < 16; ++j)
+                    if (col + j < p.k) d[j >> 2] |= (int)((uint32_t)(uint8_t)src[j] << (8 * (j & 3)));
+                v = (v4i){d[0], d[1], d[2], d[3]};
+            }
+        }
+        return v;
+    };
+    auto load_w = [&](int kt, uint4 (&w)[RB]) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            const int rb = rb0 + r;
+            w[r] = rb < rb_count ? wbase[((size_t)rb * p.kt_count + kt) * 64]
+                                 : make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
+        }
+    };
+
+    v4i acc[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) acc[r] = (v4i){0, 0, 0, 0};
+    int rowsum = 0;
+
+    constexpr int PF = RB == 1 ? 4 : (RB == 2 ? 3 : 2);  // bounded by the register file
+    // All loads of a batch of PF k-tiles are issued before the first MFMA of the batch, and the next
+    // batch is requested while the current one is computed: the weight stream is what the kernel waits for.
+    uint4 wcur[PF][RB], wnxt[PF][RB];
+    v4i acur[PF][4], anxt[PF][4];
+    auto load_batch = [&](int kt0, uint4 (&w)[PF][RB], v4i (&a)[PF][4]) {
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            const int kt = kt0 + 4 * u;
+            if (kt < p.kt_count) {
+                load_w(kt, w[u]);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) a[u][t] = load_a(kt, t);
+            }
+        }
+    };
+    load_batch(wave, wcur, acur);
+    for (int kt0 = wave; kt0 < p.kt_count; kt0 += 4 * PF) {
+        load_batch(kt0 + 4 * PF, wnxt, anxt);
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            if (kt0 + 4 * u >= p.kt_count) continue;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const v4i af = acur[u][t];
+                rowsum = __builtin_amdgcn_sdot4(af[0], 0x01010101, rowsum, false);
+                rowsum = __builtin_amdgcn_sdot4(af[1], 0x01010101, rowsum, false);
+                rowsum = __builtin_amdgcn_sdot4(af[2], 0x01010101, rowsum, false);
+                rowsum = __builtin_amdgcn_sdot4(af[3], 0x01010101, rowsum, false);
+#pragma unroll
+                for (int r = 0; r < RB; ++r) {
+                    const uint4 w4 = wcur[u][r];
+                    const uint32_t wd = t == 0 ? w4.x : (t == 1 ? w4.y : (t == 2 ? w4.z : w4.w));
+                    v4i bf;
+                    bf[0] = (int)(wd & 0x03030303u);
+                    bf[1] = (int)((wd >> 2) & 0x03030303u);
+                    bf[2] = (int)((wd >> 4) & 0x03030303u);
+                    bf[3] = (int)((wd >> 6) & 0x03030303u);
+                    acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf, acc[r], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+#pragma unroll
+            for (int r = 0; r < RB; ++r) wcur[u][r] = wnxt[u][r];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acur[u][t] = anxt[u][t];
+        }
+    }
+
+    // sum_k a[lr, k] over this wavefront's tiles: lanes lr, lr+16, lr+32, lr+48 hold the four column groups
+    rowsum += __shfl_xor(rowsum, 16, 64);
+    rowsum += __shfl_xor(rowsum, 32, 64);
+    if (lane < 16) red_sum[wave][lane] = rowsum;
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave - 1][r][lane][i] = acc[r][i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const float ws = P.out ? *P.w_scale : 0.0f;
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            const int n = (rb0 + r) * TILE_ROWS + lr;  // result register i of lane l is C[4*(l/16) + i][l mod 16]
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int t = lg * 4 + i;
+                if (n < P.n && t < p.m) {
+                    const int asum = red_sum[0][t] + red_sum[1][t] + red_sum[2][t] + red_sum[3][t];
+                    const int total = acc[r][i] + red[0][r][lane][i] + red[1][r][lane][i] + red[2][r][lane][i] - asum;
+                    const size_t o = (size_t)t * P.n + n;
+                    if (P.acc) P.acc[o] = total;
+                    if (P.out) {
+                        float v = f32_div(f32_mul((float)total, ws), p.a_scale[t]);
+                        if (P.bias) v = f32_add(v, P.bias[n]);
+                        if (P.residual) v = f32_add(v, P.residual[o]);
+                        P.out[o] = v;
+                    }
+                }
+            }
+        }
+    }
+}
+
 // The reference's flat row-major packing, any n and k (rows need not start on a byte boundary).
 // One wavefront per output row; lane l takes columns 4l..4l+3, 4l+256.., gathers their codes one by one.
 __global__ __launch_bounds__(256) void gemv_rowmajor_kernel(const uint8_t *packed, const int8_t *a,
@@ -342,23 +500,9 @@ int launch_mb_mode(const GemvParams &p, hipStream_t stream)
 }
 
 template <int MODE>
-int launch_mode(const GemvParams &p, int mb, hipStream_t stream)
+int launch_mode(const GemvParams &p, hipStream_t stream)
 {
-    switch (mb) {
-        case 8: return launch_mb_mode<8, MODE>(p, stream);
-        case 4: return launch_mb_mode<4, MODE>(p, stream);
-        case 2: return launch_mb_mode<2, MODE>(p, stream);
-        default: return launch_mb_mode<1, MODE>(p, stream);
-    }
-}
-
-// rows per launch that fit the 60 KB LDS budget
-int rows_per_launch(size_t m, size_t k)
-{
-    const size_t row_lds = k_tiles(k) * 16 * sizeof(uint4);
-    int mb = m > 4 ? 8 : (m > 2 ? 4 : (m > 1 ? 2 : 1));
-    while (mb > 1 && mb * row_lds > 60 * 1024) mb >>= 1;
-    return mb;
+    return launch_mb_mode<1, MODE>(p, stream);  // one token row per launch; 2..16 rows take gemv_mfma_kernel
 }
 
 int fill_projs(GemvParams &p, const GemvProj *projs, int nproj, size_t t0, size_t k)
@@ -381,6 +525,28 @@ int fill_projs(GemvParams &p, const GemvProj *projs, int nproj, size_t t0, size_
     return rb_end;
 }
 
+template <int RB>
+int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const float *a_scale, size_t m, size_t k,
+                   hipStream_t stream)
+{
+    GemvMfmaParams p = {};
+    int end = 0;
+    for (int j = 0; j < nproj; ++j) {
+        const GemvProj &s = projs[j];
+        GemvProjDev &d = p.proj[j];
+        d.w = s.tiled; d.w_scale = s.w_scale; d.bias = s.bias; d.residual = s.residual; d.out = s.out; d.acc = s.acc;
+        d.n = (int)s.n;
+        end += (int)((row_blocks(s.n) + RB - 1) / RB);
+        d.rb_end = end;
+    }
+    for (int j = nproj; j < GEMV_MAX_PROJ; ++j) p.proj[j] = p.proj[nproj - 1];
+    p.nproj = nproj; p.a = a; p.a_scale = a_scale; p.m = (int)m; p.k = (int)k; p.kt_count = (int)k_tiles(k);
+    if (end == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL((gemv_mfma_kernel<RB>), dim3((unsigned)end), dim3(256), 0, stream, p);
+    BITNET_HIP_CHECK_LAUNCH("gemv_mfma_kernel");
+    return BITNET_HIP_OK;
+}
+
 }  // namespace
 
 int launch_gemv_rowmajor(const uint8_t *packed, const int8_t *a, int32_t *out, size_t n, size_t k,
@@ -397,30 +563,48 @@ int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const f
                       hipStream_t stream)
 {
     if (m == 0 || nproj <= 0) return BITNET_HIP_OK;
+    if (m >= 2 && m <= (size_t)GEMV_MFMA_MAX_M) {
+        // 2..16 tokens: the MFMA variant.  Workgroups take more row blocks when there are plenty of them, so that
+        // fewer workgroups re-read the activation matrix.
+        size_t blocks = 0;
+        for (int j = 0; j < nproj; ++j) blocks += row_blocks(projs[j].n);
+        if (blocks >= 800) return launch_mfma_rb<4>(projs, nproj, a, a_scale, m, k, stream);
+        if (blocks >= 400) return launch_mfma_rb<2>(projs, nproj, a, a_scale, m, k, stream);
+        return launch_mfma_rb<1>(projs, nproj, a, a_scale, m, k, stream);
+    }
+    if (m > 1) {  // more rows than one MFMA row block: in groups of 16
+        for (size_t t0 = 0; t0 < m; t0 += (size_t)GEMV_MFMA_MAX_M) {
+            GemvProj sub[GEMV_MAX_PROJ];
+            const size_t rows = m - t0 < (size_t)GEMV_MFMA_MAX_M ? m - t0 : (size_t)GEMV_MFMA_MAX_M;
+            for (int j = 0; j < nproj; ++j) {
+                sub[j] = projs[j];
+                if (sub[j].residual) sub[j].residual += t0 * sub[j].n;
+                if (sub[j].out) sub[j].out += t0 * sub[j].n;
+                if (sub[j].acc) sub[j].acc += t0 * sub[j].n;
+            }
+            int rc = launch_mfma_rb<1>(sub, nproj, a + t0 * k, a_scale ? a_scale + t0 : nullptr, rows, k, stream);
+            if (rc != BITNET_HIP_OK) return rc;
+        }
+        return BITNET_HIP_OK;
+    }
     if (k_tiles(k) * 16 * sizeof(uint4) > 60 * 1024)
         return fail(BITNET_HIP_UNSUPPORTED, "decode GEMV: k=%zu does not fit the LDS activation buffer", k);
-    const int mb = rows_per_launch(m, k);
-    for (size_t t0 = 0; t0 < m; t0 += (size_t)mb) {
-        GemvParams p = {};
-        if (fill_projs(p, projs, nproj, t0, k) == 0) return BITNET_HIP_OK;
-        p.m = (int)((m - t0) < (size_t)mb ? (m - t0) : (size_t)mb);
-        p.a = a + t0 * k;
-        p.a_scale = a_scale ? a_scale + t0 : nullptr;
-        int rc = launch_mode<MODE_PREQUANT>(p, mb, stream);
-        if (rc != BITNET_HIP_OK) return rc;
-    }
-    return BITNET_HIP_OK;
+    GemvParams p = {};
+    if (fill_projs(p, projs, nproj, 0, k) == 0) return BITNET_HIP_OK;
+    p.m = 1;
+    p.a = a;
+    p.a_scale = a_scale;
+    return launch_mode<MODE_PREQUANT>(p, stream);
 }
 
 bool gemv_fused_supported(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
                           size_t head_dim, const float *gamma)
 {
     auto al16 = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
-    if (m == 0 || m > (size_t)GEMV_MAX_M) return false;
+    if (m != 1) return false;  // several tokens: stand-alone quantiser (rows in parallel) + MFMA GEMV
     if (k % 4 != 0 || ldx % 4 != 0 || k > (size_t)FUSED_NCH * 1024) return false;
     if (!al16(x) || (x2 && !al16(x2)) || (gamma && !al16(gamma))) return false;
     if (input_mode == BITNET_HIP_INPUT_GQA_BROADCAST && head_dim % 4 != 0) return false;
-    if ((size_t)rows_per_launch(m, k) < m) return false;  // one launch must hold every row
     return k_tiles(k) * 16 * sizeof(uint4) <= 60 * 1024;
 }
 
@@ -436,11 +620,10 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
     p.src.head_dim = (int)(head_dim ? head_dim : 1); p.src.gqa_group = (int)(gqa_group ? gqa_group : 1);
     p.src.sum_order = sum_order; p.src.eps = eps;
     p.q_out = q_out; p.a_scale_out = a_scale_out; p.a_sum_out = a_sum_out;
-    const int mb = rows_per_launch(m, k);
     switch (input_mode) {
-        case BITNET_HIP_INPUT_PLAIN: return launch_mode<BITNET_HIP_INPUT_PLAIN>(p, mb, stream);
-        case BITNET_HIP_INPUT_RELU2_MUL: return launch_mode<BITNET_HIP_INPUT_RELU2_MUL>(p, mb, stream);
-        default: return launch_mode<BITNET_HIP_INPUT_GQA_BROADCAST>(p, mb, stream);
+        case BITNET_HIP_INPUT_PLAIN: return launch_mode<BITNET_HIP_INPUT_PLAIN>(p, stream);
+        case BITNET_HIP_INPUT_RELU2_MUL: return launch_mode<BITNET_HIP_INPUT_RELU2_MUL>(p, stream);
+        default: return launch_mode<BITNET_HIP_INPUT_GQA_BROADCAST>(p, stream);
     }
 }
 

@@ -375,9 +375,13 @@ class BitLinear:
             q = torch.empty((m, self.config.in_features), dtype=torch.int8, device=x.device)
             a_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
             acc = torch.empty((m, nout), dtype=torch.int32, device=x.device)
+        # scratch for the quantised activations comes from torch's caching allocator (the library would otherwise
+        # allocate stream-ordered memory itself on every call)
+        ws_bytes = lib.bitnet_hip_bitlinear_workspace_size(self._h, m) if m > 0 else 0
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=x.device) if ws_bytes else None
         _check(lib.bitnet_hip_bitlinear_forward(self._h, _ptr(x), dims, x.dim(), _ptr(gamma), self.config.rms_norm_eps,
-                                                self.config.sum_order, _ptr(residual), _ptr(out), None, 0, _ptr(q),
-                                                _ptr(a_scale), _ptr(acc), _stream(stream)))
+                                                self.config.sum_order, _ptr(residual), _ptr(out), _ptr(ws), ws_bytes,
+                                                _ptr(q), _ptr(a_scale), _ptr(acc), _stream(stream)))
         if debug:
             return out, q, a_scale, acc
         return out
