@@ -15,22 +15,25 @@
 // codes c = w + 1 in {0,1,2}; the epilogue subtracts sum_k a[t, k] per token row (accumulated on the fly
 // while the activation tile passes through registers on its way to LDS).
 //
-// Two kernels share this scheme.
+// Three kernels share this scheme.
 //
 // gemm_dma_kernel (k a multiple of 256, 16-byte aligned activations, row sums supplied by the activation
 // quantiser): activations AND weight tiles travel global -> LDS with LDS-direct loads
-// (global_load_lds_dwordx4), never through registers.  Three LDS stages of 128 columns are kept in flight;
-// the wait counts are placed by hand (s_waitcnt vmcnt(N)) so that two stages of loads stay outstanding
+// (global_load_lds_dwordx4), never through registers.  D LDS stages of 128 columns are kept in flight;
+// the wait counts are placed by hand (s_waitcnt vmcnt(N)) so that D - 1 stages of loads stay outstanding
 // while one is computed.  An LDS-direct load writes lane l's 16 bytes at base + 16*l, so the XOR swizzle
 // that keeps the fragment reads free of bank conflicts is applied to the global address each lane fetches.
+// The MFMA takes the weight fragment as its first operand, so a lane ends up with four consecutive output
+// columns of one token row and the epilogue stores 16 bytes per lane.
+//
+// gemm_dma8_kernel: the same data path with eight wavefronts per workgroup, for launches with about one tile
+// per compute unit (see its own comment).
 //
 // gemm_tiled_kernel (any shape, computes the row sums itself): activations pass through registers.
 // Activations are staged through LDS one weight tile (256 columns) at a time, double buffered: the global
 // loads of stage s+1 are issued before the 4 k-steps of stage s are computed and written to LDS after them,
 // one barrier per stage.  Rows are padded to 272 bytes so that the 16-byte fragment reads of 8 consecutive
 // lanes fall in distinct banks.
-#include <cstdlib>
-
 #include "kernels.hpp"
 
 namespace bitnet {
@@ -252,24 +255,38 @@ __device__ __forceinline__ void wait_vm()
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-constexpr int DMA_SK = 128;  // columns per activation stage
-constexpr int DMA_NST = 3;   // activation stages in LDS
+constexpr int DMA_SK = 128;  // columns per activation stage; a 256-column weight tile serves two stages
 
-template <int BM, int BN>
-constexpr size_t dma_lds_bytes() { return (size_t)DMA_NST * BM * DMA_SK + 2 * (BN / 16) * 1024; }
+// D activation stages and NB weight buffers live in LDS; loads run P = D - 1 stages ahead of the MFMAs.
+template <int D>
+constexpr int dma_nb() { return (D - 1 + 2 + 1) / 2; }
+template <int BM, int BN, int D>
+constexpr size_t dma_lds_bytes() { return (size_t)D * BM * DMA_SK + (size_t)dma_nb<D>() * (BN / 16) * 1024; }
 
-template <int BM, int BN>
-__global__ __launch_bounds__(256, 2) void gemm_dma_kernel(GemmParams p)
+// Loads of the groups issued after stage s's own group and before the wait at the top of stage s: the groups
+// of stages s+1 .. s+P-1; a group holds A_DMA activation loads, plus B_DMA weight loads when its stage is even.
+template <int PHASE, int P, int A_DMA, int B_DMA>
+constexpr int dma_in_flight()
+{
+    int n = 0;
+    for (int j = 1; j < P; ++j) n += A_DMA + (((PHASE + j) & 1) == 0 ? B_DMA : 0);
+    return n;
+}
+
+template <int BM, int BN, int D, int OCC>
+__global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
 {
     constexpr int WTM = BM / 2, WTN = BN / 2, FM = WTM / 16, FN = WTN / 16;
+    constexpr int P = D - 1, NB = dma_nb<D>();
     constexpr int A_STAGE = BM * DMA_SK;
     constexpr int A_DMA = A_STAGE / 1024 / 4;  // LDS-direct loads per wavefront per activation stage
     constexpr int B_TILES = BN / 16;           // weight tiles per 256 columns
     constexpr int B_DMA = (B_TILES + 3) / 4;   // per wavefront (the last ones may repeat a tile)
     constexpr int B_STAGE = B_TILES * 1024;
-    static_assert(A_STAGE % 4096 == 0 && WTM % 16 == 0 && WTN % 16 == 0, "tile shape");
+    static_assert(A_STAGE % 4096 == 0 && WTM % 16 == 0 && WTN % 16 == 0 && D >= 3, "tile shape");
+    static_assert(dma_in_flight<0, P, A_DMA, B_DMA>() < 64 && dma_in_flight<1, P, A_DMA, B_DMA>() < 64, "vmcnt range");
 
-    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [NST][A_STAGE] then [2][B_STAGE]
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [D][A_STAGE] then [NB][B_STAGE]
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1, lr = lane & 15, lg = lane >> 4;
@@ -298,24 +315,26 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_kernel(GemmParams p)
         if (grow >= p.m) grow = p.m - 1;
         a_src[q] = p.a + (size_t)grow * p.k + lc * 16;
     }
-    auto issue_a = [&](int s) {
-        const uint32_t dst = lds_base + (s % DMA_NST) * A_STAGE + wave * A_DMA * 1024;
-#pragma unroll
-        for (int q = 0; q < A_DMA; ++q) dma16(a_src[q] + (size_t)s * DMA_SK, dst + q * 1024);
-    };
     // Weight tiles: wavefront w fetches tiles w, w+4, ... of the workgroup's BN/16 row blocks; lane l = slot l.
     const int rb0 = n0 / 16;
     const int rb_last = (p.n + 15) / 16 - 1;
-    auto issue_b = [&](int kt) {
-        const uint32_t dst = lds_base + DMA_NST * A_STAGE + (kt & 1) * B_STAGE;
+    // The load group of stage s: the weight tile of k-tile s/2 when s is even, then the activation stage.
+    auto issue = [&](int s) {
+        if ((s & 1) == 0) {
+            const int kt = s >> 1;
+            const uint32_t dst = lds_base + D * A_STAGE + (kt % NB) * B_STAGE;
 #pragma unroll
-        for (int q = 0; q < B_DMA; ++q) {
-            int tix = wave + 4 * q;
-            if (tix >= B_TILES) tix = B_TILES - 1;
-            int rb = rb0 + tix;
-            if (rb > rb_last) rb = rb_last;
-            dma16(p.w + (((size_t)rb * p.kt_count + kt) * 64 + lane) * 16, dst + tix * 1024);
+            for (int q = 0; q < B_DMA; ++q) {
+                int tix = wave + 4 * q;
+                if (tix >= B_TILES) tix = B_TILES - 1;
+                int rb = rb0 + tix;
+                if (rb > rb_last) rb = rb_last;
+                dma16(p.w + (((size_t)rb * p.kt_count + kt) * 64 + lane) * 16, dst + tix * 1024);
+            }
         }
+        const uint32_t dst = lds_base + (s % D) * A_STAGE + wave * A_DMA * 1024;
+#pragma unroll
+        for (int q = 0; q < A_DMA; ++q) dma16(a_src[q] + (size_t)s * DMA_SK, dst + q * 1024);
     };
 
     v4i acc[FM][FN];
@@ -324,21 +343,26 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_kernel(GemmParams p)
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j] = (v4i){0, 0, 0, 0};
 
-    issue_b(0);
-    issue_a(0);
-    issue_a(1);
+#pragma unroll
+    for (int s = 0; s < P; ++s)
+        if (s < nstage) issue(s);
 
     uint32_t a_rd[FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i) a_rd[i] = (wm * WTM + i * 16 + lr) * DMA_SK;
     const int sw = lr & 7;
 
-    auto compute = [&](int s, int kt, bool second_half) {
-        const uint8_t *abuf = lds + (s % DMA_NST) * A_STAGE;
-        const uint8_t *bbuf = lds + DMA_NST * A_STAGE + (kt & 1) * B_STAGE + (wn * FN) * 1024 + lane * 16;
-        uint4 bp[FN];
+    // The MFMA computes C^T: the weight fragment is the first operand, so that result register r of lane l is
+    // out[token row l % 16][output column 4*(l/16) + r]: four consecutive columns, one 16-byte store.
+    uint4 bp[FN];  // the wavefront's slots of the current weight tiles: read at an even stage, used by two
+    auto compute = [&](int s, bool second_half) {
+        const int kt = s >> 1;
+        const uint8_t *abuf = lds + (s % D) * A_STAGE;
+        if (!second_half) {
+            const uint8_t *bbuf = lds + D * A_STAGE + (kt % NB) * B_STAGE + (wn * FN) * 1024 + lane * 16;
 #pragma unroll
-        for (int j = 0; j < FN; ++j) bp[j] = *reinterpret_cast<const uint4 *>(bbuf + j * 1024);
+            for (int j = 0; j < FN; ++j) bp[j] = *reinterpret_cast<const uint4 *>(bbuf + j * 1024);
+        }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             v4i afrag[FM];
@@ -355,61 +379,296 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_kernel(GemmParams p)
                 bfrag[3] = (int)((wd >> 6) & 0x03030303u);
 #pragma unroll
                 for (int i = 0; i < FM; ++i)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[i], bfrag, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bfrag, afrag[i], acc[i][j], 0, 0, 0);
             }
         }
     };
 
-    // Loads retire in issue order.  At the top of stage s everything issued before the previous stage's
-    // issue group must have landed; that group (A_DMA loads, plus B_DMA after an even stage) may stay in flight.
+    // Loads retire in issue order.  At the top of stage s its own group must have landed; the groups of the
+    // P - 1 later stages stay in flight.  The last P - 1 stages, with fewer groups behind them, drain everything.
     for (int s = 0; s < nstage; s += 2) {
-        const int kt = s >> 1;
-        wait_vm<A_DMA>();  // the previous (odd) stage issued one activation stage only
+        if (s + P <= nstage) wait_vm<dma_in_flight<0, P, A_DMA, B_DMA>()>(); else wait_vm<0>();
         __syncthreads();
-        if (kt + 1 < p.kt_count) issue_b(kt + 1);
-        if (s + 2 < nstage) issue_a(s + 2);
-        compute(s, kt, false);
+        if (s + P < nstage) issue(s + P);
+        compute(s, false);
 
-        if (s + 2 < nstage) {
-            if (kt + 1 < p.kt_count) wait_vm<A_DMA + B_DMA>(); else wait_vm<A_DMA>();
-        } else {
-            wait_vm<0>();
-        }
+        if (s + 1 + P <= nstage) wait_vm<dma_in_flight<1, P, A_DMA, B_DMA>()>(); else wait_vm<0>();
         __syncthreads();
-        if (s + 3 < nstage) issue_a(s + 3);
-        compute(s + 1, kt, true);
+        if (s + 1 + P < nstage) issue(s + 1 + P);
+        compute(s + 1, true);
     }
 
     const float ws = p.out ? *p.w_scale : 0.0f;
     const unsigned ws_expo = (__builtin_bit_cast(unsigned, ws) >> 23) & 0xffu;
     const bool ws_fast = ws > 0.0f && ws_expo > 64u && ws_expo < 160u;
+    const bool vec_ok = (p.n & 3) == 0;  // 16-byte alignment of out[row][4c]
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
+        const int row = m0 + wm * WTM + i * 16 + lr;
+        const bool row_ok = row < p.m;
+        const int rs = row_ok ? p.a_sum[row] : 0;
+        const float as = (p.out && row_ok) ? p.a_scale[row] : 1.0f;
+        const float as_recip = f32_div(1.0f, as);
+        // the short division needs a well-behaved divisor (per row) and dividends in range: float(total) * ws
+        // is zero or has ws's exponent plus at most 24, so one check on ws covers them.  The choice is made
+        // per wavefront so that the usual case runs no plain division at all.
+        const bool row_fast = ws_fast && invariant_divisor_ok(as);
+        const bool wave_fast = __builtin_amdgcn_ballot_w64(!row_fast) == 0;
+        if (!row_ok) continue;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int row = m0 + wm * WTM + i * 16 + lg * 4 + r;
-            if (row >= p.m) continue;
-            const int rs = p.a_sum[row];
-            const float as = p.out ? p.a_scale[row] : 1.0f;
-            const float as_recip = f32_div(1.0f, as);
-            // the short division needs a well-behaved divisor (per row) and dividends in range: float(total) * ws
-            // is zero or has ws's exponent plus at most 24, so one check on ws covers them.  The choice is made
-            // per wavefront so that the usual case runs no plain division at all.
-            const bool row_fast = ws_fast && invariant_divisor_ok(as);
-            const bool wave_fast = __builtin_amdgcn_ballot_w64(!row_fast) == 0;
+        for (int j = 0; j < FN; ++j) {
+            const int col = n0 + wn * WTN + j * 16 + lg * 4;
+            if (col >= p.n) continue;
+            const size_t o = (size_t)row * p.n + col;
+            int tot[4];
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                tot[r] = acc[i][j][r] - rs;
+                const float scaled = f32_mul((float)tot[r], ws);
+                v[r] = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
+            }
+            if (vec_ok) {  // col + 3 < n follows from n % 4 == 0
+                if (p.acc) *reinterpret_cast<int4 *>(p.acc + o) = make_int4(tot[0], tot[1], tot[2], tot[3]);
+                if (p.out) {
+                    if (p.bias) {
+                        const float4 b = *reinterpret_cast<const float4 *>(p.bias + col);
+                        v[0] = f32_add(v[0], b.x); v[1] = f32_add(v[1], b.y); v[2] = f32_add(v[2], b.z); v[3] = f32_add(v[3], b.w);
+                    }
+                    if (p.residual) {
+                        const float4 q = *reinterpret_cast<const float4 *>(p.residual + o);
+                        v[0] = f32_add(v[0], q.x); v[1] = f32_add(v[1], q.y); v[2] = f32_add(v[2], q.z); v[3] = f32_add(v[3], q.w);
+                    }
+                    *reinterpret_cast<float4 *>(p.out + o) = make_float4(v[0], v[1], v[2], v[3]);
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (col + r >= p.n) continue;
+                    if (p.acc) p.acc[o + r] = tot[r];
+                    if (p.out) {
+                        float y = v[r];
+                        if (p.bias) y = f32_add(y, p.bias[col + r]);
+                        if (p.residual) y = f32_add(y, p.residual[o + r]);
+                        p.out[o + r] = y;
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int D, int OCC>
+int launch_dma(GemmParams p, hipStream_t stream)
+{
+    p.tiles_m = (p.m + BM - 1) / BM;
+    p.tiles_n = (p.n + BN - 1) / BN;
+    const int total = p.tiles_m * p.tiles_n;
+    const int grid = ((total + 7) / 8) * 8;
+    constexpr size_t lds = dma_lds_bytes<BM, BN, D>();
+    static_assert(lds <= 160 * 1024 && lds * OCC <= 160 * 1024, "LDS budget");
+    static bool attr_set = false;
+    if (lds > 64 * 1024 && !attr_set) {
+        BITNET_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_dma_kernel<BM, BN, D, OCC>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, D, OCC>), dim3(grid), dim3(256), lds, stream, p);
+    BITNET_HIP_CHECK_LAUNCH("gemm_dma_kernel");
+    return BITNET_HIP_OK;
+}
+
+// ---- eight wavefronts per workgroup, the k range of every stage split between two groups of four ---------
+//
+// One wavefront per SIMD cannot keep the MFMA pipe busy (its own LDS waits and unpack instructions sit between
+// its MFMAs); two can.  When a launch has too few tiles for two workgroups per compute unit, the second
+// wavefront per SIMD comes from inside the workgroup instead: 512 threads, wavefronts 0..3 take columns
+// 0..127 of every 256-column stage and wavefronts 4..7 columns 128..255, each group accumulating the whole
+// BM x BN tile.  The two partial tiles are exchanged through LDS at the end (int32 sums: exact), each group
+// finishing half of the fragments.  A stage is one 256-column weight tile plus BM x 256 activation bytes.
+constexpr int D8_NST = 3;
+template <int BM, int BN>
+constexpr size_t dma8_lds_bytes() { return (size_t)D8_NST * (BM * 256 + (BN / 16) * 1024); }
+
+template <int BM, int BN>
+__global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
+{
+    constexpr int WTM = BM / 2, WTN = BN / 2, FM = WTM / 16, FN = WTN / 16;
+    constexpr int A_STAGE = BM * 256;
+    constexpr int A_DMA = A_STAGE / 1024 / 8;   // LDS-direct loads per wavefront per stage
+    constexpr int B_TILES = BN / 16;
+    constexpr int B_DMA = (B_TILES + 7) / 8;    // per wavefront (the last ones may repeat a tile)
+    constexpr int B_STAGE = B_TILES * 1024;
+    constexpr int STAGE = A_STAGE + B_STAGE;
+    constexpr int GROUP = A_DMA + B_DMA;
+    static_assert(A_STAGE % 8192 == 0 && WTM % 32 == 0 && WTN % 16 == 0, "tile shape");
+    static_assert((FM / 2) * FN * 4 * 256 * 8 <= D8_NST * STAGE, "exchange area");
+
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [NST][A half 0 | A half 1 | B]
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kg = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1, lr = lane & 15, lg = lane >> 4;
+
+    int tile_id;
+    {
+        const int total = p.tiles_m * p.tiles_n;
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        const int per_xcd = (total + 7) >> 3;
+        tile_id = xcd * per_xcd + idx;
+        if (tile_id >= total) return;
+    }
+    const int tm = tile_id / p.tiles_n, tn = tile_id % p.tiles_n;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // Activation loads: chunk c = wave*A_DMA + q of a stage is 8 rows x 128 columns: half c / (BM/8), rows
+    // 8*(c % (BM/8)) .. +7.  Lane l lands in row l/8 at physical 16-byte chunk l%8 and fetches logical chunk
+    // (l%8) ^ (row & 7).  Rows past m re-read row m-1 (their results are never stored).
+    const int8_t *a_src[A_DMA];
+#pragma unroll
+    for (int q = 0; q < A_DMA; ++q) {
+        const int c = wave * A_DMA + q;
+        const int half = c / (BM / 8), row = 8 * (c % (BM / 8)) + (lane >> 3);
+        const int lc = (lane & 7) ^ (row & 7);
+        int grow = m0 + row;
+        if (grow >= p.m) grow = p.m - 1;
+        a_src[q] = p.a + (size_t)grow * p.k + half * 128 + lc * 16;
+    }
+    const int rb0 = n0 / 16;
+    const int rb_last = (p.n + 15) / 16 - 1;
+    auto issue = [&](int kt) {
+        const uint32_t stage = lds_base + (kt % D8_NST) * STAGE;
+#pragma unroll
+        for (int q = 0; q < B_DMA; ++q) {
+            int tix = wave + 8 * q;
+            if (tix >= B_TILES) tix = B_TILES - 1;
+            int rb = rb0 + tix;
+            if (rb > rb_last) rb = rb_last;
+            dma16(p.w + (((size_t)rb * p.kt_count + kt) * 64 + lane) * 16, stage + A_STAGE + tix * 1024);
+        }
+#pragma unroll
+        for (int q = 0; q < A_DMA; ++q)
+            dma16(a_src[q] + (size_t)kt * 256, stage + (wave * A_DMA + q) * 1024);
+    };
+
+    v4i acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = (v4i){0, 0, 0, 0};
+
+    issue(0);
+    if (p.kt_count > 1) issue(1);
+
+    uint32_t a_rd[FM];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) a_rd[i] = kg * (BM * 128) + (wm * WTM + i * 16 + lr) * 128;
+    const int sw = lr & 7;
+
+    for (int kt = 0; kt < p.kt_count; ++kt) {
+        if (kt + 1 < p.kt_count) wait_vm<GROUP>(); else wait_vm<0>();
+        __syncthreads();
+        if (kt + 2 < p.kt_count) issue(kt + 2);
+        const uint8_t *abuf = lds + (kt % D8_NST) * STAGE;
+        const uint8_t *bbuf = abuf + A_STAGE + (wn * FN) * 1024 + lane * 16 + kg * 8;
+        uint2 bp[FN];  // dwords 2*kg, 2*kg+1 of the slot: this group's two k-steps
+#pragma unroll
+        for (int j = 0; j < FN; ++j) bp[j] = *reinterpret_cast<const uint2 *>(bbuf + j * 1024);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            v4i afrag[FM];
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+                afrag[i] = *reinterpret_cast<const v4i *>(abuf + a_rd[i] + (((t * 4 + lg) ^ sw) << 4));
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
-                const int col = n0 + wn * WTN + j * 16 + lr;
-                if (col >= p.n) continue;
-                const int total = acc[i][j][r] - rs;
-                const size_t o = (size_t)row * p.n + col;
-                if (p.acc) p.acc[o] = total;
+                const uint32_t wd = t == 0 ? bp[j].x : bp[j].y;
+                v4i bfrag;
+                bfrag[0] = (int)(wd & 0x03030303u);
+                bfrag[1] = (int)((wd >> 2) & 0x03030303u);
+                bfrag[2] = (int)((wd >> 4) & 0x03030303u);
+                bfrag[3] = (int)((wd >> 6) & 0x03030303u);
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bfrag, afrag[i], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- exchange: group 0 finishes fragments i < FM/2, group 1 the others ----
+    __syncthreads();  // every wavefront is done with the stage buffers
+    {
+        constexpr int HALF = FM / 2;
+        v4i *xch = reinterpret_cast<v4i *>(lds);
+        const int mine = wave, partner = wave ^ 4;
+        // what this wavefront gives away: the half of the fragments the partner finishes
+#pragma unroll
+        for (int i = 0; i < HALF; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+                xch[((mine * HALF + i) * FN + j) * 64 + lane] = acc[kg == 0 ? i + HALF : i][j];
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < HALF; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                const v4i o = xch[((partner * HALF + i) * FN + j) * 64 + lane];
+                if (kg == 0) acc[i][j] += o; else acc[i + HALF][j] += o;
+            }
+    }
+
+    const float ws = p.out ? *p.w_scale : 0.0f;
+    const unsigned ws_expo = (__builtin_bit_cast(unsigned, ws) >> 23) & 0xffu;
+    const bool ws_fast = ws > 0.0f && ws_expo > 64u && ws_expo < 160u;
+    const bool vec_ok = (p.n & 3) == 0;
+#pragma unroll
+    for (int ii = 0; ii < FM / 2; ++ii) {
+        const int i = kg == 0 ? ii : ii + FM / 2;
+        const int row = m0 + wm * WTM + i * 16 + lr;
+        const bool row_ok = row < p.m;
+        const int rs = row_ok ? p.a_sum[row] : 0;
+        const float as = (p.out && row_ok) ? p.a_scale[row] : 1.0f;
+        const float as_recip = f32_div(1.0f, as);
+        const bool row_fast = ws_fast && invariant_divisor_ok(as);
+        const bool wave_fast = __builtin_amdgcn_ballot_w64(!row_fast) == 0;
+        if (!row_ok) continue;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int col = n0 + wn * WTN + j * 16 + lg * 4;
+            if (col >= p.n) continue;
+            const size_t o = (size_t)row * p.n + col;
+            const v4i a4 = kg == 0 ? acc[ii][j] : acc[ii + FM / 2][j];
+            int tot[4];
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                tot[r] = a4[r] - rs;
+                const float scaled = f32_mul((float)tot[r], ws);
+                v[r] = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
+            }
+            if (vec_ok) {
+                if (p.acc) *reinterpret_cast<int4 *>(p.acc + o) = make_int4(tot[0], tot[1], tot[2], tot[3]);
                 if (p.out) {
-                    const float scaled = f32_mul((float)total, ws);
-                    float v = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
-                    if (p.bias) v = f32_add(v, p.bias[col]);
-                    if (p.residual) v = f32_add(v, p.residual[o]);
-                    p.out[o] = v;
+                    if (p.bias) {
+                        const float4 b = *reinterpret_cast<const float4 *>(p.bias + col);
+                        v[0] = f32_add(v[0], b.x); v[1] = f32_add(v[1], b.y); v[2] = f32_add(v[2], b.z); v[3] = f32_add(v[3], b.w);
+                    }
+                    if (p.residual) {
+                        const float4 q = *reinterpret_cast<const float4 *>(p.residual + o);
+                        v[0] = f32_add(v[0], q.x); v[1] = f32_add(v[1], q.y); v[2] = f32_add(v[2], q.z); v[3] = f32_add(v[3], q.w);
+                    }
+                    *reinterpret_cast<float4 *>(p.out + o) = make_float4(v[0], v[1], v[2], v[3]);
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (col + r >= p.n) continue;
+                    if (p.acc) p.acc[o + r] = tot[r];
+                    if (p.out) {
+                        float y = v[r];
+                        if (p.bias) y = f32_add(y, p.bias[col + r]);
+                        if (p.residual) y = f32_add(y, p.residual[o + r]);
+                        p.out[o + r] = y;
+                    }
                 }
             }
         }
@@ -417,21 +676,22 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_kernel(GemmParams p)
 }
 
 template <int BM, int BN>
-int launch_dma(GemmParams p, hipStream_t stream)
+int launch_dma8(GemmParams p, hipStream_t stream)
 {
     p.tiles_m = (p.m + BM - 1) / BM;
     p.tiles_n = (p.n + BN - 1) / BN;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    constexpr size_t lds = dma_lds_bytes<BM, BN>();
+    constexpr size_t lds = dma8_lds_bytes<BM, BN>();
+    static_assert(lds <= 160 * 1024, "LDS budget");
     static bool attr_set = false;
-    if (lds > 64 * 1024 && !attr_set) {
-        BITNET_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_dma_kernel<BM, BN>),
+    if (!attr_set) {
+        BITNET_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_dma8_kernel<BM, BN>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_set = true;
     }
-    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN>), dim3(grid), dim3(256), lds, stream, p);
-    BITNET_HIP_CHECK_LAUNCH("gemm_dma_kernel");
+    hipLaunchKernelGGL((gemm_dma8_kernel<BM, BN>), dim3(grid), dim3(512), lds, stream, p);
+    BITNET_HIP_CHECK_LAUNCH("gemm_dma8_kernel");
     return BITNET_HIP_OK;
 }
 
@@ -465,33 +725,20 @@ int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_su
     p.w = tiled; p.a = a; p.acc = acc; p.w_scale = w_scale; p.a_scale = a_scale; p.bias = bias;
     p.residual = residual; p.a_sum = a_sum; p.out = out; p.m = (int)m; p.n = (int)n; p.k = (int)k; p.kt_count = (int)k_tiles(k);
     p.tiles_m = p.tiles_n = 0;
-    // Tile choice: wide in n (weights live in registers, so a wider tile costs no LDS traffic); among the
-    // candidates take the one whose tile count wastes the fewest slots of the last round over 256 CUs.
     const bool dma_ok = a_sum != nullptr && m >= 96 && k % 256 == 0 && k >= 512 &&
-                        (reinterpret_cast<uintptr_t>(a) & 15) == 0 && !getenv("BITNET_HIP_GEMM_NO_DMA");
+                        (reinterpret_cast<uintptr_t>(a) & 15) == 0;
     if (dma_ok) {
-        // Tile width: the time of a launch is set by the compute unit that gets the most tiles, each tile
-        // costing about its width (a 256-wide tile is ~10 % cheaper per column: fewer LDS reads per MFMA).
-        auto cost = [&](size_t bn, double per_col) {
-            const size_t tiles = ((m + 127) / 128) * ((n + bn - 1) / bn);
-            return (double)((tiles + 255) / 256) * (double)bn * per_col;
-        };
-        int bn = 160;
-        double best = cost(160, 1.0);
-        if (cost(256, 0.9) < best) { best = cost(256, 0.9); bn = 256; }
-        if (cost(128, 1.03) < best) { best = cost(128, 1.03); bn = 128; }
-        if (const char *force = getenv("BITNET_HIP_GEMM_TILE")) bn = atoi(force);  // tuning aid
-        if (bn == 256) return launch_dma<128, 256>(p, stream);
-        if (bn == 128) return launch_dma<128, 128>(p, stream);
-        return launch_dma<128, 160>(p, stream);
+        // Three shapes of the LDS-direct kernel, chosen by how many 128 x 160 tiles the output holds
+        // (256 compute units; the MFMA pipe of a SIMD needs two resident wavefronts to stay busy):
+        //   four or more tiles per compute unit  -> 128 x 160, two workgroups of 4 wavefronts per compute unit;
+        //   between a half and one tile per unit -> 128 x 160, one workgroup of 8 wavefronts (k split inside it);
+        //   otherwise                            -> 64 x 160, three workgroups of 4 wavefronts per compute unit.
+        const size_t tiles = ((m + 127) / 128) * ((n + 159) / 160);
+        if (tiles >= 1024) return launch_dma<128, 160, 3, 2>(p, stream);
+        if (tiles >= 128 && tiles <= 256) return launch_dma8<128, 160>(p, stream);
+        return launch_dma<64, 160, 3, 3>(p, stream);
     }
     if (m < 96) return launch_tile<64, 128>(p, stream);
-    if (const char *force = getenv("BITNET_HIP_GEMM_TILE")) {  // tuning aid
-        const int bn = atoi(force);
-        if (bn == 256) return launch_tile<128, 256>(p, stream);
-        if (bn == 160) return launch_tile<128, 160>(p, stream);
-        if (bn == 128) return launch_tile<128, 128>(p, stream);
-    }
     auto waste = [&](size_t bn) {
         const size_t tiles = ((m + 127) / 128) * ((n + bn - 1) / bn), slots = 256;
         const size_t rounds = (tiles + slots - 1) / slots;
