@@ -607,13 +607,24 @@ struct bitnet_hip_decoder {
     int32_t *a_sum = nullptr;
     float *qb = nullptr, *kb = nullptr, *vb = nullptr, *x1 = nullptr, *gate = nullptr, *up = nullptr;
     float *ping = nullptr;
+    // single-launch decode (decode_stack.hip): pointer table, barrier flags (+ abort word), host-visible status
+    StackLayer *table = nullptr;
+    float *ring = nullptr;     // activations of the single-launch path, one slice per block
+    unsigned *flags = nullptr;
+    unsigned *host_status = nullptr;
+    unsigned epoch = 0;
+    int grid = 0;              // one workgroup per compute unit
+    bool single_launch = false;  // shapes fit and the device takes cooperative launches
+    bool single_launch_enabled = false;  // opt-in: measured on MI355X it only matches the launch-per-group path
+    std::mutex stack_lock;     // launches share the flags: one at a time
 
     ~bitnet_hip_decoder()
     {
         for (auto *p : proj) delete p;
-        void *bufs[] = {gamma, a8, a_scale, a_sum, qb, kb, vb, x1, gate, up, ping};
+        void *bufs[] = {gamma, a8, a_scale, a_sum, qb, kb, vb, x1, gate, up, ping, table, flags, ring};
         for (void *b : bufs)
             if (b) (void)hipFree(b);
+        if (host_status) (void)hipHostFree(host_status);
     }
 };
 
@@ -666,6 +677,32 @@ int bitnet_hip_decoder_create(size_t layers, size_t hidden, size_t ffn, size_t q
         std::vector<float> ones(layers * 2 * hidden, 1.0f);
         hipError_t e = hipMemcpy(d->gamma, ones.data(), sizeof(float) * ones.size(), hipMemcpyHostToDevice);
         if (e != hipSuccess) rc = fail(BITNET_HIP_DEVICE_ERROR, "decoder_create: hipMemcpy failed: %s", hipGetErrorString(e));
+    }
+    if (rc == BITNET_HIP_OK) {
+        // single-launch path: one workgroup per compute unit, if the shapes fit its register and LDS plan
+        int dev = 0, cus = 0, coop = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+            hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) == hipSuccess && coop &&
+            decode_stack_supported(hidden, ffn, kv_dim, head_dim, sum_order, cus)) {
+            d->grid = cus;
+            std::vector<StackLayer> host_table(layers);
+            for (size_t l = 0; l < layers; ++l)
+                for (int p = 0; p < 7; ++p) {
+                    host_table[l].w[p] = d->proj[l * 7 + p]->tiled;
+                    host_table[l].w_scale[p] = d->proj[l * 7 + p]->w_scale;
+                }
+            dev_alloc(&d->table, sizeof(StackLayer) * layers);
+            dev_alloc(&d->flags, sizeof(unsigned) * ((size_t)cus + 1));
+            dev_alloc(&d->ring, sizeof(float) * layers * decode_stack_ring_stride(hidden, ffn, kv_dim));
+            if (rc == BITNET_HIP_OK) {
+                hipError_t e = hipMemcpy(d->table, host_table.data(), sizeof(StackLayer) * layers, hipMemcpyHostToDevice);
+                if (e == hipSuccess) e = hipMemset(d->flags, 0, sizeof(unsigned) * ((size_t)cus + 1));
+                if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void **>(&d->host_status), sizeof(unsigned), hipHostMallocMapped);
+                if (e == hipSuccess) { *d->host_status = 0; d->single_launch = true; }
+                else rc = fail(BITNET_HIP_DEVICE_ERROR, "decoder_create: single-launch set-up failed: %s", hipGetErrorString(e));
+            }
+        }
     }
     if (rc != BITNET_HIP_OK) {
         delete d;
@@ -727,6 +764,30 @@ int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin
     const size_t H = dec->hidden, F = dec->ffn, KV = dec->kv_heads * dec->head_dim;
     const size_t group = dec->q_heads / dec->kv_heads;
     int rc = BITNET_HIP_OK;
+    if (dec->host_status && *dec->host_status != 0)
+        return fail(BITNET_HIP_KERNEL_ERROR, "decoder_decode: an earlier single-launch decode gave up at a grid barrier");
+    auto aligned16 = [](const void *p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(s, &capturing);
+    if (m == 1 && dec->single_launch && dec->single_launch_enabled && capturing == hipStreamCaptureStatusNone &&
+        layer_end - layer_begin <= decode_stack_max_layers() &&
+        aligned16(x_in) && aligned16(x_out) && aligned16(q_last) && aligned16(k_last)) {
+        StackParams sp;
+        sp.table = dec->table; sp.layer_begin = (int)layer_begin; sp.layer_end = (int)layer_end;
+        sp.step_begin = 0; sp.step_end = 4 * (int)(layer_end - layer_begin);
+        sp.x_in = x_in; sp.x_out = x_out; sp.ring = dec->ring;
+        sp.ring_stride = (int)decode_stack_ring_stride(H, F, KV);
+        sp.q_last = q_last; sp.k_last = k_last; sp.gamma = dec->gamma;
+        sp.hidden = (int)H; sp.ffn = (int)F; sp.kv_dim = (int)KV; sp.head_dim = (int)dec->head_dim; sp.gqa_group = (int)group;
+        sp.eps = dec->eps;
+        sp.flags = dec->flags; sp.abort_word = dec->flags + dec->grid; sp.host_status = dec->host_status;
+        sp.spin_limit = 0;
+        std::lock_guard<std::mutex> guard(dec->stack_lock);
+        sp.epoch0 = dec->epoch;
+        rc = launch_decode_stack(sp, dec->grid, s);
+        if (rc == BITNET_HIP_OK) dec->epoch += (unsigned)(4 * (layer_end - layer_begin) - 1);
+        return rc;
+    }
     // one launch group: `count` projections reading the same (transformed) input
     auto run = [&](bitnet_hip_bitlinear *const *layers, int count, const float *x, const float *x2, size_t ldx, int mode,
                    const float *gamma, const float *res0, float *const *outs) {
@@ -753,6 +814,13 @@ int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin
         x = x2;
     }
     return rc;
+}
+
+int bitnet_hip_decoder_set_single_launch(bitnet_hip_decoder *dec, int enabled)
+{
+    if (!dec) return fail(BITNET_HIP_NULL_POINTER, "decoder_set_single_launch: null argument");
+    dec->single_launch_enabled = enabled != 0;
+    return dec->single_launch ? 1 : 0;
 }
 
 int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t m, float *x_out, float *q_last,

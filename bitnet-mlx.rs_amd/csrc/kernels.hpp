@@ -63,4 +63,33 @@ int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_su
                       int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,
                       const float *residual, float *out, hipStream_t stream);
 
+// decode_stack.hip: the projections of a run of decoder blocks at one token in a single cooperative launch
+struct StackLayer {  // one block: re-tiled weights and scales of q, k, v, o, gate, up, down (BITNET_HIP_PROJ_*)
+    const uint8_t *w[7];
+    const float *w_scale[7];
+};
+struct StackParams {
+    const StackLayer *table;  // [layers], device memory
+    int layer_begin, layer_end;
+    int step_begin, step_end;  // steps of the launch, 4 per block, counted from block layer_begin's first
+    const float *x_in;
+    float *x_out;
+    float *ring;              // [layers][ring_stride]: per block q | k | v | x1 | gate | up | x_next
+    int ring_stride;          // floats
+    float *q_last, *k_last;   // optional destinations of the last block's q and k
+    const float *gamma;       // [layers][2][hidden]
+    int hidden, ffn, kv_dim, head_dim, gqa_group;
+    float eps;
+    unsigned *flags;          // [grid] barrier flags, monotonic epochs
+    unsigned *abort_word;     // device; set when a workgroup gave up waiting
+    unsigned *host_status;    // host-mapped copy of the same fact
+    unsigned epoch0;          // epoch of the last barrier of the previous launch
+    long long spin_limit;
+    int lds_row_bytes;        // set by the launcher
+};
+bool decode_stack_supported(size_t hidden, size_t ffn, size_t kv_dim, size_t head_dim, int sum_order, int grid);
+size_t decode_stack_max_layers();  // blocks one launch can take
+size_t decode_stack_ring_stride(size_t hidden, size_t ffn, size_t kv_dim);
+int launch_decode_stack(const StackParams &params, int grid, hipStream_t stream);
+
 }  // namespace bitnet

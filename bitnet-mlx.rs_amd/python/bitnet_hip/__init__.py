@@ -105,6 +105,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_bitlinear_forward_multi": (i32, [C.POINTER(vp), sz, vp, sz, vp, f32, i32, C.POINTER(vp), vp, sz, vp]),
         "bitnet_hip_bitlinear_matmul": (i32, [vp, vp, vp, sz, vp, vp, vp, vp, vp]),
         "bitnet_hip_decoder_decode_layers": (i32, [vp, sz, sz, vp, sz, vp, vp, vp, vp]),
+        "bitnet_hip_decoder_set_single_launch": (i32, [vp, i32]),
         "bitnet_hip_decoder_create": (i32, [sz, sz, sz, sz, sz, sz, f32, i32, sz, C.POINTER(vp)]),
         "bitnet_hip_decoder_destroy": (None, [vp]),
         "bitnet_hip_decoder_projection": (i32, [vp, sz, i32, C.POINTER(vp)]),
@@ -469,6 +470,14 @@ class DecoderProjections:
 
     def weight_bytes(self) -> int:
         return load_library().bitnet_hip_decoder_weight_bytes(self._h)
+
+    def set_single_launch(self, enabled: bool) -> bool:
+        """Turn the one-cooperative-launch path for one-token decode on or off (default off); returns whether this
+        decoder has it."""
+        rc = load_library().bitnet_hip_decoder_set_single_launch(self._h, int(enabled))
+        if rc < 0:
+            _check(-rc)
+        return rc == 1
 
     def decode(self, x: torch.Tensor, out: Optional[torch.Tensor] = None, want_qk: bool = False, stream=None,
                layers: Optional[Sequence[int]] = None):

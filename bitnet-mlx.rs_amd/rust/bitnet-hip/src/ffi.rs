@@ -100,4 +100,5 @@ extern "C" {
     pub fn bitnet_hip_decoder_decode_layers(dec: *mut bitnet_hip_decoder, layer_begin: usize, layer_end: usize,
                                             x_in: *const f32, m: usize, x_out: *mut f32, q_last: *mut f32,
                                             k_last: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_decoder_set_single_launch(dec: *mut bitnet_hip_decoder, enabled: c_int) -> c_int;
 }

@@ -259,6 +259,17 @@ int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t
 int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin, size_t layer_end,
                                      const float *x_in, size_t m, float *x_out, float *q_last, float *k_last,
                                      void *stream);
+/* Optional at one token: the blocks' projections as ONE cooperative launch with barriers across the grid in
+ * place of launch boundaries (same results, bit for bit), for shapes that fit and up to 32 blocks per call.  Off
+ * by default: on MI355X a barrier across the eight XCDs costs about what a kernel boundary costs, so the path
+ * only matches the launch-per-group one (about 5 % faster over a 30-block stack, slower for single blocks
+ * because a cooperative launch is dearer to start).  It is ignored with more than one token and while the
+ * stream is being captured into a graph.  enabled = 1 turns it on, 0 off.  Returns 1 if the path is available
+ * for this decoder, 0 if not, a negative status on error.  A wait at a grid barrier that exceeds 50 ms is
+ * abandoned by every workgroup; the next decode call on the decoder then fails with BITNET_HIP_KERNEL_ERROR.
+ * (The reference runs its blocks layer by layer, bitnet-inference/src/engine/transformer_layers.rs:626-710; this
+ * switch only selects how the same work is issued.) */
+int bitnet_hip_decoder_set_single_launch(bitnet_hip_decoder *dec, int enabled);
 
 #ifdef __cplusplus
 }

@@ -560,6 +560,37 @@ def test_decoder_stack_small_bit_exact(layers):
     assert ei.value.kind == "ShapeMismatch"
 
 
+@pytest.mark.parametrize("dims,layers", [((2560, 6912, 20, 5, 128), 4), ((256, 512, 4, 2, 64), 3),
+                                         ((1024, 2816, 8, 8, 128), 2)])
+def test_decoder_single_launch_matches_oracle_and_per_launch_path(dims, layers):
+    """One token: the whole run of blocks as one cooperative launch (grid barriers between the steps) gives the
+    oracle's bits, the same as the (default) launch-per-step path; repeated calls, sub-ranges of blocks and
+    in-place hidden states included."""
+    rng = np.random.default_rng(layers + dims[0])
+    dec, ref = build_decoder(rng, layers, *dims, max_tokens=2)
+    assert dec.set_single_launch(True), "the single-launch path should be available at these shapes"
+    x = synth_activations(rng, 1, dims[0])
+    x_ref, q_ref, k_ref = oracle_stack(ref, x, *dims)
+    for _ in range(3):  # the barrier epochs keep growing from call to call
+        out, q, k = dec.decode(dev(x), want_qk=True)
+        assert np.array_equal(host(out), x_ref)
+        assert np.array_equal(host(q), q_ref) and np.array_equal(host(k), k_ref)
+    dec.set_single_launch(False)
+    out2, q2, k2 = dec.decode(dev(x), want_qk=True)
+    assert np.array_equal(host(out2), x_ref) and np.array_equal(host(q2), q_ref) and np.array_equal(host(k2), k_ref)
+    dec.set_single_launch(True)
+    # blocks 1 .. layers-1 only, hidden state updated in place
+    x1_ref = oracle_stack(ref[:1], x, *dims)[0]
+    buf = dev(x1_ref.copy())
+    dec.decode(buf, out=buf, layers=(1, layers))
+    assert np.array_equal(host(buf), x_ref)
+    # one block at a time, as the benchmark does
+    cur = dev(x)
+    for l in range(layers):
+        cur = dec.decode(cur, layers=(l, l + 1))
+    assert np.array_equal(host(cur), x_ref)
+
+
 # ---- C++ host mirror -----------------------------------------------------------------------------------------
 
 def test_cpp_host_mirror_selftest():
