@@ -192,15 +192,6 @@ __device__ __forceinline__ void prefetch(const Phase &P, uint4 (&wreg)[SLOTS])
     }
 }
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for every global load in
-// flight, that is for the weight tiles requested ahead of time, at each of the barriers of a step.
-__device__ __forceinline__ void lds_barrier()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 // Device-scope (write-through) store: visible to the other XCDs once acknowledged.
 __device__ __forceinline__ void store_device_scope(float *ptr, float v)
 {

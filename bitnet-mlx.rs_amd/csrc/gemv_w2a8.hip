@@ -275,6 +275,127 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
     }
 }
 
+// One token, f32 input: the quantiser runs in the prologue (see the head of this file).  Every load of the
+// workgroup - input row, RMSNorm weights, all of its weight tiles - is issued up front and unconditionally
+// (indices past the end are clamped and the values discarded), in the order in which the data is needed.  Loads
+// return in issue order, so the compiler can wait for "all but the last n" and the weight tiles stay in
+// flight while the row is normalised and quantised; the workgroup barriers order LDS traffic only, for the same
+// reason.  NCH: 16-byte chunks of the row per thread, and weight tiles per wavefront (k <= 1024 * NCH).
+template <int MODE, bool NORM, int NCH>
+__global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
+{
+    extern __shared__ uint4 lds_a[];  // int8 activations, 16 per uint4, zero past K
+    __shared__ int red[4][TILE_ROWS];
+    __shared__ float red_f[2][4];
+    __shared__ int red_i[4];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int chunks = p.k >> 2, lds_words = p.kt_count * 64;
+
+    int pj = 0;
+#pragma unroll
+    for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
+        if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
+    const GemvProjDev &P = p.proj[pj];
+    const int rb = (int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0);
+    const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + (size_t)rb * p.kt_count * 64 + lane;
+
+    float4 v[NCH], gm[NCH];
+    uint4 wt[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int c = min(tid + 256 * i, chunks - 1);
+        v[i] = load_chunk<MODE, true>(p.src, 0, c);
+    }
+    if constexpr (NORM) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) gm[i] = load_gamma_chunk(p.src, min(tid + 256 * i, chunks - 1), true);
+    }
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) wt[u] = tiles[(size_t)min(wave + 4 * u, p.kt_count - 1) * 64];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+        if (tid + 256 * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+    // thread tid is virtual lane tid of the declared summation order
+    RowDivisor rdiv = {1.0f, 1.0f, false};
+    if constexpr (NORM) {
+        float ss;
+        if (p.src.sum_order == BITNET_HIP_SUM_SEQUENTIAL) {
+            ss = sum_squares_sequential<MODE>(p.src, 0);
+        } else {
+            float part = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) part = sum_squares4(part, v[i]);
+            part = wave_sum_f32(part);
+            if (lane == 0) red_f[0][wave] = part;
+            lds_barrier();
+            ss = f32_add(f32_add(f32_add(red_f[0][0], red_f[0][1]), red_f[0][2]), red_f[0][3]);
+        }
+        rdiv = make_row_divisor(rms_from_ss(ss, p.k, p.src.eps));
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        if (NORM && tid + 256 * i < chunks) v[i] = normalize4(v[i], rdiv, gm[i]);
+        amax = absmax4(amax, v[i]);
+    }
+    amax = wave_max_f32(amax);
+    if (lane == 0) red_f[1][wave] = amax;
+    lds_barrier();
+    amax = fmaxf(fmaxf(red_f[1][0], red_f[1][1]), fmaxf(red_f[1][2], red_f[1][3]));
+    const float scale = scale_from_absmax(amax);
+    uint32_t *lds_w = reinterpret_cast<uint32_t *>(lds_a);
+    int isum = 0;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int c = tid + 256 * i;
+        if (c < chunks) {
+            const uint32_t packed = quant4_packed(v[i], scale, &isum);
+            lds_w[c] = packed;
+            if (p.q_out && blockIdx.x == 0) reinterpret_cast<uint32_t *>(p.q_out)[c] = packed;
+        } else if (c < lds_words) {
+            lds_w[c] = 0;
+        }
+    }
+    isum = wave_sum_i32(isum);
+    if (lane == 0) red_i[wave] = isum;
+    lds_barrier();
+
+    int acc = 0;
+    const int kq = lane >> 4;  // lane group: columns 64t + 16kq .. +15 of each tile, t = 0..3
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) {
+        const int kt = wave + 4 * u;
+        if (kt < p.kt_count) acc = dot64(wt[u], lds_a + kt * 16 + kq, acc);
+    }
+    // the four lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 32, 64);
+    if (lane < TILE_ROWS) red[wave][lane] = acc;
+    lds_barrier();
+
+    if (tid < TILE_ROWS) {
+        const int n = rb * TILE_ROWS + tid;
+        const int asum = red_i[0] + red_i[1] + red_i[2] + red_i[3];
+        if (blockIdx.x == 0 && tid == 0) {
+            if (p.a_scale_out) p.a_scale_out[0] = scale;
+            if (p.a_sum_out) p.a_sum_out[0] = asum;
+        }
+        if (n < P.n) {
+            const int total = red[0][tid] + red[1][tid] + red[2][tid] + red[3][tid] - asum;
+            if (P.acc) P.acc[n] = total;
+            if (P.out) {
+                float y = f32_mul((float)total, *P.w_scale);
+                y = f32_div(y, scale);
+                if (P.bias) y = f32_add(y, P.bias[n]);
+                if (P.residual) y = f32_add(y, P.residual[n]);
+                P.out[n] = y;
+            }
+        }
+    }
+}
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 struct GemvMfmaParams {
@@ -484,6 +605,20 @@ int launch_mode(const GemvParams &p, hipStream_t stream)
     return launch_mb_mode<1, MODE>(p, stream);  // one token row per launch; 2..16 rows take gemv_mfma_kernel
 }
 
+template <int MODE>
+int launch_fused_mode(const GemvParams &p, hipStream_t stream)
+{
+    const size_t lds = (size_t)p.kt_count * 16 * sizeof(uint4);
+    const dim3 grid((unsigned)p.proj[p.nproj - 1].rb_end);
+    const bool norm = p.src.gamma != nullptr, small = p.k <= 3 * 1024;
+    if (norm && small) hipLaunchKernelGGL((gemv_fused_kernel<MODE, true, 3>), grid, dim3(256), lds, stream, p);
+    else if (norm) hipLaunchKernelGGL((gemv_fused_kernel<MODE, true, FUSED_NCH>), grid, dim3(256), lds, stream, p);
+    else if (small) hipLaunchKernelGGL((gemv_fused_kernel<MODE, false, 3>), grid, dim3(256), lds, stream, p);
+    else hipLaunchKernelGGL((gemv_fused_kernel<MODE, false, FUSED_NCH>), grid, dim3(256), lds, stream, p);
+    BITNET_HIP_CHECK_LAUNCH("gemv_fused_kernel");
+    return BITNET_HIP_OK;
+}
+
 int fill_projs(GemvParams &p, const GemvProj *projs, int nproj, size_t t0, size_t k)
 {
     int rb_end = 0;
@@ -600,9 +735,9 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
     p.src.sum_order = sum_order; p.src.eps = eps;
     p.q_out = q_out; p.a_scale_out = a_scale_out; p.a_sum_out = a_sum_out;
     switch (input_mode) {
-        case BITNET_HIP_INPUT_PLAIN: return launch_mode<BITNET_HIP_INPUT_PLAIN>(p, stream);
-        case BITNET_HIP_INPUT_RELU2_MUL: return launch_mode<BITNET_HIP_INPUT_RELU2_MUL>(p, stream);
-        default: return launch_mode<BITNET_HIP_INPUT_GQA_BROADCAST>(p, stream);
+        case BITNET_HIP_INPUT_PLAIN: return launch_fused_mode<BITNET_HIP_INPUT_PLAIN>(p, stream);
+        case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused_mode<BITNET_HIP_INPUT_RELU2_MUL>(p, stream);
+        default: return launch_fused_mode<BITNET_HIP_INPUT_GQA_BROADCAST>(p, stream);
     }
 }
 

@@ -27,6 +27,15 @@
 
 namespace bitnet {
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load in flight,
+// which would stall a kernel that requests its weight tiles ahead of the code that needs them.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 struct RowSource {
     const float *x;      // [m, ldx]
     const float *x2;     // second operand of RELU2_MUL
