@@ -58,12 +58,12 @@ def time_events(torch, fn):
     return start.elapsed_time(stop)
 
 
-LAUNCHES_PER_STEP = 4  # q+k+v | o | gate+up | down, each one gemv_tiled_kernel<1, MODE> launch
+LAUNCHES_PER_STEP = 4  # q+k+v | o | gate+up | down, each one gemv_fused_kernel<MODE, NORM, NCH> launch
 # HBM bytes per launch of that kernel from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (two runs of this
 # script with --no-extras --calibration-copy), each scaled by what the same counter reads for the plain
 # 256 MiB copy: FETCH_SIZE reads 0.5 KiB per KiB fetched (factor 2.0), WRITE_SIZE 1.0 (factor 1.0).
 # Summary: profiles/decode_layer_b1_gemv_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_778_957
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_701_875
 
 
 def decode_roofline(event_ms, steps):
@@ -73,7 +73,7 @@ def decode_roofline(event_ms, steps):
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-        "kernel": "gemv_tiled_kernel<1, MODE> (decode GEMV, activation quantiser in the prologue)",
+        "kernel": "gemv_fused_kernel<MODE, NORM, NCH> (decode GEMV, activation quantiser in the prologue)",
         "launches": launches, "avg_launch_us": round(event_ms * 1e3 / launches, 3),
         "bytes_per_launch": LAYER_BYTES // LAUNCHES_PER_STEP,
         "how": "HIP events on the launch stream around the timed region, which holds only this kernel "
@@ -123,7 +123,12 @@ def prefill_rates(bh, torch, dec, gen, reps):
         ms = time_events(torch, lambda: [bl.matmul_quantized(a, a_scale, out=out, a_sum=a_sum) for _ in range(reps)]) / reps
         tops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
         res[name] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
-        del a, out
+        # the whole BitLinear forward on f32 activations (absmax int8 quantiser + GEMM + scale epilogue), for reference
+        x = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32)
+        bl.forward(x)
+        fwd_ms = time_events(torch, lambda: [bl.forward(x) for _ in range(reps)]) / reps
+        res[name]["forward_f32_in_ms"] = round(fwd_ms, 4)
+        del a, out, x
     return res
 
 
@@ -203,6 +208,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=60)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip roofline / prefill / CPU legs (profiling runs)")
+    ap.add_argument("--only-prefill", type=int, default=0, metavar="REPS",
+                    help="run only the two M=2048 prefill GEMMs REPS times each and print their rates (profiling runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -218,6 +225,9 @@ def main():
 
     bh.init(0)
     dec, gen = build_stack(bh, torch, LAYERS)
+    if args.only_prefill > 0:
+        print(json.dumps({"prefill": prefill_rates(bh, torch, dec, gen, reps=args.only_prefill)}))
+        return
     x = torch.randn((1, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
 
     def step(i):

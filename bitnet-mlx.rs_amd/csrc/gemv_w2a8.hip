@@ -408,7 +408,10 @@ struct GemvMfmaParams {
     int kt_count;
 };
 
-template <int RB>
+// FAST: k is a multiple of 256 and the activations are 16-byte aligned.  Every load is then unconditional
+// (indices past the end are clamped, the values discarded), so the compiler can count the loads in flight
+// and the next batch of tiles really stays outstanding while the current one is multiplied.
+template <int RB, bool FAST>
 __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 {
     __shared__ int red[3][RB][64][4];  // partial accumulators of wavefronts 1..3
@@ -432,6 +435,10 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
     const bool a_vec = (p.k % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0);
     const int8_t *arow = p.a + (size_t)(row_ok ? lr : 0) * p.k + lg * 16;
     auto load_a = [&](int kt, int t) -> v4i {
+        if constexpr (FAST) {
+            const v4i v = *reinterpret_cast<const v4i *>(arow + min(kt, p.kt_count - 1) * TILE_K + t * 64);
+            return row_ok ? v : (v4i){0, 0, 0, 0};
+        }
         v4i v = (v4i){0, 0, 0, 0};
         const int col = kt * TILE_K + t * 64 + lg * 16;
         if (row_ok && col < p.k) {
@@ -451,8 +458,11 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             const int rb = rb0 + r;
-            w[r] = rb < rb_count ? wbase[((size_t)rb * p.kt_count + kt) * 64]
-                                 : make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
+            if constexpr (FAST)  // results of row blocks past the end are never stored
+                w[r] = wbase[((size_t)min(rb, rb_count - 1) * p.kt_count + min(kt, p.kt_count - 1)) * 64];
+            else
+                w[r] = rb < rb_count ? wbase[((size_t)rb * p.kt_count + kt) * 64]
+                                     : make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
         }
     };
 
@@ -470,7 +480,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
             const int kt = kt0 + 4 * u;
-            if (kt < p.kt_count) {
+            if (FAST || kt < p.kt_count) {
                 load_w(kt, w[u]);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) a[u][t] = load_a(kt, t);
@@ -522,7 +532,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 #pragma unroll
             for (int i = 0; i < 4; ++i) red[wave - 1][r][lane][i] = acc[r][i];
     }
-    __syncthreads();
+    lds_barrier();
     if (wave == 0) {
         const float ws = P.out ? *P.w_scale : 0.0f;
 #pragma unroll
@@ -656,7 +666,10 @@ int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const floa
     for (int j = nproj; j < GEMV_MAX_PROJ; ++j) p.proj[j] = p.proj[nproj - 1];
     p.nproj = nproj; p.a = a; p.a_scale = a_scale; p.m = (int)m; p.k = (int)k; p.kt_count = (int)k_tiles(k);
     if (end == 0) return BITNET_HIP_OK;
-    hipLaunchKernelGGL((gemv_mfma_kernel<RB>), dim3((unsigned)end), dim3(256), 0, stream, p);
+    if (k % TILE_K == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0)
+        hipLaunchKernelGGL((gemv_mfma_kernel<RB, true>), dim3((unsigned)end), dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL((gemv_mfma_kernel<RB, false>), dim3((unsigned)end), dim3(256), 0, stream, p);
     BITNET_HIP_CHECK_LAUNCH("gemv_mfma_kernel");
     return BITNET_HIP_OK;
 }
