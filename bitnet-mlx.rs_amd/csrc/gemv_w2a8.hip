@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
 #pragma unroll
     for (int u = 0; u < GEMV_PREFETCH; ++u) {
         int kt = wave + 4 * u;
-        wbuf[u] = kt < p.kt_count ? tiles[(size_t)kt * 64 + lane] : make_uint4(0, 0, 0, 0);
+        wbuf[u] = tiles[(size_t)min(kt, p.kt_count - 1) * 64 + lane];  // unconditional: the waits can be counted
     }
 
     if constexpr (MODE == MODE_PREQUANT) {
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
 #pragma unroll
         for (int u = 0; u < GEMV_PREFETCH; ++u) {
             int kt = kt0 + 4 * (GEMV_PREFETCH + u);
-            wnext[u] = kt < p.kt_count ? tiles[(size_t)kt * 64 + lane] : make_uint4(0, 0, 0, 0);
+            wnext[u] = tiles[(size_t)min(kt, p.kt_count - 1) * 64 + lane];
         }
 #pragma unroll
         for (int u = 0; u < GEMV_PREFETCH; ++u) {
@@ -281,11 +281,11 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
 // return in issue order, so the compiler can wait for "all but the last n" and the weight tiles stay in
 // flight while the row is normalised and quantised; the workgroup barriers order LDS traffic only, for the same
 // reason.  NCH: 16-byte chunks of the row per thread, and weight tiles per wavefront (k <= 1024 * NCH).
-template <int MODE, bool NORM, int NCH>
+template <int MODE, bool NORM, int NCH, int RBW>
 __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
 {
     extern __shared__ uint4 lds_a[];  // int8 activations, 16 per uint4, zero past K
-    __shared__ int red[4][TILE_ROWS];
+    __shared__ int red[4][RBW][TILE_ROWS];
     __shared__ float red_f[2][4];
     __shared__ int red_i[4];
 
@@ -297,11 +297,12 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
     for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
         if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
     const GemvProjDev &P = p.proj[pj];
-    const int rb = (int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0);
-    const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + (size_t)rb * p.kt_count * 64 + lane;
+    const int rb0 = ((int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0)) * RBW;  // rb_end counts groups of RBW row blocks
+    const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
+    const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + lane;
 
     float4 v[NCH], gm[NCH];
-    uint4 wt[NCH];
+    uint4 wt[RBW][NCH];
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
         const int c = min(tid + 256 * i, chunks - 1);
@@ -312,7 +313,10 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
         for (int i = 0; i < NCH; ++i) gm[i] = load_gamma_chunk(p.src, min(tid + 256 * i, chunks - 1), true);
     }
 #pragma unroll
-    for (int u = 0; u < NCH; ++u) wt[u] = tiles[(size_t)min(wave + 4 * u, p.kt_count - 1) * 64];
+    for (int r = 0; r < RBW; ++r)
+#pragma unroll
+        for (int u = 0; u < NCH; ++u)  // row blocks past the end repeat the last one; their results are not stored
+            wt[r][u] = tiles[((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 4 * u, p.kt_count - 1)) * 64];
 #pragma unroll
     for (int i = 0; i < NCH; ++i)
         if (tid + 256 * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -362,28 +366,32 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
     if (lane == 0) red_i[wave] = isum;
     lds_barrier();
 
-    int acc = 0;
     const int kq = lane >> 4;  // lane group: columns 64t + 16kq .. +15 of each tile, t = 0..3
 #pragma unroll
-    for (int u = 0; u < NCH; ++u) {
-        const int kt = wave + 4 * u;
-        if (kt < p.kt_count) acc = dot64(wt[u], lds_a + kt * 16 + kq, acc);
+    for (int r = 0; r < RBW; ++r) {
+        int acc = 0;
+#pragma unroll
+        for (int u = 0; u < NCH; ++u) {
+            const int kt = wave + 4 * u;
+            if (kt < p.kt_count) acc = dot64(wt[r][u], lds_a + kt * 16 + kq, acc);
+        }
+        // the four lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
+        acc += __shfl_xor(acc, 16, 64);
+        acc += __shfl_xor(acc, 32, 64);
+        if (lane < TILE_ROWS) red[wave][r][lane] = acc;
     }
-    // the four lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
-    if (lane < TILE_ROWS) red[wave][lane] = acc;
     lds_barrier();
 
-    if (tid < TILE_ROWS) {
-        const int n = rb * TILE_ROWS + tid;
+    if (tid < TILE_ROWS * RBW) {
+        const int r = tid >> 4, row = tid & 15;
+        const int n = (rb0 + r) * TILE_ROWS + row;
         const int asum = red_i[0] + red_i[1] + red_i[2] + red_i[3];
         if (blockIdx.x == 0 && tid == 0) {
             if (p.a_scale_out) p.a_scale_out[0] = scale;
             if (p.a_sum_out) p.a_sum_out[0] = asum;
         }
         if (n < P.n) {
-            const int total = red[0][tid] + red[1][tid] + red[2][tid] + red[3][tid] - asum;
+            const int total = red[0][r][row] + red[1][r][row] + red[2][r][row] + red[3][r][row] - asum;
             if (P.acc) P.acc[n] = total;
             if (P.out) {
                 float y = f32_mul((float)total, *P.w_scale);
@@ -615,21 +623,22 @@ int launch_mode(const GemvParams &p, hipStream_t stream)
     return launch_mb_mode<1, MODE>(p, stream);  // one token row per launch; 2..16 rows take gemv_mfma_kernel
 }
 
-template <int MODE>
+template <int MODE, int RBW>
 int launch_fused_mode(const GemvParams &p, hipStream_t stream)
 {
     const size_t lds = (size_t)p.kt_count * 16 * sizeof(uint4);
     const dim3 grid((unsigned)p.proj[p.nproj - 1].rb_end);
     const bool norm = p.src.gamma != nullptr, small = p.k <= 3 * 1024;
-    if (norm && small) hipLaunchKernelGGL((gemv_fused_kernel<MODE, true, 3>), grid, dim3(256), lds, stream, p);
-    else if (norm) hipLaunchKernelGGL((gemv_fused_kernel<MODE, true, FUSED_NCH>), grid, dim3(256), lds, stream, p);
-    else if (small) hipLaunchKernelGGL((gemv_fused_kernel<MODE, false, 3>), grid, dim3(256), lds, stream, p);
-    else hipLaunchKernelGGL((gemv_fused_kernel<MODE, false, FUSED_NCH>), grid, dim3(256), lds, stream, p);
+    if (norm && small) hipLaunchKernelGGL((gemv_fused_kernel<MODE, true, 3, RBW>), grid, dim3(256), lds, stream, p);
+    else if (norm) hipLaunchKernelGGL((gemv_fused_kernel<MODE, true, FUSED_NCH, RBW>), grid, dim3(256), lds, stream, p);
+    else if (small) hipLaunchKernelGGL((gemv_fused_kernel<MODE, false, 3, RBW>), grid, dim3(256), lds, stream, p);
+    else hipLaunchKernelGGL((gemv_fused_kernel<MODE, false, FUSED_NCH, RBW>), grid, dim3(256), lds, stream, p);
     BITNET_HIP_CHECK_LAUNCH("gemv_fused_kernel");
     return BITNET_HIP_OK;
 }
 
-int fill_projs(GemvParams &p, const GemvProj *projs, int nproj, size_t t0, size_t k)
+// rbw: row blocks per workgroup (rb_end then counts groups of rbw row blocks, per projection)
+int fill_projs(GemvParams &p, const GemvProj *projs, int nproj, size_t t0, size_t k, int rbw = 1)
 {
     int rb_end = 0;
     for (int j = 0; j < nproj; ++j) {
@@ -639,7 +648,7 @@ int fill_projs(GemvParams &p, const GemvProj *projs, int nproj, size_t t0, size_
         d.residual = s.residual ? s.residual + t0 * s.n : nullptr;
         d.out = s.out ? s.out + t0 * s.n : nullptr;
         d.acc = s.acc ? s.acc + t0 * s.n : nullptr;
-        rb_end += (int)row_blocks(s.n);
+        rb_end += (int)((row_blocks(s.n) + rbw - 1) / rbw);
         d.rb_end = rb_end;
     }
     for (int j = nproj; j < GEMV_MAX_PROJ; ++j) p.proj[j] = p.proj[nproj - 1];
@@ -740,17 +749,29 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
                       int sum_order, int8_t *q_out, float *a_scale_out, int32_t *a_sum_out, hipStream_t stream)
 {
     if (m == 0 || nproj <= 0) return BITNET_HIP_OK;
+    // Every workgroup quantises the whole input row for itself, so launches with many row blocks give each
+    // workgroup two (short rows only: the tiles of both must fit its registers).
+    size_t blocks = 0;
+    for (int j = 0; j < nproj; ++j) blocks += row_blocks(projs[j].n);
+    const int rbw = (blocks > 512 && k <= 3 * 1024) ? 2 : 1;
     GemvParams p = {};
-    if (fill_projs(p, projs, nproj, 0, k) == 0) return BITNET_HIP_OK;
+    if (fill_projs(p, projs, nproj, 0, k, rbw) == 0) return BITNET_HIP_OK;
     p.m = (int)m;
     p.src.x = x; p.src.x2 = x2; p.src.gamma = gamma; p.src.ldx = ldx; p.src.k = (int)k;
     p.src.head_dim = (int)(head_dim ? head_dim : 1); p.src.gqa_group = (int)(gqa_group ? gqa_group : 1);
     p.src.sum_order = sum_order; p.src.eps = eps;
     p.q_out = q_out; p.a_scale_out = a_scale_out; p.a_sum_out = a_sum_out;
+    if (rbw == 2) {
+        switch (input_mode) {
+            case BITNET_HIP_INPUT_PLAIN: return launch_fused_mode<BITNET_HIP_INPUT_PLAIN, 2>(p, stream);
+            case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused_mode<BITNET_HIP_INPUT_RELU2_MUL, 2>(p, stream);
+            default: return launch_fused_mode<BITNET_HIP_INPUT_GQA_BROADCAST, 2>(p, stream);
+        }
+    }
     switch (input_mode) {
-        case BITNET_HIP_INPUT_PLAIN: return launch_fused_mode<BITNET_HIP_INPUT_PLAIN>(p, stream);
-        case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused_mode<BITNET_HIP_INPUT_RELU2_MUL>(p, stream);
-        default: return launch_fused_mode<BITNET_HIP_INPUT_GQA_BROADCAST>(p, stream);
+        case BITNET_HIP_INPUT_PLAIN: return launch_fused_mode<BITNET_HIP_INPUT_PLAIN, 1>(p, stream);
+        case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused_mode<BITNET_HIP_INPUT_RELU2_MUL, 1>(p, stream);
+        default: return launch_fused_mode<BITNET_HIP_INPUT_GQA_BROADCAST, 1>(p, stream);
     }
 }
 
