@@ -416,14 +416,15 @@ struct GemvMfmaParams {
     int kt_count;
 };
 
+// MT: groups of 16 token rows (m <= 16 * MT); a decoded weight dword then feeds MT MFMAs.
 // FAST: k is a multiple of 256 and the activations are 16-byte aligned.  Every load is then unconditional
 // (indices past the end are clamped, the values discarded), so the compiler can count the loads in flight
 // and the next batch of tiles really stays outstanding while the current one is multiplied.
-template <int RB, bool FAST>
+template <int RB, int MT, bool FAST>
 __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 {
-    __shared__ int red[3][RB][64][4];  // partial accumulators of wavefronts 1..3
-    __shared__ int red_sum[4][16];     // per wavefront: sum_k a[t, k] over its k-tiles
+    __shared__ int red[3][RB][MT][64][4];  // partial accumulators of wavefronts 1..3
+    __shared__ int red_sum[4][MT][16];     // per wavefront: sum_k a[t, k] over its k-tiles
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 15, lg = lane >> 4;
@@ -438,19 +439,25 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
     const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
     const uint4 *wbase = reinterpret_cast<const uint4 *>(P.w) + lane;
 
-    // A operand of this lane: token row lr, the 16 columns 64t + 16lg of each k-tile (rows past m read as zero)
-    const bool row_ok = lr < p.m;
+    // A operand of this lane in token group g: token row 16g + lr, the 16 columns 64t + 16lg of each k-tile
+    // (rows past m read as zero)
     const bool a_vec = (p.k % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0);
-    const int8_t *arow = p.a + (size_t)(row_ok ? lr : 0) * p.k + lg * 16;
-    auto load_a = [&](int kt, int t) -> v4i {
+    bool row_ok[MT];
+    const int8_t *arow[MT];
+#pragma unroll
+    for (int g = 0; g < MT; ++g) {
+        row_ok[g] = 16 * g + lr < p.m;
+        arow[g] = p.a + (size_t)(row_ok[g] ? 16 * g + lr : 0) * p.k + lg * 16;
+    }
+    auto load_a = [&](int g, int kt, int t) -> v4i {
         if constexpr (FAST) {
-            const v4i v = *reinterpret_cast<const v4i *>(arow + min(kt, p.kt_count - 1) * TILE_K + t * 64);
-            return row_ok ? v : (v4i){0, 0, 0, 0};
+            const v4i v = *reinterpret_cast<const v4i *>(arow[g] + min(kt, p.kt_count - 1) * TILE_K + t * 64);
+            return row_ok[g] ? v : (v4i){0, 0, 0, 0};
         }
         v4i v = (v4i){0, 0, 0, 0};
         const int col = kt * TILE_K + t * 64 + lg * 16;
-        if (row_ok && col < p.k) {
-            const int8_t *src = arow + kt * TILE_K + t * 64;
+        if (row_ok[g] && col < p.k) {
+            const int8_t *src = arow[g] + kt * TILE_K + t * 64;
             if (a_vec) {
                 v = *reinterpret_cast<const v4i *>(src);
             } else {
@@ -474,24 +481,30 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         }
     };
 
-    v4i acc[RB];
+    v4i acc[RB][MT];
+    int rowsum[MT];
 #pragma unroll
-    for (int r = 0; r < RB; ++r) acc[r] = (v4i){0, 0, 0, 0};
-    int rowsum = 0;
+    for (int g = 0; g < MT; ++g) {
+        rowsum[g] = 0;
+#pragma unroll
+        for (int r = 0; r < RB; ++r) acc[r][g] = (v4i){0, 0, 0, 0};
+    }
 
-    constexpr int PF = RB == 1 ? 4 : (RB == 2 ? 3 : 2);  // bounded by the register file
+    constexpr int PF = RB * MT == 1 ? 4 : (RB * MT == 2 ? 3 : (MT <= 2 ? 2 : 1));  // bounded by the register file
     // All loads of a batch of PF k-tiles are issued before the first MFMA of the batch, and the next
     // batch is requested while the current one is computed: the weight stream is what the kernel waits for.
     uint4 wcur[PF][RB], wnxt[PF][RB];
-    v4i acur[PF][4], anxt[PF][4];
-    auto load_batch = [&](int kt0, uint4 (&w)[PF][RB], v4i (&a)[PF][4]) {
+    v4i acur[PF][MT][4], anxt[PF][MT][4];
+    auto load_batch = [&](int kt0, uint4 (&w)[PF][RB], v4i (&a)[PF][MT][4]) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
             const int kt = kt0 + 4 * u;
             if (FAST || kt < p.kt_count) {
                 load_w(kt, w[u]);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) a[u][t] = load_a(kt, t);
+                for (int g = 0; g < MT; ++g)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) a[u][g][t] = load_a(g, kt, t);
             }
         }
     };
@@ -503,11 +516,14 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
             if (kt0 + 4 * u >= p.kt_count) continue;
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                const v4i af = acur[u][t];
-                rowsum = __builtin_amdgcn_sdot4(af[0], 0x01010101, rowsum, false);
-                rowsum = __builtin_amdgcn_sdot4(af[1], 0x01010101, rowsum, false);
-                rowsum = __builtin_amdgcn_sdot4(af[2], 0x01010101, rowsum, false);
-                rowsum = __builtin_amdgcn_sdot4(af[3], 0x01010101, rowsum, false);
+#pragma unroll
+                for (int g = 0; g < MT; ++g) {
+                    const v4i af = acur[u][g][t];
+                    rowsum[g] = __builtin_amdgcn_sdot4(af[0], 0x01010101, rowsum[g], false);
+                    rowsum[g] = __builtin_amdgcn_sdot4(af[1], 0x01010101, rowsum[g], false);
+                    rowsum[g] = __builtin_amdgcn_sdot4(af[2], 0x01010101, rowsum[g], false);
+                    rowsum[g] = __builtin_amdgcn_sdot4(af[3], 0x01010101, rowsum[g], false);
+                }
 #pragma unroll
                 for (int r = 0; r < RB; ++r) {
                     const uint4 w4 = wcur[u][r];
@@ -517,7 +533,9 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
                     bf[1] = (int)((wd >> 2) & 0x03030303u);
                     bf[2] = (int)((wd >> 4) & 0x03030303u);
                     bf[3] = (int)((wd >> 6) & 0x03030303u);
-                    acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf, acc[r], 0, 0, 0);
+#pragma unroll
+                    for (int g = 0; g < MT; ++g)
+                        acc[r][g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(acur[u][g][t], bf, acc[r][g], 0, 0, 0);
                 }
             }
         }
@@ -526,19 +544,26 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 #pragma unroll
             for (int r = 0; r < RB; ++r) wcur[u][r] = wnxt[u][r];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) acur[u][t] = anxt[u][t];
+            for (int g = 0; g < MT; ++g)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acur[u][g][t] = anxt[u][g][t];
         }
     }
 
-    // sum_k a[lr, k] over this wavefront's tiles: lanes lr, lr+16, lr+32, lr+48 hold the four column groups
-    rowsum += __shfl_xor(rowsum, 16, 64);
-    rowsum += __shfl_xor(rowsum, 32, 64);
-    if (lane < 16) red_sum[wave][lane] = rowsum;
+    // sum_k a[row, k] over this wavefront's tiles: lanes lr, lr+16, lr+32, lr+48 hold the four column groups
+#pragma unroll
+    for (int g = 0; g < MT; ++g) {
+        rowsum[g] += __shfl_xor(rowsum[g], 16, 64);
+        rowsum[g] += __shfl_xor(rowsum[g], 32, 64);
+        if (lane < 16) red_sum[wave][g][lane] = rowsum[g];
+    }
     if (wave > 0) {
 #pragma unroll
         for (int r = 0; r < RB; ++r)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) red[wave - 1][r][lane][i] = acc[r][i];
+            for (int g = 0; g < MT; ++g)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[wave - 1][r][g][lane][i] = acc[r][g][i];
     }
     lds_barrier();
     if (wave == 0) {
@@ -547,18 +572,22 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         for (int r = 0; r < RB; ++r) {
             const int n = (rb0 + r) * TILE_ROWS + lr;  // result register i of lane l is C[4*(l/16) + i][l mod 16]
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int t = lg * 4 + i;
-                if (n < P.n && t < p.m) {
-                    const int asum = red_sum[0][t] + red_sum[1][t] + red_sum[2][t] + red_sum[3][t];
-                    const int total = acc[r][i] + red[0][r][lane][i] + red[1][r][lane][i] + red[2][r][lane][i] - asum;
-                    const size_t o = (size_t)t * P.n + n;
-                    if (P.acc) P.acc[o] = total;
-                    if (P.out) {
-                        float v = f32_div(f32_mul((float)total, ws), p.a_scale[t]);
-                        if (P.bias) v = f32_add(v, P.bias[n]);
-                        if (P.residual) v = f32_add(v, P.residual[o]);
-                        P.out[o] = v;
+            for (int g = 0; g < MT; ++g) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int tl = lg * 4 + i, t = 16 * g + tl;
+                    if (n < P.n && t < p.m) {
+                        const int asum = red_sum[0][g][tl] + red_sum[1][g][tl] + red_sum[2][g][tl] + red_sum[3][g][tl];
+                        const int total = acc[r][g][i] + red[0][r][g][lane][i] + red[1][r][g][lane][i] +
+                                          red[2][r][g][lane][i] - asum;
+                        const size_t o = (size_t)t * P.n + n;
+                        if (P.acc) P.acc[o] = total;
+                        if (P.out) {
+                            float v = f32_div(f32_mul((float)total, ws), p.a_scale[t]);
+                            if (P.bias) v = f32_add(v, P.bias[n]);
+                            if (P.residual) v = f32_add(v, P.residual[o]);
+                            P.out[o] = v;
+                        }
                     }
                 }
             }
@@ -658,7 +687,7 @@ int fill_projs(GemvParams &p, const GemvProj *projs, int nproj, size_t t0, size_
     return rb_end;
 }
 
-template <int RB>
+template <int RB, int MT>
 int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const float *a_scale, size_t m, size_t k,
                    hipStream_t stream)
 {
@@ -676,9 +705,9 @@ int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const floa
     p.nproj = nproj; p.a = a; p.a_scale = a_scale; p.m = (int)m; p.k = (int)k; p.kt_count = (int)k_tiles(k);
     if (end == 0) return BITNET_HIP_OK;
     if (k % TILE_K == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0)
-        hipLaunchKernelGGL((gemv_mfma_kernel<RB, true>), dim3((unsigned)end), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((gemv_mfma_kernel<RB, MT, true>), dim3((unsigned)end), dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL((gemv_mfma_kernel<RB, false>), dim3((unsigned)end), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((gemv_mfma_kernel<RB, MT, false>), dim3((unsigned)end), dim3(256), 0, stream, p);
     BITNET_HIP_CHECK_LAUNCH("gemv_mfma_kernel");
     return BITNET_HIP_OK;
 }
@@ -699,16 +728,11 @@ int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const f
                       hipStream_t stream)
 {
     if (m == 0 || nproj <= 0) return BITNET_HIP_OK;
-    if (m >= 2 && m <= (size_t)GEMV_MFMA_MAX_M) {
-        // 2..16 tokens: the MFMA variant.  Workgroups take more row blocks when there are plenty of them, so that
-        // fewer workgroups re-read the activation matrix.
+    if (m >= 2) {
+        // Several tokens: the MFMA variant, up to 64 token rows per launch (more: in groups of 64).  Workgroups
+        // take more row blocks when there are plenty of them, so that fewer workgroups re-read the activations.
         size_t blocks = 0;
         for (int j = 0; j < nproj; ++j) blocks += row_blocks(projs[j].n);
-        if (blocks >= 800) return launch_mfma_rb<4>(projs, nproj, a, a_scale, m, k, stream);
-        if (blocks >= 400) return launch_mfma_rb<2>(projs, nproj, a, a_scale, m, k, stream);
-        return launch_mfma_rb<1>(projs, nproj, a, a_scale, m, k, stream);
-    }
-    if (m > 1) {  // more rows than one MFMA row block: in groups of 16
         for (size_t t0 = 0; t0 < m; t0 += (size_t)GEMV_MFMA_MAX_M) {
             GemvProj sub[GEMV_MAX_PROJ];
             const size_t rows = m - t0 < (size_t)GEMV_MFMA_MAX_M ? m - t0 : (size_t)GEMV_MFMA_MAX_M;
@@ -718,7 +742,14 @@ int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const f
                 if (sub[j].out) sub[j].out += t0 * sub[j].n;
                 if (sub[j].acc) sub[j].acc += t0 * sub[j].n;
             }
-            int rc = launch_mfma_rb<1>(sub, nproj, a + t0 * k, a_scale ? a_scale + t0 : nullptr, rows, k, stream);
+            const int8_t *a0 = a + t0 * k;
+            const float *s0 = a_scale ? a_scale + t0 : nullptr;
+            int rc;
+            if (rows > 32) rc = launch_mfma_rb<1, 4>(sub, nproj, a0, s0, rows, k, stream);
+            else if (rows > 16) rc = launch_mfma_rb<1, 2>(sub, nproj, a0, s0, rows, k, stream);
+            else if (blocks >= 800) rc = launch_mfma_rb<4, 1>(sub, nproj, a0, s0, rows, k, stream);
+            else if (blocks >= 400) rc = launch_mfma_rb<2, 1>(sub, nproj, a0, s0, rows, k, stream);
+            else rc = launch_mfma_rb<1, 1>(sub, nproj, a0, s0, rows, k, stream);
             if (rc != BITNET_HIP_OK) return rc;
         }
         return BITNET_HIP_OK;

@@ -32,8 +32,8 @@ int launch_untile(const uint8_t *tiled, size_t n, size_t k, uint8_t *packed, hip
 // gemv_w2a8.hip
 int launch_gemv_rowmajor(const uint8_t *packed, const int8_t *a, int32_t *out, size_t n, size_t k,
                          hipStream_t stream);
-constexpr int GEMV_MAX_M = 16;      // token rows the decode-GEMV path takes (more go to the prefill GEMM)
-constexpr int GEMV_MFMA_MAX_M = 16; // 2..16 rows use the MFMA variant of the decode GEMV
+constexpr int GEMV_MAX_M = 95;      // token rows the decode-GEMV path takes (more go to the prefill GEMM)
+constexpr int GEMV_MFMA_MAX_M = 64; // rows per launch of the MFMA variant of the decode GEMV (2 and more rows)
 constexpr int GEMV_MAX_PROJ = 3;  // projections sharing one input row per launch (q,k,v / gate,up)
 // One projection of a decode-GEMV launch: re-tiled weights [n, k], its scale, optional bias [n] and
 // residual [m, n]; out [m, n] f32 and acc [m, n] int32 are each optional.

@@ -257,8 +257,12 @@ def test_decode_gemv_bit_exact(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 1, 1), (1, 5, 7), (2, 17, 257), (3, 33, 100), (1, 16, 255), (4, 15, 512),
-                                   (1, 48, 16384), (8, 31, 3000)])
+                                   (1, 48, 16384), (8, 31, 3000), (17, 40, 512), (33, 100, 300), (48, 33, 768),
+                                   (65, 50, 512), (95, 170, 1024), (20, 7000, 256)])
 def test_decode_gemv_ragged_shapes(m, n, k):
+    """Token counts 1, 2..16, 17..32, 33..64 and 65..95 take different variants of the decode GEMV (dot-product
+    chain, MFMA with 1, 2 or 4 groups of 16 token rows, two launches); k a multiple of 256 or not selects the
+    unconditional-load variant or the bounds-checked one."""
     rng = np.random.default_rng(m + 10 * n + 100 * k)
     packed, ws, a, a_scale = make_problem(rng, m, n, k, full_range=True)
     tiled = bh.retile_weights(dev(packed), n, k)
@@ -291,7 +295,7 @@ def test_decode_gemv_extremes_and_identities():
     assert np.array_equal(host(r12), host(r1) + host(r2))
 
 
-@pytest.mark.parametrize("m", [16, 64])
+@pytest.mark.parametrize("m", [16, 24, 64])
 @pytest.mark.parametrize("n,k", [(6912, 2560), (2560, 6912)])
 def test_batched_decode_sweep_bit_exact(m, n, k):
     rng = np.random.default_rng(m + n)
