@@ -436,6 +436,46 @@ int bitnet_hip_bitlinear_set_weights_packed(bitnet_hip_bitlinear *layer, const u
     return BITNET_HIP_OK;
 }
 
+int bitnet_hip_bitlinear_set_weights_gguf(bitnet_hip_bitlinear *layer, const uint8_t *data, size_t len, size_t rows,
+                                          size_t cols, int layout, int on_device, float *scale_out, float *offset_out,
+                                          void *stream)
+{
+    if (!layer || !data) return fail(BITNET_HIP_NULL_POINTER, "set_weights_gguf: null argument");
+    if (layout != BITNET_HIP_LAYOUT_OUT_IN && layout != BITNET_HIP_LAYOUT_IN_OUT)
+        return fail(BITNET_HIP_INVALID_CONFIG, "set_weights_gguf: unknown layout %d", layout);
+    const size_t n = layer->out_features, k = layer->in_features;
+    const size_t er = layout == BITNET_HIP_LAYOUT_OUT_IN ? n : k, ec = layout == BITNET_HIP_LAYOUT_OUT_IN ? k : n;
+    if (rows != er || cols != ec) {
+        size_t e[2] = {er, ec}, a[2] = {rows, cols};
+        return fail_shape(e, 2, a, 2, "GGUF tensor dimensions");
+    }
+    const size_t codes = (n * k + 3) / 4, need = 8 + codes;
+    if (len < need) {
+        size_t e[1] = {need}, a[1] = {len};
+        return fail_shape(e, 1, a, 1, "Insufficient packed data (8-byte scale/offset header + 2-bit codes)");
+    }
+    hipStream_t s = as_stream(stream);
+    float header[2];  // little-endian host, as f32::from_le_bytes on the reference's targets
+    if (on_device) BITNET_HIP_TRY(hipMemcpy(header, data, 8, hipMemcpyDeviceToHost));
+    else memcpy(header, data, 8);
+    if (scale_out) *scale_out = header[0];
+    if (offset_out) *offset_out = header[1];
+    // the codes start 8 bytes into the tensor: stage them at an aligned device address, in their own orientation
+    DeviceTemp flat;
+    int rc = flat.alloc(codes);
+    if (rc != BITNET_HIP_OK) return rc;
+    std::unique_lock<std::shared_mutex> guard(layer->lock);
+    BITNET_HIP_TRY(hipMemcpyAsync(flat.ptr, data + 8, codes, on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, s));
+    BITNET_HIP_TRY(hipMemcpyAsync(layer->w_scale, &header[0], sizeof(float), hipMemcpyHostToDevice, s));
+    rc = launch_retile(static_cast<const uint8_t *>(flat.ptr), n, k, layout, layer->tiled, s);
+    if (rc != BITNET_HIP_OK) return rc;
+    rc = launch_untile(layer->tiled, n, k, layer->packed, s);  // canonical [out, in] bytes, code 3 stored as code 1
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipStreamSynchronize(s));
+    layer->has_weights = true;
+    return BITNET_HIP_OK;
+}
+
 int bitnet_hip_bitlinear_set_bias(bitnet_hip_bitlinear *layer, const float *bias, size_t len, int on_device, void *stream)
 {
     if (!layer || !bias) return fail(BITNET_HIP_NULL_POINTER, "set_bias: null argument");

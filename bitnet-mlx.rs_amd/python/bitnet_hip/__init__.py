@@ -98,6 +98,8 @@ def load_library() -> C.CDLL:
         "bitnet_hip_bitlinear_destroy": (None, [vp]),
         "bitnet_hip_bitlinear_set_weights_f32": (i32, [vp, vp, sz, sz, i32, i32, i32, f32, vp]),
         "bitnet_hip_bitlinear_set_weights_packed": (i32, [vp, vp, sz, f32, i32, vp]),
+        "bitnet_hip_bitlinear_set_weights_gguf": (i32, [vp, vp, sz, sz, sz, i32, i32, C.POINTER(C.c_float),
+                                                  C.POINTER(C.c_float), vp]),
         "bitnet_hip_bitlinear_set_bias": (i32, [vp, vp, sz, i32, vp]),
         "bitnet_hip_bitlinear_get_quantized": (i32, [vp, C.POINTER(f32), vp, sz]),
         "bitnet_hip_bitlinear_workspace_size": (sz, [vp, sz]),
@@ -344,6 +346,19 @@ class BitLinear:
             raise BitLinearError(INVALID_CONFIG, "packed weights must be contiguous u8")
         _check(load_library().bitnet_hip_bitlinear_set_weights_packed(self._h, _ptr(packed), packed.numel(), w_scale,
                                                                       int(packed.is_cuda), _stream(stream)))
+
+    def load_gguf_ternary(self, data: torch.Tensor, layout: int = LAYOUT_OUT_IN, stream=None):
+        """A GGUF BitnetB158 tensor (8-byte scale/offset header + 2-bit codes, GgufLoader::decode_ternary_weights,
+        gguf.rs:1089-1165) as a contiguous u8 tensor, host or device.  Returns (scale, offset) of the header."""
+        if data.dtype != torch.uint8 or not data.is_contiguous():
+            raise BitLinearError(INVALID_CONFIG, "GGUF tensor bytes must be contiguous u8")
+        n, k = self.config.out_features, self.config.in_features
+        rows, cols = (n, k) if layout == LAYOUT_OUT_IN else (k, n)
+        scale, offset = C.c_float(0), C.c_float(0)
+        _check(load_library().bitnet_hip_bitlinear_set_weights_gguf(self._h, _ptr(data), data.numel(), rows, cols, layout,
+                                                                    int(data.is_cuda), C.byref(scale), C.byref(offset),
+                                                                    _stream(stream)))
+        return scale.value, offset.value
 
     def update_bias(self, bias: torch.Tensor, stream=None):
         if bias.dtype != torch.float32 or not bias.is_contiguous():

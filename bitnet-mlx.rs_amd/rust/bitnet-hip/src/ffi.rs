@@ -69,6 +69,10 @@ extern "C" {
     pub fn bitnet_hip_bitlinear_set_weights_packed(layer: *mut bitnet_hip_bitlinear, packed: *const u8,
                                                    packed_len: usize, w_scale: f32, on_device: c_int,
                                                    stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_bitlinear_set_weights_gguf(layer: *mut bitnet_hip_bitlinear, data: *const u8, len: usize,
+                                                 rows: usize, cols: usize, layout: c_int, on_device: c_int,
+                                                 scale_out: *mut f32, offset_out: *mut f32,
+                                                 stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_bitlinear_set_bias(layer: *mut bitnet_hip_bitlinear, bias: *const f32, len: usize,
                                          on_device: c_int, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_bitlinear_get_quantized(layer: *mut bitnet_hip_bitlinear, w_scale: *mut f32, packed: *mut u8,

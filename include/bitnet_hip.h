@@ -178,6 +178,17 @@ int bitnet_hip_bitlinear_set_weights_f32(bitnet_hip_bitlinear *layer, const floa
  * BitLinearForward::forward_with_quantized_weights (forward.rs:46-50) / GGUF-decoded tensors. */
 int bitnet_hip_bitlinear_set_weights_packed(bitnet_hip_bitlinear *layer, const uint8_t *packed,
                                             size_t packed_len, float w_scale, int on_device, void *stream);
+/* A GGUF tensor of type BitnetB158 as GgufLoader::decode_ternary_weights reads it (bitnet-inference/src/gguf.rs:
+ * 1089-1165): 4 bytes scale (f32, little endian), 4 bytes offset (f32, little endian), then the 2-bit codes, 4 per
+ * byte, flat over a rows x cols matrix in `layout` orientation (BITNET_HIP_LAYOUT_IN_OUT for the transposed
+ * tensors of inference_integration.rs:431).  `data` is a HOST pointer (if on_device == 0) to the whole tensor,
+ * header included.  The header's scale becomes the layer's w_scale; scale and offset are also returned through
+ * scale_out / offset_out (either may be NULL).  Unlike the reference, which accepts any buffer of at least
+ * ceil(rows*cols/4) bytes and then silently decodes fewer elements, a buffer shorter than 8 + ceil(rows*cols/4)
+ * bytes is a SHAPE_MISMATCH ("Insufficient packed data", gguf.rs:1098-1102). */
+int bitnet_hip_bitlinear_set_weights_gguf(bitnet_hip_bitlinear *layer, const uint8_t *data, size_t len, size_t rows,
+                                          size_t cols, int layout, int on_device, float *scale_out,
+                                          float *offset_out, void *stream);
 /* BitLinear::update_bias (layer.rs:329-352): INVALID_CONFIG if the layer was created without bias. */
 int bitnet_hip_bitlinear_set_bias(bitnet_hip_bitlinear *layer, const float *bias, size_t len, int on_device,
                                   void *stream);

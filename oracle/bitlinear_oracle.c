@@ -12,6 +12,7 @@
  *
  * Parity status of each function (what pins it besides this restatement):
  *   orc_pack_2bit / orc_unpack_2bit      pinned: byte fixtures and round trips held by the reference's tests
+ *   orc_gguf_decode_ternary              pinned: the reference's own decode test (header + 0x24 -> [-1,0,1,-1])
  *   orc_round_clip, orc_ternarize_*      pinned: reference tables (round_clip ties, strict '>' threshold)
  *   orc_absmean                          pinned: reference vector [1,-2,3,-4] -> 2.5; order declared here
  *   orc_gemv_w2a8 / orc_gemm_w2a8        pinned: reference 3x4 GEMV / 2x3x2 GEMM vectors + brute force
@@ -317,6 +318,28 @@ void orc_unpack_2bit(const uint8_t *packed, size_t n, int8_t *q)
 {
     static const int8_t lut[4] = {-1, 0, 1, 0};
     for (size_t i = 0; i < n; ++i) q[i] = lut[(packed[i / 4] >> (2 * (i % 4))) & 3u];
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * GGUF tensor of type BitnetB158.   reference: bitnet-inference/src/gguf.rs:1089-1165
+ *   bytes 0..3 scale (f32, little endian), bytes 4..7 offset (f32, little endian), then the 2-bit codes of
+ *   P1, 4 per byte.  The reference accepts any buffer of at least ceil(count/4) bytes and strips the header
+ *   only when the buffer has 8 bytes or more (:1097-1121); elements whose code byte is missing are not
+ *   produced (its Vec is simply shorter, :1150).  Returns the number of elements decoded.
+ * ---------------------------------------------------------------------------------------------- */
+size_t orc_gguf_decode_ternary(const uint8_t *data, size_t len, size_t count, int8_t *q, float *scale, float *offset)
+{
+    static const int8_t lut[4] = {-1, 0, 1, 0};
+    *scale = 1.0f;
+    *offset = 0.0f;
+    if (len < (count + 3) / 4) return (size_t)-1; /* "Insufficient packed data" (:1098-1102) */
+    if (len >= 4) memcpy(scale, data, 4);         /* little-endian host assumed */
+    if (len >= 8) memcpy(offset, data + 4, 4);
+    const size_t start = len >= 8 ? 8 : 0;
+    size_t produced = 0;
+    for (size_t b = start; b < len && produced < count; ++b)
+        for (int j = 0; j < 4 && produced < count; ++j) q[produced++] = lut[(data[b] >> (2 * j)) & 3u];
+    return produced;
 }
 
 /* ------------------------------------------------------------------------------------------------

@@ -36,6 +36,7 @@ def lib() -> C.CDLL:
         _lib.orc_quantize_weights_reference.restype = C.c_float
         _lib.orc_pack_2bit.restype = C.c_size_t
         _lib.orc_packed_size.restype = C.c_size_t
+        _lib.orc_gguf_decode_ternary.restype = C.c_size_t
         _lib.cpu_baseline_max_threads.restype = C.c_int
         _lib.cpu_baseline_isa.restype = C.c_int
     return _lib
@@ -159,6 +160,18 @@ def unpack_2bit(packed, n):
     q = np.empty((n,), dtype=np.int8)
     lib().orc_unpack_2bit(_p(packed), _sz(n), _p(q))
     return q
+
+
+def gguf_decode_ternary(data, count):
+    """GgufLoader::decode_ternary_weights (gguf.rs:1089-1165): returns (q int8 [produced], scale, offset), or None
+    where the reference reports "Insufficient packed data"."""
+    data = np.ascontiguousarray(data, dtype=np.uint8)
+    q = np.empty((max(count, 1),), dtype=np.int8)
+    scale, offset = C.c_float(0), C.c_float(0)
+    got = lib().orc_gguf_decode_ternary(_p(data), _sz(data.size), _sz(count), _p(q), C.byref(scale), C.byref(offset))
+    if got == C.c_size_t(-1).value:
+        return None
+    return q[:got].copy(), scale.value, offset.value
 
 
 def gemm_w2a8(packed, a, n_out):

@@ -595,6 +595,39 @@ def test_decoder_single_launch_matches_oracle_and_per_launch_path(dims, layers):
     assert np.array_equal(host(cur), x_ref)
 
 
+@pytest.mark.parametrize("layout", [bh.LAYOUT_OUT_IN, bh.LAYOUT_IN_OUT])
+@pytest.mark.parametrize("n,k", [(1, 4), (48, 300), (640, 2560)])
+def test_gguf_ternary_tensor_ingestion(n, k, layout):
+    """A GGUF BitnetB158 tensor (8-byte header + 2-bit codes, either orientation, code 3 included) loaded straight
+    into the layer: the layer then holds what the reference's decoder yields, and its forward matches the oracle."""
+    rng = np.random.default_rng(n * 7 + k + layout)
+    codes = rng.integers(0, 4, size=(n, k)).astype(np.uint8)  # code 3 decodes to 0 (gguf.rs:1139)
+    if (n, k) == (1, 4):
+        codes = np.array([[0, 1, 2, 0]], np.uint8)  # the reference's test vector 0x24 (gguf.rs:2421-2436)
+    src = codes if layout == bh.LAYOUT_OUT_IN else codes.T
+    flat = np.ascontiguousarray(src).reshape(-1)
+    flat = np.concatenate([flat, np.zeros((-flat.size) % 4, np.uint8)])
+    body = (flat[0::4] | (flat[1::4] << 2) | (flat[2::4] << 4) | (flat[3::4] << 6)).astype(np.uint8)
+    scale = np.float32(0.0173)
+    tensor = np.concatenate([np.frombuffer(np.array([scale, 0.5], "<f4").tobytes(), np.uint8), body])
+    q_ref, s_ref, o_ref = orc.gguf_decode_ternary(tensor, n * k)
+    w_ref = q_ref.reshape(src.shape) if layout == bh.LAYOUT_OUT_IN else q_ref.reshape(src.shape).T
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "gguf")
+    for data in (torch.from_numpy(tensor.copy()), dev(tensor)):
+        got_scale, got_offset = layer.load_gguf_ternary(data, layout)
+        assert (got_scale, got_offset) == (s_ref, o_ref)
+        packed, ws = layer.get_quantized_weights()
+        assert ws == s_ref
+        assert np.array_equal(orc.unpack_2bit(packed.numpy(), n * k).reshape(n, k), w_ref)
+    x = synth_activations(rng, 3, k)
+    out = layer.forward(dev(x))
+    ref = orc.bitlinear_forward(x, orc.pack_2bit(np.ascontiguousarray(w_ref).reshape(-1)), n, float(s_ref))[0]
+    assert np.array_equal(host(out), ref)
+    with pytest.raises(bh.BitLinearError) as ei:
+        layer.load_gguf_ternary(torch.from_numpy(tensor[:-1].copy()), layout)
+    assert ei.value.kind == "ShapeMismatch"
+
+
 # ---- C++ host mirror -----------------------------------------------------------------------------------------
 
 def test_cpp_host_mirror_selftest():

@@ -27,6 +27,25 @@ def test_gguf_header_fixture():
     assert orc.unpack_2bit(raw[c["header_bytes"]:], c["count"]).tolist() == c["expected"]
 
 
+def test_gguf_decode_restatement_against_reference_test():
+    """GgufLoader::decode_ternary_weights: the reference's own test vector (gguf.rs:2421-2436), its header
+    handling (scale/offset read little endian, :1105-1117) and its length rule (:1097-1102)."""
+    c = G["gguf_header_fixture"]
+    raw = np.array(c["bytes"], dtype=np.uint8)
+    q, scale, offset = orc.gguf_decode_ternary(raw, c["count"])
+    assert q.tolist() == c["expected"]
+    # the test writes 1.0 big endian; read little endian (f32::from_le_bytes) those bytes are 0x0000803F
+    assert np.float32(scale).view(np.uint32) == 0x0000803F and offset == 0.0
+    hdr = np.frombuffer(np.array([0.75, -2.0], dtype="<f4").tobytes(), dtype=np.uint8)
+    q, scale, offset = orc.gguf_decode_ternary(np.concatenate([hdr, np.array([0xE4, 0x24], np.uint8)]), 7)
+    assert (scale, offset) == (0.75, -2.0) and q.tolist() == [-1, 0, 1, 0, -1, 0, 1]
+    # fewer than ceil(count/4) bytes: "Insufficient packed data"
+    assert orc.gguf_decode_ternary(np.zeros(3, np.uint8), 16) is None
+    # at least ceil(count/4) bytes but no room for the header: the reference decodes what is left, silently short
+    q, _, _ = orc.gguf_decode_ternary(np.full(10, 0x24, np.uint8), 40)
+    assert q.size == 8
+
+
 def test_pack_matches_reference_bytes():
     # inverse direction of the same fixtures: [-1,0,1,-1] must pack to 0b00100100
     assert orc.pack_2bit([-1, 0, 1, -1]).tolist() == [0b00100100]
