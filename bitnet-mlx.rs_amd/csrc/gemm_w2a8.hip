@@ -244,10 +244,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p)
 
 // ---- LDS-direct pipeline -------------------------------------------------------------------------------
 
-__device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_off)
+// LDS-direct load of 16 bytes per lane: m0 carries the LDS base of the wavefront's 1 KiB destination, lane l
+// lands at base + 16*l.  The global address is a scalar base plus a 32-bit per-lane byte offset: the offsets are
+// loop invariant, so advancing a stage costs two scalar additions and no vector instruction.
+__device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_off)
 {
-    // m0 carries the LDS base of the wavefront's 1 KiB destination; lane l lands at base + 16*l
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off\n\t" : : "v"(gptr), "s"(lds_off) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1\n\t" : : "v"(voff), "s"(sbase), "s"(lds_off) : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void wait_vm()
@@ -306,35 +308,39 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
     // Activation loads: load q of this wavefront covers tile rows 8*(wave*A_DMA + q) .. +7; lane l lands in
     // row l/8 at physical 16-byte chunk l%8 and therefore fetches logical chunk (l%8) ^ (row & 7).
     // Rows past m re-read row m-1 (their results are never stored).
-    const int8_t *a_src[A_DMA];
+    uint32_t a_off[A_DMA];  // byte offsets into the activation matrix (below 4 GiB: checked by the launcher)
 #pragma unroll
     for (int q = 0; q < A_DMA; ++q) {
         const int row = 8 * (wave * A_DMA + q) + (lane >> 3);
         const int lc = (lane & 7) ^ (row & 7);
         int grow = m0 + row;
         if (grow >= p.m) grow = p.m - 1;
-        a_src[q] = p.a + (size_t)grow * p.k + lc * 16;
+        a_off[q] = (uint32_t)grow * (uint32_t)p.k + lc * 16;
     }
     // Weight tiles: wavefront w fetches tiles w, w+4, ... of the workgroup's BN/16 row blocks; lane l = slot l.
     const int rb0 = n0 / 16;
     const int rb_last = (p.n + 15) / 16 - 1;
+    uint32_t b_off[B_DMA], b_dst[B_DMA];  // byte offsets into the re-tiled weights, tile positions in a weight stage
+#pragma unroll
+    for (int q = 0; q < B_DMA; ++q) {
+        int tix = wave + 4 * q;
+        if (tix >= B_TILES) tix = B_TILES - 1;
+        int rb = rb0 + tix;
+        if (rb > rb_last) rb = rb_last;
+        b_off[q] = ((uint32_t)rb * (uint32_t)p.kt_count * 64 + lane) * 16;
+        b_dst[q] = tix * 1024;
+    }
     // The load group of stage s: the weight tile of k-tile s/2 when s is even, then the activation stage.
     auto issue = [&](int s) {
         if ((s & 1) == 0) {
             const int kt = s >> 1;
             const uint32_t dst = lds_base + D * A_STAGE + (kt % NB) * B_STAGE;
 #pragma unroll
-            for (int q = 0; q < B_DMA; ++q) {
-                int tix = wave + 4 * q;
-                if (tix >= B_TILES) tix = B_TILES - 1;
-                int rb = rb0 + tix;
-                if (rb > rb_last) rb = rb_last;
-                dma16(p.w + (((size_t)rb * p.kt_count + kt) * 64 + lane) * 16, dst + tix * 1024);
-            }
+            for (int q = 0; q < B_DMA; ++q) dma16(p.w + (size_t)kt * 1024, b_off[q], dst + b_dst[q]);
         }
         const uint32_t dst = lds_base + (s % D) * A_STAGE + wave * A_DMA * 1024;
 #pragma unroll
-        for (int q = 0; q < A_DMA; ++q) dma16(a_src[q] + (size_t)s * DMA_SK, dst + q * 1024);
+        for (int q = 0; q < A_DMA; ++q) dma16(p.a + (size_t)s * DMA_SK, a_off[q], dst + q * 1024);
     };
 
     v4i acc[FM][FN];
@@ -523,7 +529,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
     // Activation loads: chunk c = wave*A_DMA + q of a stage is 8 rows x 128 columns: half c / (BM/8), rows
     // 8*(c % (BM/8)) .. +7.  Lane l lands in row l/8 at physical 16-byte chunk l%8 and fetches logical chunk
     // (l%8) ^ (row & 7).  Rows past m re-read row m-1 (their results are never stored).
-    const int8_t *a_src[A_DMA];
+    uint32_t a_off[A_DMA];  // byte offsets into the activation matrix (below 4 GiB: checked by the launcher)
 #pragma unroll
     for (int q = 0; q < A_DMA; ++q) {
         const int c = wave * A_DMA + q;
@@ -531,23 +537,26 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
         const int lc = (lane & 7) ^ (row & 7);
         int grow = m0 + row;
         if (grow >= p.m) grow = p.m - 1;
-        a_src[q] = p.a + (size_t)grow * p.k + half * 128 + lc * 16;
+        a_off[q] = (uint32_t)grow * (uint32_t)p.k + half * 128 + lc * 16;
     }
     const int rb0 = n0 / 16;
     const int rb_last = (p.n + 15) / 16 - 1;
+    uint32_t b_off[B_DMA], b_dst[B_DMA];
+#pragma unroll
+    for (int q = 0; q < B_DMA; ++q) {
+        int tix = wave + 8 * q;
+        if (tix >= B_TILES) tix = B_TILES - 1;
+        int rb = rb0 + tix;
+        if (rb > rb_last) rb = rb_last;
+        b_off[q] = ((uint32_t)rb * (uint32_t)p.kt_count * 64 + lane) * 16;
+        b_dst[q] = A_STAGE + tix * 1024;
+    }
     auto issue = [&](int kt) {
         const uint32_t stage = lds_base + (kt % D8_NST) * STAGE;
 #pragma unroll
-        for (int q = 0; q < B_DMA; ++q) {
-            int tix = wave + 8 * q;
-            if (tix >= B_TILES) tix = B_TILES - 1;
-            int rb = rb0 + tix;
-            if (rb > rb_last) rb = rb_last;
-            dma16(p.w + (((size_t)rb * p.kt_count + kt) * 64 + lane) * 16, stage + A_STAGE + tix * 1024);
-        }
+        for (int q = 0; q < B_DMA; ++q) dma16(p.w + (size_t)kt * 1024, b_off[q], stage + b_dst[q]);
 #pragma unroll
-        for (int q = 0; q < A_DMA; ++q)
-            dma16(a_src[q] + (size_t)kt * 256, stage + (wave * A_DMA + q) * 1024);
+        for (int q = 0; q < A_DMA; ++q) dma16(p.a + (size_t)kt * 256, a_off[q], stage + (wave * A_DMA + q) * 1024);
     };
 
     v4i acc[FM][FN];
@@ -564,10 +573,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
     for (int i = 0; i < FM; ++i) a_rd[i] = kg * (BM * 128) + (wm * WTM + i * 16 + lr) * 128;
     const int sw = lr & 7;
 
-    for (int kt = 0; kt < p.kt_count; ++kt) {
-        if (kt + 1 < p.kt_count) wait_vm<GROUP>(); else wait_vm<0>();
-        __syncthreads();
-        if (kt + 2 < p.kt_count) issue(kt + 2);
+    auto compute = [&](int kt) {
         const uint8_t *abuf = lds + (kt % D8_NST) * STAGE;
         const uint8_t *bbuf = abuf + A_STAGE + (wn * FN) * 1024 + lane * 16 + kg * 8;
         uint2 bp[FN];  // dwords 2*kg, 2*kg+1 of the slot: this group's two k-steps
@@ -592,6 +598,12 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bfrag, afrag[i], acc[i][j], 0, 0, 0);
             }
         }
+    };
+    for (int kt = 0; kt < p.kt_count; ++kt) {
+        if (kt + 1 < p.kt_count) wait_vm<GROUP>(); else wait_vm<0>();
+        __syncthreads();
+        if (kt + 2 < p.kt_count) issue(kt + 2);
+        compute(kt);
     }
 
     // ---- exchange: group 0 finishes fragments i < FM/2, group 1 the others ----
@@ -726,7 +738,8 @@ int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_su
     p.residual = residual; p.a_sum = a_sum; p.out = out; p.m = (int)m; p.n = (int)n; p.k = (int)k; p.kt_count = (int)k_tiles(k);
     p.tiles_m = p.tiles_n = 0;
     const bool dma_ok = a_sum != nullptr && m >= 96 && k % 256 == 0 && k >= 512 &&
-                        (reinterpret_cast<uintptr_t>(a) & 15) == 0;
+                        (reinterpret_cast<uintptr_t>(a) & 15) == 0 &&
+                        m * k < (1ull << 32) && tiled_bytes(n, k) < (1ull << 32);  // 32-bit lane offsets
     if (dma_ok) {
         // Three shapes of the LDS-direct kernel, chosen by how many 128 x 160 tiles the output holds
         // (256 compute units; the MFMA pipe of a SIMD needs two resident wavefronts to stay busy):
