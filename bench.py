@@ -129,6 +129,14 @@ def prefill_rates(bh, torch, dec, gen, reps):
         fwd_ms = time_events(torch, lambda: [bl.forward(x) for _ in range(reps)]) / reps
         res[name]["forward_f32_in_ms"] = round(fwd_ms, 4)
         del a, out, x
+    # projections that share their input in one call: one quantiser pass, one GEMM launch for all of them
+    x = torch.randn((m, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
+    for name, projs in (("q_k_v_2048x3840x2560", (0, 1, 2)), ("gate_up_2048x13824x2560", (4, 5))):
+        layers = [dec.projection(0, p) for p in projs]
+        bh.forward_multi(layers, x)
+        ms = time_events(torch, lambda: [bh.forward_multi(layers, x) for _ in range(reps)]) / reps
+        ops = 2.0 * m * HIDDEN * sum(dec.proj_shape(p)[0] for p in projs)
+        res[name] = {"forward_f32_in_ms": round(ms, 4), "tops_incl_quantiser": round(ops / (ms * 1e-3) / 1e12, 1)}
     return res
 
 

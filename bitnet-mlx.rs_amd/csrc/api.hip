@@ -136,10 +136,21 @@ int run_projections(bitnet_hip_bitlinear *const *layers, int count, const float 
         }
         return BITNET_HIP_OK;
     }
-    for (int j = 0; j < count; ++j) {
-        GemvProj pj = proj_of(j);
-        rc = launch_gemm_tiled(pj.tiled, q, a_sum, m, pj.n, k, pj.acc, pj.w_scale, a_scale, pj.bias, pj.residual, pj.out, s);
-        if (rc != BITNET_HIP_OK) return rc;
+    for (int j0 = 0; j0 < count; j0 += GEMM_MAX_PROJ) {
+        GemvProj pjs[GEMM_MAX_PROJ];
+        const int nj = count - j0 < GEMM_MAX_PROJ ? count - j0 : GEMM_MAX_PROJ;
+        for (int j = 0; j < nj; ++j) pjs[j] = proj_of(j0 + j);
+        rc = launch_gemm_multi(pjs, nj, q, a_sum, a_scale, m, k, s);  // all of them in one launch where that applies
+        if (rc == BITNET_HIP_UNSUPPORTED) {
+            for (int j = 0; j < nj; ++j) {
+                const GemvProj &pj = pjs[j];
+                rc = launch_gemm_tiled(pj.tiled, q, a_sum, m, pj.n, k, pj.acc, pj.w_scale, a_scale, pj.bias, pj.residual,
+                                       pj.out, s);
+                if (rc != BITNET_HIP_OK) return rc;
+            }
+        } else if (rc != BITNET_HIP_OK) {
+            return rc;
+        }
     }
     return BITNET_HIP_OK;
 }

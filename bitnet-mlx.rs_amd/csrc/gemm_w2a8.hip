@@ -42,7 +42,21 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
+struct GemmProjDev {  // one projection of a launch of the LDS-direct kernels
+    const uint8_t *w;
+    const float *w_scale;
+    const float *bias;
+    const float *residual;
+    float *out;
+    int32_t *acc;
+    int n;
+    int tn_end;  // column tiles of projections 0..this one, cumulative
+};
+
 struct GemmParams {
+    GemmProjDev proj[GEMM_MAX_PROJ];  // LDS-direct kernels: projections sharing the activation matrix
+    int nproj;
+    // single-projection view (the register-staged kernel)
     const uint8_t *w;
     const int8_t *a;
     int32_t *acc;
@@ -301,7 +315,13 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
         tile_id = xcd * per_xcd + idx;
         if (tile_id >= total) return;
     }
-    const int tm = tile_id / p.tiles_n, tn = tile_id % p.tiles_n;
+    // tiles_n counts the column tiles of all projections of the launch, one after the other
+    const int tm = tile_id / p.tiles_n, tn_all = tile_id % p.tiles_n;
+    int pj = 0;
+    if (p.nproj > 1 && tn_all >= p.proj[0].tn_end) pj = 1;
+    if (p.nproj > 2 && tn_all >= p.proj[1].tn_end) pj = 2;
+    const GemmProjDev PJ = p.proj[pj];  // uniform over the workgroup
+    const int tn = tn_all - (pj ? p.proj[pj - 1].tn_end : 0);
     const int m0 = tm * BM, n0 = tn * BN;
     const int nstage = p.kt_count * 2;
 
@@ -319,7 +339,7 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
     }
     // Weight tiles: wavefront w fetches tiles w, w+4, ... of the workgroup's BN/16 row blocks; lane l = slot l.
     const int rb0 = n0 / 16;
-    const int rb_last = (p.n + 15) / 16 - 1;
+    const int rb_last = (PJ.n + 15) / 16 - 1;
     uint32_t b_off[B_DMA], b_dst[B_DMA];  // byte offsets into the re-tiled weights, tile positions in a weight stage
 #pragma unroll
     for (int q = 0; q < B_DMA; ++q) {
@@ -336,7 +356,7 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
             const int kt = s >> 1;
             const uint32_t dst = lds_base + D * A_STAGE + (kt % NB) * B_STAGE;
 #pragma unroll
-            for (int q = 0; q < B_DMA; ++q) dma16(p.w + (size_t)kt * 1024, b_off[q], dst + b_dst[q]);
+            for (int q = 0; q < B_DMA; ++q) dma16(PJ.w + (size_t)kt * 1024, b_off[q], dst + b_dst[q]);
         }
         const uint32_t dst = lds_base + (s % D) * A_STAGE + wave * A_DMA * 1024;
 #pragma unroll
@@ -404,16 +424,16 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
         compute(s + 1, true);
     }
 
-    const float ws = p.out ? *p.w_scale : 0.0f;
+    const float ws = PJ.out ? *PJ.w_scale : 0.0f;
     const unsigned ws_expo = (__builtin_bit_cast(unsigned, ws) >> 23) & 0xffu;
     const bool ws_fast = ws > 0.0f && ws_expo > 64u && ws_expo < 160u;
-    const bool vec_ok = (p.n & 3) == 0;  // 16-byte alignment of out[row][4c]
+    const bool vec_ok = (PJ.n & 3) == 0;  // 16-byte alignment of out[row][4c]
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
         const int row = m0 + wm * WTM + i * 16 + lr;
         const bool row_ok = row < p.m;
         const int rs = row_ok ? p.a_sum[row] : 0;
-        const float as = (p.out && row_ok) ? p.a_scale[row] : 1.0f;
+        const float as = (PJ.out && row_ok) ? p.a_scale[row] : 1.0f;
         const float as_recip = f32_div(1.0f, as);
         // the short division needs a well-behaved divisor (per row) and dividends in range: float(total) * ws
         // is zero or has ws's exponent plus at most 24, so one check on ws covers them.  The choice is made
@@ -424,8 +444,8 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             const int col = n0 + wn * WTN + j * 16 + lg * 4;
-            if (col >= p.n) continue;
-            const size_t o = (size_t)row * p.n + col;
+            if (col >= PJ.n) continue;
+            const size_t o = (size_t)row * PJ.n + col;
             int tot[4];
             float v[4];
 #pragma unroll
@@ -435,28 +455,28 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
                 v[r] = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
             }
             if (vec_ok) {  // col + 3 < n follows from n % 4 == 0
-                if (p.acc) *reinterpret_cast<int4 *>(p.acc + o) = make_int4(tot[0], tot[1], tot[2], tot[3]);
-                if (p.out) {
-                    if (p.bias) {
-                        const float4 b = *reinterpret_cast<const float4 *>(p.bias + col);
+                if (PJ.acc) *reinterpret_cast<int4 *>(PJ.acc + o) = make_int4(tot[0], tot[1], tot[2], tot[3]);
+                if (PJ.out) {
+                    if (PJ.bias) {
+                        const float4 b = *reinterpret_cast<const float4 *>(PJ.bias + col);
                         v[0] = f32_add(v[0], b.x); v[1] = f32_add(v[1], b.y); v[2] = f32_add(v[2], b.z); v[3] = f32_add(v[3], b.w);
                     }
-                    if (p.residual) {
-                        const float4 q = *reinterpret_cast<const float4 *>(p.residual + o);
+                    if (PJ.residual) {
+                        const float4 q = *reinterpret_cast<const float4 *>(PJ.residual + o);
                         v[0] = f32_add(v[0], q.x); v[1] = f32_add(v[1], q.y); v[2] = f32_add(v[2], q.z); v[3] = f32_add(v[3], q.w);
                     }
-                    *reinterpret_cast<float4 *>(p.out + o) = make_float4(v[0], v[1], v[2], v[3]);
+                    *reinterpret_cast<float4 *>(PJ.out + o) = make_float4(v[0], v[1], v[2], v[3]);
                 }
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    if (col + r >= p.n) continue;
-                    if (p.acc) p.acc[o + r] = tot[r];
-                    if (p.out) {
+                    if (col + r >= PJ.n) continue;
+                    if (PJ.acc) PJ.acc[o + r] = tot[r];
+                    if (PJ.out) {
                         float y = v[r];
-                        if (p.bias) y = f32_add(y, p.bias[col + r]);
-                        if (p.residual) y = f32_add(y, p.residual[o + r]);
-                        p.out[o + r] = y;
+                        if (PJ.bias) y = f32_add(y, PJ.bias[col + r]);
+                        if (PJ.residual) y = f32_add(y, PJ.residual[o + r]);
+                        PJ.out[o + r] = y;
                     }
                 }
             }
@@ -468,7 +488,8 @@ template <int BM, int BN, int D, int OCC>
 int launch_dma(GemmParams p, hipStream_t stream)
 {
     p.tiles_m = (p.m + BM - 1) / BM;
-    p.tiles_n = (p.n + BN - 1) / BN;
+    p.tiles_n = 0;
+    for (int j = 0; j < p.nproj; ++j) p.proj[j].tn_end = p.tiles_n += (p.proj[j].n + BN - 1) / BN;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
     constexpr size_t lds = dma_lds_bytes<BM, BN, D>();
@@ -523,7 +544,13 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
         tile_id = xcd * per_xcd + idx;
         if (tile_id >= total) return;
     }
-    const int tm = tile_id / p.tiles_n, tn = tile_id % p.tiles_n;
+    // tiles_n counts the column tiles of all projections of the launch, one after the other
+    const int tm = tile_id / p.tiles_n, tn_all = tile_id % p.tiles_n;
+    int pj = 0;
+    if (p.nproj > 1 && tn_all >= p.proj[0].tn_end) pj = 1;
+    if (p.nproj > 2 && tn_all >= p.proj[1].tn_end) pj = 2;
+    const GemmProjDev PJ = p.proj[pj];  // uniform over the workgroup
+    const int tn = tn_all - (pj ? p.proj[pj - 1].tn_end : 0);
     const int m0 = tm * BM, n0 = tn * BN;
 
     // Activation loads: chunk c = wave*A_DMA + q of a stage is 8 rows x 128 columns: half c / (BM/8), rows
@@ -540,7 +567,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
         a_off[q] = (uint32_t)grow * (uint32_t)p.k + half * 128 + lc * 16;
     }
     const int rb0 = n0 / 16;
-    const int rb_last = (p.n + 15) / 16 - 1;
+    const int rb_last = (PJ.n + 15) / 16 - 1;
     uint32_t b_off[B_DMA], b_dst[B_DMA];
 #pragma unroll
     for (int q = 0; q < B_DMA; ++q) {
@@ -554,7 +581,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
     auto issue = [&](int kt) {
         const uint32_t stage = lds_base + (kt % D8_NST) * STAGE;
 #pragma unroll
-        for (int q = 0; q < B_DMA; ++q) dma16(p.w + (size_t)kt * 1024, b_off[q], stage + b_dst[q]);
+        for (int q = 0; q < B_DMA; ++q) dma16(PJ.w + (size_t)kt * 1024, b_off[q], stage + b_dst[q]);
 #pragma unroll
         for (int q = 0; q < A_DMA; ++q) dma16(p.a + (size_t)kt * 256, a_off[q], stage + (wave * A_DMA + q) * 1024);
     };
@@ -628,17 +655,17 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
             }
     }
 
-    const float ws = p.out ? *p.w_scale : 0.0f;
+    const float ws = PJ.out ? *PJ.w_scale : 0.0f;
     const unsigned ws_expo = (__builtin_bit_cast(unsigned, ws) >> 23) & 0xffu;
     const bool ws_fast = ws > 0.0f && ws_expo > 64u && ws_expo < 160u;
-    const bool vec_ok = (p.n & 3) == 0;
+    const bool vec_ok = (PJ.n & 3) == 0;
 #pragma unroll
     for (int ii = 0; ii < FM / 2; ++ii) {
         const int i = kg == 0 ? ii : ii + FM / 2;
         const int row = m0 + wm * WTM + i * 16 + lr;
         const bool row_ok = row < p.m;
         const int rs = row_ok ? p.a_sum[row] : 0;
-        const float as = (p.out && row_ok) ? p.a_scale[row] : 1.0f;
+        const float as = (PJ.out && row_ok) ? p.a_scale[row] : 1.0f;
         const float as_recip = f32_div(1.0f, as);
         const bool row_fast = ws_fast && invariant_divisor_ok(as);
         const bool wave_fast = __builtin_amdgcn_ballot_w64(!row_fast) == 0;
@@ -646,8 +673,8 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             const int col = n0 + wn * WTN + j * 16 + lg * 4;
-            if (col >= p.n) continue;
-            const size_t o = (size_t)row * p.n + col;
+            if (col >= PJ.n) continue;
+            const size_t o = (size_t)row * PJ.n + col;
             const v4i a4 = kg == 0 ? acc[ii][j] : acc[ii + FM / 2][j];
             int tot[4];
             float v[4];
@@ -658,28 +685,28 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
                 v[r] = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
             }
             if (vec_ok) {
-                if (p.acc) *reinterpret_cast<int4 *>(p.acc + o) = make_int4(tot[0], tot[1], tot[2], tot[3]);
-                if (p.out) {
-                    if (p.bias) {
-                        const float4 b = *reinterpret_cast<const float4 *>(p.bias + col);
+                if (PJ.acc) *reinterpret_cast<int4 *>(PJ.acc + o) = make_int4(tot[0], tot[1], tot[2], tot[3]);
+                if (PJ.out) {
+                    if (PJ.bias) {
+                        const float4 b = *reinterpret_cast<const float4 *>(PJ.bias + col);
                         v[0] = f32_add(v[0], b.x); v[1] = f32_add(v[1], b.y); v[2] = f32_add(v[2], b.z); v[3] = f32_add(v[3], b.w);
                     }
-                    if (p.residual) {
-                        const float4 q = *reinterpret_cast<const float4 *>(p.residual + o);
+                    if (PJ.residual) {
+                        const float4 q = *reinterpret_cast<const float4 *>(PJ.residual + o);
                         v[0] = f32_add(v[0], q.x); v[1] = f32_add(v[1], q.y); v[2] = f32_add(v[2], q.z); v[3] = f32_add(v[3], q.w);
                     }
-                    *reinterpret_cast<float4 *>(p.out + o) = make_float4(v[0], v[1], v[2], v[3]);
+                    *reinterpret_cast<float4 *>(PJ.out + o) = make_float4(v[0], v[1], v[2], v[3]);
                 }
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    if (col + r >= p.n) continue;
-                    if (p.acc) p.acc[o + r] = tot[r];
-                    if (p.out) {
+                    if (col + r >= PJ.n) continue;
+                    if (PJ.acc) PJ.acc[o + r] = tot[r];
+                    if (PJ.out) {
                         float y = v[r];
-                        if (p.bias) y = f32_add(y, p.bias[col + r]);
-                        if (p.residual) y = f32_add(y, p.residual[o + r]);
-                        p.out[o + r] = y;
+                        if (PJ.bias) y = f32_add(y, PJ.bias[col + r]);
+                        if (PJ.residual) y = f32_add(y, PJ.residual[o + r]);
+                        PJ.out[o + r] = y;
                     }
                 }
             }
@@ -691,7 +718,8 @@ template <int BM, int BN>
 int launch_dma8(GemmParams p, hipStream_t stream)
 {
     p.tiles_m = (p.m + BM - 1) / BM;
-    p.tiles_n = (p.n + BN - 1) / BN;
+    p.tiles_n = 0;
+    for (int j = 0; j < p.nproj; ++j) p.proj[j].tn_end = p.tiles_n += (p.proj[j].n + BN - 1) / BN;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
     constexpr size_t lds = dma8_lds_bytes<BM, BN>();
@@ -728,29 +756,53 @@ int launch_tile(GemmParams p, hipStream_t stream)
 
 }  // namespace
 
+// Up to GEMM_MAX_PROJ projections of the same activation matrix in one launch of the LDS-direct kernels (q, k, v
+// or gate, up at prefill: small projections alone would leave most compute units idle).  Returns
+// BITNET_HIP_UNSUPPORTED (without a message) when the shapes do not fit those kernels.
+int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const int32_t *a_sum, const float *a_scale,
+                      size_t m, size_t k, hipStream_t stream)
+{
+    if (m == 0 || nproj <= 0) return BITNET_HIP_OK;
+    if (nproj > GEMM_MAX_PROJ) return BITNET_HIP_UNSUPPORTED;
+    bool dma_ok = a_sum != nullptr && m >= 96 && k % 256 == 0 && k >= 512 && (reinterpret_cast<uintptr_t>(a) & 15) == 0 &&
+                  m * k < (1ull << 32);  // 32-bit lane offsets
+    size_t tiles = 0;
+    GemmParams p = {};
+    for (int j = 0; j < nproj && dma_ok; ++j) {
+        const GemvProj &s = projs[j];
+        dma_ok = s.n > 0 && s.n <= 0x7fffffffu && tiled_bytes(s.n, k) < (1ull << 32);
+        tiles += ((m + 127) / 128) * ((s.n + 159) / 160);
+        GemmProjDev &d = p.proj[j];
+        d.w = s.tiled; d.w_scale = s.w_scale; d.bias = s.bias; d.residual = s.residual; d.out = s.out; d.acc = s.acc;
+        d.n = (int)s.n; d.tn_end = 0;
+    }
+    if (!dma_ok) return BITNET_HIP_UNSUPPORTED;
+    for (int j = nproj; j < GEMM_MAX_PROJ; ++j) p.proj[j] = p.proj[nproj - 1];
+    p.nproj = nproj; p.a = a; p.a_sum = a_sum; p.a_scale = a_scale; p.m = (int)m; p.k = (int)k; p.kt_count = (int)k_tiles(k);
+    // Three shapes of the LDS-direct kernel, chosen by how many 128 x 160 tiles the outputs hold
+    // (256 compute units; the MFMA pipe of a SIMD needs two resident wavefronts to stay busy):
+    //   four or more tiles per compute unit  -> 128 x 160, two workgroups of 4 wavefronts per compute unit;
+    //   between a half and one tile per unit -> 128 x 160, one workgroup of 8 wavefronts (k split inside it);
+    //   otherwise                            -> 64 x 160, three workgroups of 4 wavefronts per compute unit.
+    if (tiles >= 1024) return launch_dma<128, 160, 3, 2>(p, stream);
+    if (tiles >= 128 && tiles <= 256) return launch_dma8<128, 160>(p, stream);
+    return launch_dma<64, 160, 3, 3>(p, stream);
+}
+
 int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_sum, size_t m, size_t n, size_t k,
                       int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,
                       const float *residual, float *out, hipStream_t stream)
 {
     if (m == 0 || n == 0) return BITNET_HIP_OK;
-    GemmParams p;
+    {
+        const GemvProj one = {tiled, w_scale, bias, residual, out, acc, n};
+        const int rc = launch_gemm_multi(&one, 1, a, a_sum, a_scale, m, k, stream);
+        if (rc != BITNET_HIP_UNSUPPORTED) return rc;
+    }
+    GemmParams p = {};
     p.w = tiled; p.a = a; p.acc = acc; p.w_scale = w_scale; p.a_scale = a_scale; p.bias = bias;
     p.residual = residual; p.a_sum = a_sum; p.out = out; p.m = (int)m; p.n = (int)n; p.k = (int)k; p.kt_count = (int)k_tiles(k);
     p.tiles_m = p.tiles_n = 0;
-    const bool dma_ok = a_sum != nullptr && m >= 96 && k % 256 == 0 && k >= 512 &&
-                        (reinterpret_cast<uintptr_t>(a) & 15) == 0 &&
-                        m * k < (1ull << 32) && tiled_bytes(n, k) < (1ull << 32);  // 32-bit lane offsets
-    if (dma_ok) {
-        // Three shapes of the LDS-direct kernel, chosen by how many 128 x 160 tiles the output holds
-        // (256 compute units; the MFMA pipe of a SIMD needs two resident wavefronts to stay busy):
-        //   four or more tiles per compute unit  -> 128 x 160, two workgroups of 4 wavefronts per compute unit;
-        //   between a half and one tile per unit -> 128 x 160, one workgroup of 8 wavefronts (k split inside it);
-        //   otherwise                            -> 64 x 160, three workgroups of 4 wavefronts per compute unit.
-        const size_t tiles = ((m + 127) / 128) * ((n + 159) / 160);
-        if (tiles >= 1024) return launch_dma<128, 160, 3, 2>(p, stream);
-        if (tiles >= 128 && tiles <= 256) return launch_dma8<128, 160>(p, stream);
-        return launch_dma<64, 160, 3, 3>(p, stream);
-    }
     if (m < 96) return launch_tile<64, 128>(p, stream);
     auto waste = [&](size_t bn) {
         const size_t tiles = ((m + 127) / 128) * ((n + bn - 1) / bn), slots = 256;

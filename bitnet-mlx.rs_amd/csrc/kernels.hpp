@@ -58,6 +58,10 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
                       int sum_order, int8_t *q_out, float *a_scale_out, int32_t *a_sum_out, hipStream_t stream);
 
 // gemm_w2a8.hip
+constexpr int GEMM_MAX_PROJ = 3;  // projections sharing one activation matrix per launch of the LDS-direct kernels
+// several projections in one launch; BITNET_HIP_UNSUPPORTED (no message) if the LDS-direct kernels do not apply
+int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const int32_t *a_sum, const float *a_scale,
+                      size_t m, size_t k, hipStream_t stream);
 // a_sum (sum_k a[t, k] per row, from the activation quantiser) may be NULL: the slower kernel then computes it
 int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_sum, size_t m, size_t n, size_t k,
                       int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,

@@ -431,9 +431,10 @@ def test_bitlinear_forward_shapes_bias_norm_and_layouts():
     assert np.array_equal(host(layer_p.forward(dev(x))), ref0)
 
 
-@pytest.mark.parametrize("m", [1, 3, 8, 20, 200])
+@pytest.mark.parametrize("m", [1, 3, 8, 20, 200, 1100])
 def test_forward_multi_matches_single_forwards(m):
-    """q/k/v-style: several layers on one input give exactly what each layer gives alone, and what the oracle gives."""
+    """q/k/v-style: several layers on one input give exactly what each layer gives alone, and what the oracle gives.
+    (m = 200 and 1100: the projections share launches of the 64 x 160 and of the eight-wavefront prefill GEMM.)"""
     rng = np.random.default_rng(40 + m)
     k = 2560
     ns = [2560, 640, 640, 96]
@@ -456,6 +457,29 @@ def test_forward_multi_matches_single_forwards(m):
     with pytest.raises(bh.BitLinearError) as ei:
         bh.forward_multi([layers[0], other], dev(x))
     assert ei.value.kind == "ShapeMismatch"
+
+
+def test_forward_multi_prefill_gate_up_one_launch():
+    """gate and up at M = 2048 share one launch of the 128 x 160 prefill GEMM (1408 tiles): sampled rows against the
+    oracle, everything against the single-layer forwards."""
+    rng = np.random.default_rng(4242)
+    m, k, n = 2048, 2560, 6912
+    g = (1 + 0.1 * rng.standard_normal(k, dtype=f32)).astype(f32)
+    x = synth_activations(rng, m, k)
+    rows = np.sort(rng.choice(m, size=24, replace=False))
+    layers, refs = [], []
+    for i in range(2):
+        w = synth_weights(rng, n, k)
+        layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), f"gu{i}")
+        layer.update_weights(dev(w))
+        layers.append(layer)
+        qw, ws = orc.quantize_weights_absmean(w)
+        refs.append(orc.bitlinear_forward(x[rows], orc.pack_2bit(qw), n, ws, g=g, eps=1e-5)[0])
+    outs = bh.forward_multi(layers, dev(x), gamma=dev(g))
+    for layer, out, ref in zip(layers, outs, refs):
+        got = host(out)
+        assert np.array_equal(got[rows], ref)
+        assert np.array_equal(got, host(layer.forward(dev(x), gamma=dev(g))))
 
 
 @pytest.mark.parametrize("m", [1, 2, 5, 8])
