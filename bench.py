@@ -158,9 +158,9 @@ def stack_latency(bh, torch, dec, gen, reps=20):
                                     "gbs_packed_weights": round(dec.weight_bytes() / (ms * 1e-3) / 1e9, 1)}
     del big
     # the decode GEMV where a launch is large enough to be bound by bandwidth rather than by launch latency:
-    # 16384 x 16384 ternary weights (64 MiB packed), int8 activations already quantised, one token
-    n = k = 16384
-    layers = [bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), f"large{i}") for i in range(5)]  # 320 MiB > cache
+    # 32768 x 16384 ternary weights (128 MiB packed), int8 activations already quantised, one token
+    n, k = 32768, 16384
+    layers = [bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), f"large{i}") for i in range(4)]  # 512 MiB > cache
     packed = torch.randint(0, 256, (n * k // 4,), generator=gen, device="cuda", dtype=torch.uint8)
     for bl in layers:
         bl.set_quantized_weights(packed, 0.02)
@@ -169,8 +169,8 @@ def stack_latency(bh, torch, dec, gen, reps=20):
     y = torch.empty((1, n), device="cuda", dtype=torch.float32)
     for bl in layers:
         bl.matmul_quantized(a, a_scale, out=y)
-    ms = time_events(torch, lambda: [bl.matmul_quantized(a, a_scale, out=y) for _ in range(4) for bl in layers]) / 20
-    out["gemv_16384x16384_m1"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1),
+    ms = time_events(torch, lambda: [bl.matmul_quantized(a, a_scale, out=y) for _ in range(5) for bl in layers]) / 20
+    out["gemv_32768x16384_m1"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1),
                                   "frac_hbm_peak": round(n * k / 4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     del layers, packed
     for name, p in (("gate_2560x6912", 4), ("down_6912x2560", 6)):

@@ -508,9 +508,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
             }
         }
     };
-    load_batch(wave, wcur, acur);
-    for (int kt0 = wave; kt0 < p.kt_count; kt0 += 4 * PF) {
-        load_batch(kt0 + 4 * PF, wnxt, anxt);
+    auto compute_batch = [&](int kt0) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
             if (kt0 + 4 * u >= p.kt_count) continue;
@@ -539,14 +537,24 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
                 }
             }
         }
+    };
+    load_batch(wave, wcur, acur);
+    for (int kt0 = wave; kt0 < p.kt_count; kt0 += 4 * PF) {
+        // two straight-line bodies, so that the wait before the MFMAs is for this batch only in both of them
+        if (kt0 + 4 * PF < p.kt_count) {  // uniform over the wavefront
+            load_batch(kt0 + 4 * PF, wnxt, anxt);
+            compute_batch(kt0);
 #pragma unroll
-        for (int u = 0; u < PF; ++u) {
+            for (int u = 0; u < PF; ++u) {
 #pragma unroll
-            for (int r = 0; r < RB; ++r) wcur[u][r] = wnxt[u][r];
+                for (int r = 0; r < RB; ++r) wcur[u][r] = wnxt[u][r];
 #pragma unroll
-            for (int g = 0; g < MT; ++g)
+                for (int g = 0; g < MT; ++g)
 #pragma unroll
-                for (int t = 0; t < 4; ++t) acur[u][g][t] = anxt[u][g][t];
+                    for (int t = 0; t < 4; ++t) acur[u][g][t] = anxt[u][g][t];
+            }
+        } else {
+            compute_batch(kt0);
         }
     }
 
