@@ -224,13 +224,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
     for (int t = 0; t < MB; ++t) acc[t] = 0;
 
     const int kq = lane >> 4;  // lane group: columns 64t + 16kq .. +15 of each tile, t = 0..3
-    for (int kt0 = wave; kt0 < p.kt_count; kt0 += 4 * GEMV_PREFETCH) {
-        uint4 wnext[GEMV_PREFETCH];
-#pragma unroll
-        for (int u = 0; u < GEMV_PREFETCH; ++u) {
-            int kt = kt0 + 4 * (GEMV_PREFETCH + u);
-            wnext[u] = tiles[(size_t)min(kt, p.kt_count - 1) * 64 + lane];
-        }
+    auto dot_batch = [&](int kt0) {
 #pragma unroll
         for (int u = 0; u < GEMV_PREFETCH; ++u) {
             int kt = kt0 + 4 * u;
@@ -240,8 +234,20 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
                 for (int t = 0; t < MB; ++t) acc[t] = dot64(wbuf[u], ag + t * groups, acc[t]);
             }
         }
+    };
+    for (int kt0 = wave; kt0 < p.kt_count; kt0 += 4 * GEMV_PREFETCH) {
+        // two straight-line bodies: the last batch requests nothing more and waits for nothing but itself
+        if (kt0 + 4 * GEMV_PREFETCH < p.kt_count) {  // uniform over the wavefront
+            uint4 wnext[GEMV_PREFETCH];
 #pragma unroll
-        for (int u = 0; u < GEMV_PREFETCH; ++u) wbuf[u] = wnext[u];
+            for (int u = 0; u < GEMV_PREFETCH; ++u)
+                wnext[u] = tiles[(size_t)min(kt0 + 4 * (GEMV_PREFETCH + u), p.kt_count - 1) * 64 + lane];
+            dot_batch(kt0);
+#pragma unroll
+            for (int u = 0; u < GEMV_PREFETCH; ++u) wbuf[u] = wnext[u];
+        } else {
+            dot_batch(kt0);
+        }
     }
 
     // the four lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
