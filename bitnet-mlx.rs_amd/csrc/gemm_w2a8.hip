@@ -484,6 +484,14 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
     }
 }
 
+// Raising a kernel's dynamic LDS limit is needed once per process; a function-local static makes that once
+// thread-safe (forward may be called from many threads).
+template <typename Kernel>
+hipError_t raise_lds_limit(Kernel kernel, size_t bytes)
+{
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
 template <int BM, int BN, int D, int OCC>
 int launch_dma(GemmParams p, hipStream_t stream)
 {
@@ -494,12 +502,8 @@ int launch_dma(GemmParams p, hipStream_t stream)
     const int grid = ((total + 7) / 8) * 8;
     constexpr size_t lds = dma_lds_bytes<BM, BN, D>();
     static_assert(lds <= 160 * 1024 && lds * OCC <= 160 * 1024, "LDS budget");
-    static bool attr_set = false;
-    if (lds > 64 * 1024 && !attr_set) {
-        BITNET_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_dma_kernel<BM, BN, D, OCC>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_set = true;
-    }
+    static const hipError_t attr = lds > 64 * 1024 ? raise_lds_limit(&gemm_dma_kernel<BM, BN, D, OCC>, lds) : hipSuccess;
+    BITNET_HIP_TRY(attr);
     hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, D, OCC>), dim3(grid), dim3(256), lds, stream, p);
     BITNET_HIP_CHECK_LAUNCH("gemm_dma_kernel");
     return BITNET_HIP_OK;
@@ -724,12 +728,8 @@ int launch_dma8(GemmParams p, hipStream_t stream)
     const int grid = ((total + 7) / 8) * 8;
     constexpr size_t lds = dma8_lds_bytes<BM, BN>();
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static bool attr_set = false;
-    if (!attr_set) {
-        BITNET_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_dma8_kernel<BM, BN>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_set = true;
-    }
+    static const hipError_t attr = raise_lds_limit(&gemm_dma8_kernel<BM, BN>, lds);
+    BITNET_HIP_TRY(attr);
     hipLaunchKernelGGL((gemm_dma8_kernel<BM, BN>), dim3(grid), dim3(512), lds, stream, p);
     BITNET_HIP_CHECK_LAUNCH("gemm_dma8_kernel");
     return BITNET_HIP_OK;
@@ -743,12 +743,8 @@ int launch_tile(GemmParams p, hipStream_t stream)
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
     constexpr size_t lds = 2 * BM * LDS_PITCH + BM * sizeof(int);
-    static bool attr_set = false;  // raising the dynamic LDS limit is per kernel, once per process
-    if (lds > 64 * 1024 && !attr_set) {
-        BITNET_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tiled_kernel<BM, BN>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_set = true;
-    }
+    static const hipError_t attr = lds > 64 * 1024 ? raise_lds_limit(&gemm_tiled_kernel<BM, BN>, lds) : hipSuccess;
+    BITNET_HIP_TRY(attr);
     hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN>), dim3(grid), dim3(256), lds, stream, p);
     BITNET_HIP_CHECK_LAUNCH("gemm_tiled_kernel");
     return BITNET_HIP_OK;
