@@ -505,6 +505,49 @@ def test_bitlinear_forward_decode_debug_outputs(m):
     assert np.array_equal(host(layer.forward(dev(x), gamma=dev(g))), out_ref)
 
 
+def test_forward_from_several_threads_and_streams():
+    """BitLinear is Send + Sync in the reference (layer.rs:427-428): forward on one layer object from several host
+    threads, each on a stream of its own, at decode and prefill token counts, while nothing is shared but the
+    read-locked weights."""
+    import threading
+
+    rng = np.random.default_rng(99)
+    k, n = 2560, 640
+    w = synth_weights(rng, n, k)
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "shared")
+    layer.update_weights(dev(w))
+    qw, ws = orc.quantize_weights_absmean(w)
+    packed = orc.pack_2bit(qw)
+    cases = []
+    for t, m in enumerate([1, 1, 5, 130]):
+        x = synth_activations(rng, m, k, outliers=True)
+        cases.append((x, orc.bitlinear_forward(x, packed, n, ws)[0]))
+    errors = []
+
+    def worker(x, ref):
+        try:
+            stream = torch.cuda.Stream()  # default priority
+            xd = dev(x)
+            torch.cuda.current_stream().synchronize()
+            for _ in range(25):
+                with torch.cuda.stream(stream):
+                    out = layer.forward(xd, stream=stream)
+                stream.synchronize()
+                if not np.array_equal(host(out), ref):
+                    errors.append("mismatch")
+                    return
+        except Exception as e:  # noqa: BLE001 - reported below
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=c) for c in cases]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not errors, errors
+    assert not any(th.is_alive() for th in threads)
+
+
 def test_bitlinear_error_behaviour_matches_reference():
     """forward.rs:304-371: wrong last dimension -> ShapeMismatch; rank other than 2/3 -> ShapeMismatch."""
     layer = bh.BitLinear(bh.BitLinearConfig(in_features=4, out_features=3), "test_layer_shape")
