@@ -21,7 +21,8 @@
 // quantiser): activations AND weight tiles travel global -> LDS with LDS-direct loads
 // (global_load_lds_dwordx4), never through registers.  D LDS stages of 128 columns are kept in flight;
 // the wait counts are placed by hand (s_waitcnt vmcnt(N)) so that D - 1 stages of loads stay outstanding
-// while one is computed.  An LDS-direct load writes lane l's 16 bytes at base + 16*l, so the XOR swizzle
+// while one is computed (D = 2 in the shipped instances: a plain double buffer, which leaves LDS and registers for
+// three or four workgroups per compute unit).  An LDS-direct load writes lane l's 16 bytes at base + 16*l, so the XOR swizzle
 // that keeps the fragment reads free of bank conflicts is applied to the global address each lane fetches.
 // The MFMA takes the weight fragment as its first operand, so a lane ends up with four consecutive output
 // columns of one token row and the epilogue stores 16 bytes per lane.
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
     constexpr int B_TILES = BN / 16;           // weight tiles per 256 columns
     constexpr int B_DMA = (B_TILES + 3) / 4;   // per wavefront (the last ones may repeat a tile)
     constexpr int B_STAGE = B_TILES * 1024;
-    static_assert(A_STAGE % 4096 == 0 && WTM % 16 == 0 && WTN % 16 == 0 && D >= 3, "tile shape");
+    static_assert(A_STAGE % 4096 == 0 && WTM % 16 == 0 && WTN % 16 == 0 && D >= 2, "tile shape");
     static_assert(dma_in_flight<0, P, A_DMA, B_DMA>() < 64 && dma_in_flight<1, P, A_DMA, B_DMA>() < 64, "vmcnt range");
 
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [D][A_STAGE] then [NB][B_STAGE]
@@ -775,14 +776,17 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
     if (!dma_ok) return BITNET_HIP_UNSUPPORTED;
     for (int j = nproj; j < GEMM_MAX_PROJ; ++j) p.proj[j] = p.proj[nproj - 1];
     p.nproj = nproj; p.a = a; p.a_sum = a_sum; p.a_scale = a_scale; p.m = (int)m; p.k = (int)k; p.kt_count = (int)k_tiles(k);
-    // Three shapes of the LDS-direct kernel, chosen by how many 128 x 160 tiles the outputs hold
-    // (256 compute units; the MFMA pipe of a SIMD needs two resident wavefronts to stay busy):
-    //   four or more tiles per compute unit  -> 128 x 160, two workgroups of 4 wavefronts per compute unit;
+    // Three shapes of the LDS-direct kernel, chosen by how many 128 x 160 tiles the outputs hold (256 compute
+    // units; the MFMA pipe of a SIMD needs two or more resident wavefronts to stay busy).  Measured:
+    //   2.5 or more tiles per compute unit   -> 128 x 160, three workgroups of 4 wavefronts per compute unit, two
+    //                                           activation stages each (more resident wavefronts beat deeper
+    //                                           pipelines: 2.45 POP/s at 8192 x 2560 x 6912, against 2.23 with two
+    //                                           workgroups of three stages);
     //   between a half and one tile per unit -> 128 x 160, one workgroup of 8 wavefronts (k split inside it);
-    //   otherwise                            -> 64 x 160, three workgroups of 4 wavefronts per compute unit.
-    if (tiles >= 1024) return launch_dma<128, 160, 3, 2>(p, stream);
+    //   otherwise                            -> 64 x 160, four workgroups of 4 wavefronts per compute unit.
+    if (tiles >= 640) return launch_dma<128, 160, 2, 3>(p, stream);
     if (tiles >= 128 && tiles <= 256) return launch_dma8<128, 160>(p, stream);
-    return launch_dma<64, 160, 3, 3>(p, stream);
+    return launch_dma<64, 160, 2, 4>(p, stream);
 }
 
 int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_sum, size_t m, size_t n, size_t k,

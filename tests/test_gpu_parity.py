@@ -336,7 +336,7 @@ def test_prefill_gemm_full_size(n, k, with_sum):
 def test_gemm_ragged_shapes_both_kernels(m, n, k):
     """Token counts, widths and depths that do not fill the MFMA tiles, with bias and residual; with row sums
     (LDS-direct kernels where k allows it: the sizes cover the 64 x 160 tiles, the eight-wavefront 128 x 160
-    workgroups (129..256 tiles) and the two-per-compute-unit 128 x 160 workgroups (1024 tiles and more)) and
+    workgroups (128..256 tiles) and the four-wavefront 128 x 160 workgroups (640 tiles and more)) and
     without."""
     rng = np.random.default_rng(m + 10 * n + 100 * k)
     packed, ws, a, a_scale = make_problem(rng, m, n, k, full_range=True)
