@@ -782,10 +782,10 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
     //                                           activation stages each (more resident wavefronts beat deeper
     //                                           pipelines: 2.45 POP/s at 8192 x 2560 x 6912, against 2.23 with two
     //                                           workgroups of three stages);
-    //   between a half and one tile per unit -> 128 x 160, one workgroup of 8 wavefronts (k split inside it);
+    //   0.75 to one tile per compute unit    -> 128 x 160, one workgroup of 8 wavefronts (k split inside it);
     //   otherwise                            -> 64 x 160, four workgroups of 4 wavefronts per compute unit.
     if (tiles >= 640) return launch_dma<128, 160, 2, 3>(p, stream);
-    if (tiles >= 128 && tiles <= 256) return launch_dma8<128, 160>(p, stream);
+    if (tiles >= 192 && tiles <= 256) return launch_dma8<128, 160>(p, stream);
     return launch_dma<64, 160, 2, 4>(p, stream);
 }
 

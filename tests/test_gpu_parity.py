@@ -331,12 +331,12 @@ def test_prefill_gemm_full_size(n, k, with_sum):
 
 
 @pytest.mark.parametrize("m,n,k", [(96, 160, 512), (100, 33, 512), (257, 170, 768), (130, 6912, 2560), (300, 16, 256),
-                                   (128, 48, 300), (200, 200, 2561), (1000, 2602, 768), (1030, 2560, 512),
+                                   (128, 48, 300), (200, 200, 2561), (1500, 2602, 768), (1600, 2560, 512),
                                    (4100, 5002, 512)])
 def test_gemm_ragged_shapes_both_kernels(m, n, k):
     """Token counts, widths and depths that do not fill the MFMA tiles, with bias and residual; with row sums
     (LDS-direct kernels where k allows it: the sizes cover the 64 x 160 tiles, the eight-wavefront 128 x 160
-    workgroups (128..256 tiles) and the four-wavefront 128 x 160 workgroups (640 tiles and more)) and
+    workgroups (192..256 tiles) and the four-wavefront 128 x 160 workgroups (640 tiles and more)) and
     without."""
     rng = np.random.default_rng(m + 10 * n + 100 * k)
     packed, ws, a, a_scale = make_problem(rng, m, n, k, full_range=True)
