@@ -323,8 +323,7 @@ __device__ __forceinline__ void run_phase(const StackParams &p, const uint4 (&wr
                 int i, kt;
                 tile_of(P, T, i, kt);
                 int acc = dot64(wreg[u], lds_a + kt * 16 + kq, 0);
-                acc += __shfl_xor(acc, 16, 64);
-                acc += __shfl_xor(acc, 32, 64);
+                acc = sum_over_lane_groups(acc);
                 if (lane < TILE_ROWS) sh.red[T][lane] = acc;
             }
         }

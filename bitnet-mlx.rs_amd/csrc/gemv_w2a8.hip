@@ -253,8 +253,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
     // the four lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
 #pragma unroll
     for (int t = 0; t < MB; ++t) {
-        acc[t] += __shfl_xor(acc[t], 16, 64);
-        acc[t] += __shfl_xor(acc[t], 32, 64);
+        acc[t] = sum_over_lane_groups(acc[t]);
     }
     if (lane < TILE_ROWS) {
 #pragma unroll
@@ -314,6 +313,12 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
         const int c = min(tid + 256 * i, chunks - 1);
         v[i] = load_chunk<MODE, true>(p.src, 0, c);
     }
+    // what the epilogue threads need from memory (weight scale, bias, residual of their output row) is requested
+    // now as well, so that its latency is not paid at the end
+    const int e_n = min((rb0 + (tid >> 4)) * TILE_ROWS + (tid & 15), P.n - 1);  // meaningful for tid < 16 * RBW
+    const float e_ws = P.out ? *P.w_scale : 0.0f;
+    const float e_bias = P.bias ? P.bias[e_n] : 0.0f;
+    const float e_res = P.residual ? P.residual[e_n] : 0.0f;
     if constexpr (NORM) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) gm[i] = load_gamma_chunk(p.src, min(tid + 256 * i, chunks - 1), true);
@@ -382,8 +387,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
             if (kt < p.kt_count) acc = dot64(wt[r][u], lds_a + kt * 16 + kq, acc);
         }
         // the four lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
-        acc += __shfl_xor(acc, 16, 64);
-        acc += __shfl_xor(acc, 32, 64);
+        acc = sum_over_lane_groups(acc);
         if (lane < TILE_ROWS) red[wave][r][lane] = acc;
     }
     lds_barrier();
@@ -400,10 +404,10 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
             const int total = red[0][r][row] + red[1][r][row] + red[2][r][row] + red[3][r][row] - asum;
             if (P.acc) P.acc[n] = total;
             if (P.out) {
-                float y = f32_mul((float)total, *P.w_scale);
+                float y = f32_mul((float)total, e_ws);
                 y = f32_div(y, scale);
-                if (P.bias) y = f32_add(y, P.bias[n]);
-                if (P.residual) y = f32_add(y, P.residual[n]);
+                if (P.bias) y = f32_add(y, e_bias);
+                if (P.residual) y = f32_add(y, e_res);
                 P.out[n] = y;
             }
         }
@@ -567,8 +571,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
     // sum_k a[row, k] over this wavefront's tiles: lanes lr, lr+16, lr+32, lr+48 hold the four column groups
 #pragma unroll
     for (int g = 0; g < MT; ++g) {
-        rowsum[g] += __shfl_xor(rowsum[g], 16, 64);
-        rowsum[g] += __shfl_xor(rowsum[g], 32, 64);
+        rowsum[g] = sum_over_lane_groups(rowsum[g]);
         if (lane < 16) red_sum[wave][g][lane] = rowsum[g];
     }
     if (wave > 0) {

@@ -17,7 +17,7 @@
 //   p[l] += p[l ^ off], off = 1,2,4,8,16,32; the four group sums are added as ((s0 + s1) + s2) + s3.
 //   (After the step with offset `off` all lanes of an aligned group of 2*off lanes hold the same value, so a
 //   step may fetch its operand from ANY lane of the partner group: the kernels use DPP quad permutes and row
-//   mirrors for offsets 1..8, a swizzle for 16 and a shuffle for 32.)
+//   mirrors for offsets 1..8 and the row / half swap instructions for 16 and 32.)
 //   A 256-thread workgroup maps thread = virtual lane; a single wavefront keeps 4 partials per lane
 //   (virtual lanes l, l+64, l+128, l+192).  Elements past K count as 0.
 // BITNET_HIP_SUM_SEQUENTIAL is the reference's literal running sum over k ascending.
@@ -56,8 +56,33 @@ __device__ __forceinline__ int dpp_i32(int v)
 {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
 }
-__device__ __forceinline__ int xchg16_i32(int v) { return __builtin_amdgcn_ds_swizzle(v, (0x10 << 10) | 0x1f); }  // l ^ 16
-__device__ __forceinline__ int xchg32_i32(int v) { return __shfl_xor(v, 32, 64); }                                 // l ^ 32
+// Offsets 16 and 32 without a trip through LDS: gfx950's row and half swaps.  With both operands holding p,
+// v_permlane16_swap leaves (rows 0,0,2,2 of p) in the first and (rows 1,1,3,3) in the second, v_permlane32_swap
+// (lower half twice) and (upper half twice): every lane then holds its own value in one of them and its partner's
+// in the other, and the combining operations here are commutative.  (Inline asm: the compiler's builtin for these
+// instructions folds the two results into one.  The s_nop covers the wait states between a VALU write of the
+// operands and the swap.)
+template <typename T>
+__device__ __forceinline__ void swap_rows16(T &a, T &b)
+{
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+template <typename T>
+__device__ __forceinline__ void swap_halves32(T &a, T &b)
+{
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+
+// 4-element sum over lanes l, l ^ 16, l ^ 32, l ^ 48 (the four column groups of a weight-tile row) in every lane.
+__device__ __forceinline__ int sum_over_lane_groups(int v)
+{
+    int a = v, b = v;
+    swap_rows16(a, b);
+    a += b;
+    b = a;
+    swap_halves32(a, b);
+    return a + b;
+}
 
 #define BITNET_WAVE_REDUCE(TYPE, NAME, COMBINE)                                                    \
     __device__ __forceinline__ TYPE NAME(TYPE p)                                                   \
@@ -67,8 +92,16 @@ __device__ __forceinline__ int xchg32_i32(int v) { return __shfl_xor(v, 32, 64);
         p = step(p, dpp_i32<0x4E>(__builtin_bit_cast(int, p)));                                    \
         p = step(p, dpp_i32<0x141>(__builtin_bit_cast(int, p)));                                   \
         p = step(p, dpp_i32<0x140>(__builtin_bit_cast(int, p)));                                   \
-        p = step(p, xchg16_i32(__builtin_bit_cast(int, p)));                                       \
-        p = step(p, xchg32_i32(__builtin_bit_cast(int, p)));                                       \
+        {                                                                                          \
+            TYPE a = p, b = p;                                                                     \
+            swap_rows16(a, b);                                                                     \
+            p = COMBINE;                                                                           \
+        }                                                                                          \
+        {                                                                                          \
+            TYPE a = p, b = p;                                                                     \
+            swap_halves32(a, b);                                                                   \
+            p = COMBINE;                                                                           \
+        }                                                                                          \
         return p;                                                                                  \
     }
 BITNET_WAVE_REDUCE(float, wave_sum_f32, f32_add(a, b))
