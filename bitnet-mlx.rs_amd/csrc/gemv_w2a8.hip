@@ -491,6 +491,18 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         }
     };
 
+    // scales the epilogue will need (result register i of a lane belongs to token 16g + 4*(lane/16) + i): requested
+    // now, so that their latency is not paid at the end
+    const float ws = P.out ? *P.w_scale : 0.0f;
+    float e_scale[MT][4];
+#pragma unroll
+    for (int g = 0; g < MT; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = 16 * g + lg * 4 + i;
+            e_scale[g][i] = (P.out && t < p.m) ? p.a_scale[t] : 1.0f;
+        }
+
     v4i acc[RB][MT];
     int rowsum[MT];
 #pragma unroll
@@ -584,7 +596,6 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
     }
     lds_barrier();
     if (wave == 0) {
-        const float ws = P.out ? *P.w_scale : 0.0f;
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             const int n = (rb0 + r) * TILE_ROWS + lr;  // result register i of lane l is C[4*(l/16) + i][l mod 16]
@@ -600,7 +611,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
                         const size_t o = (size_t)t * P.n + n;
                         if (P.acc) P.acc[o] = total;
                         if (P.out) {
-                            float v = f32_div(f32_mul((float)total, ws), p.a_scale[t]);
+                            float v = f32_div(f32_mul((float)total, ws), e_scale[g][i]);
                             if (P.bias) v = f32_add(v, P.bias[n]);
                             if (P.residual) v = f32_add(v, P.residual[o]);
                             P.out[o] = v;
