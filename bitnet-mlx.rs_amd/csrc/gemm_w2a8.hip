@@ -70,6 +70,7 @@ struct GemmParams {
     int m, n, k;
     int kt_count;   // 256-column weight tiles per row block
     int tiles_m, tiles_n;
+    int rotate;     // gemm_dma_kernel: every workgroup of the launch is resident at once (see there)
 };
 
 constexpr int STAGE_K = 256;              // columns per pipeline stage = one weight tile
@@ -264,12 +265,187 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p)
 // loop invariant, so advancing a stage costs two scalar additions and no vector instruction.
 __device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_off)
 {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1\n\t" : : "v"(voff), "s"(sbase), "s"(lds_off) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1\n\t"
+                 : : "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory", "m0");
+}
+// s_setprio takes an immediate.
+__device__ __forceinline__ void set_wave_priority(int pr)
+{
+    if (pr == 0) __builtin_amdgcn_s_setprio(0);
+    else if (pr == 1) __builtin_amdgcn_s_setprio(1);
+    else if (pr == 2) __builtin_amdgcn_s_setprio(2);
+    else __builtin_amdgcn_s_setprio(3);
 }
 template <int N>
 __device__ __forceinline__ void wait_vm()
 {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// The same for 4 bytes per lane: lane l lands at base + 4*l.
+__device__ __forceinline__ void dma4(const void *sbase, uint32_t voff, uint32_t lds_off)
+{
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1\n\t"
+                 : : "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory", "m0");
+}
+
+// Per-row epilogue operands of a BM-row tile, fetched into LDS by LDS-direct loads (no registers are held across
+// the k loop): a_sum[BM] as int32, then a_scale[BM].  Wavefront w < BM/64 fetches rows 64*w .. of a_sum, the
+// next BM/64 wavefronts the same rows of a_scale (skipped when there is no f32 output and hence no a_scale).
+// Rows past m re-read row m-1.  The reader waits for vmcnt(0) and a workgroup barrier first.
+template <int BM>
+constexpr int rowp_bytes() { return BM * 8; }
+template <int BM>
+__device__ __forceinline__ void fetch_row_operands(const GemmParams &p, int m0, int wave, int lane, uint32_t lds_rowp)
+{
+    constexpr int CH = BM / 64;
+    static_assert(BM % 64 == 0, "row operand chunks");
+    if (wave < 2 * CH) {
+        const int chunk = wave < CH ? wave : wave - CH;
+        int grow = m0 + chunk * 64 + lane;
+        if (grow >= p.m) grow = p.m - 1;
+        if (wave < CH) dma4(p.a_sum, (uint32_t)grow * 4u, lds_rowp + chunk * 256);
+        else if (p.a_scale) dma4(p.a_scale, (uint32_t)grow * 4u, lds_rowp + BM * 4 + chunk * 256);
+    }
+}
+
+// The epilogue of one wavefront's fragments on the usual path: f32 output only, n % 4 == 0, w_scale and every
+// a_scale of the tile suited to the short division (the caller checks).  Straight-line code: per output element
+// a subtraction, a conversion, two multiplications, two FMAs and a sign copy; one 16-byte store per fragment row.
+// Fragment i of lane l holds token row rows[i], columns col0 + 16*j + 0..3.  FULL: the tile lies inside the
+// matrix, no bounds checks.  EXTRA: bias and / or residual may be present.
+template <int NI, int FN, bool FULL, bool EXTRA>
+__device__ __forceinline__ void store_fragments_fast(const v4i (&acc)[NI][FN], const int (&rs)[NI], const float (&as)[NI],
+                                                     const float (&rcp)[NI], float ws, const GemmProjDev &PJ, int m,
+                                                     const int (&rows)[NI], int col0)
+{
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        if (!FULL && rows[i] >= m) continue;
+        const size_t o = (size_t)rows[i] * PJ.n + col0;
+        float *orow = PJ.out + o;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            if (!FULL && col0 + j * 16 >= PJ.n) continue;  // n % 4 == 0: a fragment row is inside or outside as a whole
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                v[r] = div_by_invariant_unchecked(f32_mul((float)(acc[i][j][r] - rs[i]), ws), as[i], rcp[i]);
+            if (EXTRA) {
+                if (PJ.bias) {
+                    const float4 b = *reinterpret_cast<const float4 *>(PJ.bias + col0 + j * 16);
+                    v[0] = f32_add(v[0], b.x); v[1] = f32_add(v[1], b.y); v[2] = f32_add(v[2], b.z); v[3] = f32_add(v[3], b.w);
+                }
+                if (PJ.residual) {
+                    const float4 q = *reinterpret_cast<const float4 *>(PJ.residual + o + j * 16);
+                    v[0] = f32_add(v[0], q.x); v[1] = f32_add(v[1], q.y); v[2] = f32_add(v[2], q.z); v[3] = f32_add(v[3], q.w);
+                }
+            }
+            *reinterpret_cast<float4 *>(orow + j * 16) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+    }
+}
+
+// The epilogue for every other case (int32 accumulator output, n % 4 != 0, scales outside the short division's
+// range): the same arithmetic, choices made per fragment row, a_sum and a_scale read from global memory.
+template <int NI, int FN>
+__device__ __forceinline__ void store_fragments_general(const v4i (&acc)[NI][FN], const int (&rows)[NI], int col0, float ws,
+                                                        bool ws_fast, const GemmProjDev &PJ, const GemmParams &p)
+{
+    const bool vec_ok = (PJ.n & 3) == 0;  // 16-byte alignment of out[row][4c]
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int row = rows[i];
+        const bool row_ok = row < p.m;
+        const int rs = row_ok ? p.a_sum[row] : 0;
+        const float as = (PJ.out && row_ok) ? p.a_scale[row] : 1.0f;
+        const float as_recip = f32_div(1.0f, as);
+        // the short division needs a well-behaved divisor (per row) and dividends in range: float(total) * ws
+        // is zero or has ws's exponent plus at most 24, so one check on ws covers them.  The choice is made
+        // per wavefront so that the usual case runs no plain division at all.
+        const bool row_fast = ws_fast && invariant_divisor_ok(as);
+        const bool wave_fast = __builtin_amdgcn_ballot_w64(!row_fast) == 0;
+        if (!row_ok) continue;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int col = col0 + j * 16;
+            if (col >= PJ.n) continue;
+            const size_t o = (size_t)row * PJ.n + col;
+            int tot[4];
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                tot[r] = acc[i][j][r] - rs;
+                const float scaled = f32_mul((float)tot[r], ws);
+                v[r] = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
+            }
+            if (vec_ok) {  // col + 3 < n follows from n % 4 == 0
+                if (PJ.acc) *reinterpret_cast<int4 *>(PJ.acc + o) = make_int4(tot[0], tot[1], tot[2], tot[3]);
+                if (PJ.out) {
+                    if (PJ.bias) {
+                        const float4 b = *reinterpret_cast<const float4 *>(PJ.bias + col);
+                        v[0] = f32_add(v[0], b.x); v[1] = f32_add(v[1], b.y); v[2] = f32_add(v[2], b.z); v[3] = f32_add(v[3], b.w);
+                    }
+                    if (PJ.residual) {
+                        const float4 q = *reinterpret_cast<const float4 *>(PJ.residual + o);
+                        v[0] = f32_add(v[0], q.x); v[1] = f32_add(v[1], q.y); v[2] = f32_add(v[2], q.z); v[3] = f32_add(v[3], q.w);
+                    }
+                    *reinterpret_cast<float4 *>(PJ.out + o) = make_float4(v[0], v[1], v[2], v[3]);
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (col + r >= PJ.n) continue;
+                    if (PJ.acc) PJ.acc[o + r] = tot[r];
+                    if (PJ.out) {
+                        float y = v[r];
+                        if (PJ.bias) y = f32_add(y, PJ.bias[col + r]);
+                        if (PJ.residual) y = f32_add(y, PJ.residual[o + r]);
+                        PJ.out[o + r] = y;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// The whole epilogue of one wavefront.  Fragment i of lane l holds token row m0 + lrows[i] (lrows: row inside the
+// BM-row tile), columns col0 + 16*j + 0..3.  rowp is the LDS copy of the tile's a_sum and a_scale
+// (fetch_row_operands), complete and visible: the caller has waited for vmcnt(0) and passed a workgroup barrier.
+// full: the workgroup's tile lies inside the matrix.
+template <int BM, int NI, int FN>
+__device__ __forceinline__ void finish_fragments(const v4i (&acc)[NI][FN], const int (&lrows)[NI], int m0, int col0, bool full,
+                                                 const uint8_t *rowp, const GemmProjDev &PJ, const GemmParams &p)
+{
+    const float ws = PJ.out ? *PJ.w_scale : 0.0f;
+    const unsigned ws_expo = (__builtin_bit_cast(unsigned, ws) >> 23) & 0xffu;
+    const bool ws_fast = ws > 0.0f && ws_expo > 64u && ws_expo < 160u;
+    int rows[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) rows[i] = m0 + lrows[i];
+    if (PJ.out && !PJ.acc && (PJ.n & 3) == 0 && ws_fast) {
+        const int *sum_l = reinterpret_cast<const int *>(rowp);
+        const float *scale_l = reinterpret_cast<const float *>(rowp + BM * 4);
+        int rs[NI];
+        float as[NI], rcp[NI];
+        bool ok = true;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            rs[i] = sum_l[lrows[i]];
+            as[i] = scale_l[lrows[i]];
+            rcp[i] = f32_div(1.0f, as[i]);
+            ok = ok && invariant_divisor_ok(as[i]);
+        }
+        if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
+            const bool extra = PJ.bias != nullptr || PJ.residual != nullptr;
+            if (full && !extra) store_fragments_fast<NI, FN, true, false>(acc, rs, as, rcp, ws, PJ, p.m, rows, col0);
+            else if (full) store_fragments_fast<NI, FN, true, true>(acc, rs, as, rcp, ws, PJ, p.m, rows, col0);
+            else if (!extra) store_fragments_fast<NI, FN, false, false>(acc, rs, as, rcp, ws, PJ, p.m, rows, col0);
+            else store_fragments_fast<NI, FN, false, true>(acc, rs, as, rcp, ws, PJ, p.m, rows, col0);
+            return;
+        }
+    }
+    store_fragments_general<NI, FN>(acc, rows, col0, ws, ws_fast, PJ, p);
 }
 
 constexpr int DMA_SK = 128;  // columns per activation stage; a 256-column weight tile serves two stages
@@ -413,7 +589,14 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
 
     // Loads retire in issue order.  At the top of stage s its own group must have landed; the groups of the
     // P - 1 later stages stay in flight.  The last P - 1 stages, with fewer groups behind them, drain everything.
+    // When the whole launch is resident at once (OCC workgroups on every compute unit, all started together), the
+    // hardware's oldest-first choice among wavefronts lets the OCC workgroups of a compute unit finish one after the
+    // other, the last one running alone at a fraction of the MFMA rate.  Workgroup ids b, b + 256, ... share a
+    // compute unit; rotating their wavefront priorities every k-tile keeps them level (measured: 5 % at
+    // 2048 x 6912 x 2560).  With several rounds of workgroups the staggered finish is wanted and nothing is done.
+    const int rank = blockIdx.x >> 8;
     for (int s = 0; s < nstage; s += 2) {
+        if (p.rotate) set_wave_priority((rank + (s >> 1)) % OCC);
         if (s + P <= nstage) wait_vm<dma_in_flight<0, P, A_DMA, B_DMA>()>(); else wait_vm<0>();
         __syncthreads();
         if (s + P < nstage) issue(s + P);
@@ -422,67 +605,19 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
         if (s + 1 + P <= nstage) wait_vm<dma_in_flight<1, P, A_DMA, B_DMA>()>(); else wait_vm<0>();
         __syncthreads();
         if (s + 1 + P < nstage) issue(s + 1 + P);
+        // In the last stage the buffer of the stage before it is free: the per-row epilogue operands land there
+        // while the last MFMAs run.
+        else if (s + 2 == nstage) fetch_row_operands<BM>(p, m0, wave, lane, lds_base + (s % D) * A_STAGE);
         compute(s + 1, true);
     }
-
-    const float ws = PJ.out ? *PJ.w_scale : 0.0f;
-    const unsigned ws_expo = (__builtin_bit_cast(unsigned, ws) >> 23) & 0xffu;
-    const bool ws_fast = ws > 0.0f && ws_expo > 64u && ws_expo < 160u;
-    const bool vec_ok = (PJ.n & 3) == 0;  // 16-byte alignment of out[row][4c]
+    const uint32_t ROWP = ((nstage - 2) % D) * A_STAGE;
+    static_assert(rowp_bytes<BM>() <= A_STAGE, "row operands fit an activation stage");
+    wait_vm<0>();
+    __syncthreads();
+    int lrows[FM];
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
-        const int row = m0 + wm * WTM + i * 16 + lr;
-        const bool row_ok = row < p.m;
-        const int rs = row_ok ? p.a_sum[row] : 0;
-        const float as = (PJ.out && row_ok) ? p.a_scale[row] : 1.0f;
-        const float as_recip = f32_div(1.0f, as);
-        // the short division needs a well-behaved divisor (per row) and dividends in range: float(total) * ws
-        // is zero or has ws's exponent plus at most 24, so one check on ws covers them.  The choice is made
-        // per wavefront so that the usual case runs no plain division at all.
-        const bool row_fast = ws_fast && invariant_divisor_ok(as);
-        const bool wave_fast = __builtin_amdgcn_ballot_w64(!row_fast) == 0;
-        if (!row_ok) continue;
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const int col = n0 + wn * WTN + j * 16 + lg * 4;
-            if (col >= PJ.n) continue;
-            const size_t o = (size_t)row * PJ.n + col;
-            int tot[4];
-            float v[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                tot[r] = acc[i][j][r] - rs;
-                const float scaled = f32_mul((float)tot[r], ws);
-                v[r] = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
-            }
-            if (vec_ok) {  // col + 3 < n follows from n % 4 == 0
-                if (PJ.acc) *reinterpret_cast<int4 *>(PJ.acc + o) = make_int4(tot[0], tot[1], tot[2], tot[3]);
-                if (PJ.out) {
-                    if (PJ.bias) {
-                        const float4 b = *reinterpret_cast<const float4 *>(PJ.bias + col);
-                        v[0] = f32_add(v[0], b.x); v[1] = f32_add(v[1], b.y); v[2] = f32_add(v[2], b.z); v[3] = f32_add(v[3], b.w);
-                    }
-                    if (PJ.residual) {
-                        const float4 q = *reinterpret_cast<const float4 *>(PJ.residual + o);
-                        v[0] = f32_add(v[0], q.x); v[1] = f32_add(v[1], q.y); v[2] = f32_add(v[2], q.z); v[3] = f32_add(v[3], q.w);
-                    }
-                    *reinterpret_cast<float4 *>(PJ.out + o) = make_float4(v[0], v[1], v[2], v[3]);
-                }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if (col + r >= PJ.n) continue;
-                    if (PJ.acc) PJ.acc[o + r] = tot[r];
-                    if (PJ.out) {
-                        float y = v[r];
-                        if (PJ.bias) y = f32_add(y, PJ.bias[col + r]);
-                        if (PJ.residual) y = f32_add(y, PJ.residual[o + r]);
-                        PJ.out[o + r] = y;
-                    }
-                }
-            }
-        }
-    }
+    for (int i = 0; i < FM; ++i) lrows[i] = wm * WTM + i * 16 + lr;
+    finish_fragments<BM, FM, FN>(acc, lrows, m0, n0 + wn * WTN + lg * 4, m0 + BM <= p.m && n0 + BN <= PJ.n, lds + ROWP, PJ, p);
 }
 
 // Raising a kernel's dynamic LDS limit is needed once per process; a function-local static makes that once
@@ -501,8 +636,9 @@ int launch_dma(GemmParams p, hipStream_t stream)
     for (int j = 0; j < p.nproj; ++j) p.proj[j].tn_end = p.tiles_n += (p.proj[j].n + BN - 1) / BN;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
+    p.rotate = total <= 256 * OCC && total > 256;
     constexpr size_t lds = dma_lds_bytes<BM, BN, D>();
-    static_assert(lds <= 160 * 1024 && lds * OCC <= 160 * 1024, "LDS budget");
+    static_assert(lds <= 160 * 1024 && lds * OCC <= 160 * 1024 && OCC <= 4, "LDS budget, priorities 0..3");
     static const hipError_t attr = lds > 64 * 1024 ? raise_lds_limit(&gemm_dma_kernel<BM, BN, D, OCC>, lds) : hipSuccess;
     BITNET_HIP_TRY(attr);
     hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, D, OCC>), dim3(grid), dim3(256), lds, stream, p);
@@ -520,7 +656,7 @@ int launch_dma(GemmParams p, hipStream_t stream)
 // finishing half of the fragments.  A stage is one 256-column weight tile plus BM x 256 activation bytes.
 constexpr int D8_NST = 3;
 template <int BM, int BN>
-constexpr size_t dma8_lds_bytes() { return (size_t)D8_NST * (BM * 256 + (BN / 16) * 1024); }
+constexpr size_t dma8_lds_bytes() { return (size_t)D8_NST * (BM * 256 + (BN / 16) * 1024) + rowp_bytes<BM>(); }
 
 template <int BM, int BN>
 __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
@@ -597,6 +733,8 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j] = (v4i){0, 0, 0, 0};
 
+    constexpr uint32_t ROWP = D8_NST * STAGE;
+    fetch_row_operands<BM>(p, m0, wave, lane, lds_base + ROWP);
     issue(0);
     if (p.kt_count > 1) issue(1);
 
@@ -660,63 +798,17 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
             }
     }
 
-    const float ws = PJ.out ? *PJ.w_scale : 0.0f;
-    const unsigned ws_expo = (__builtin_bit_cast(unsigned, ws) >> 23) & 0xffu;
-    const bool ws_fast = ws > 0.0f && ws_expo > 64u && ws_expo < 160u;
-    const bool vec_ok = (PJ.n & 3) == 0;
+    // this group's finished fragments (kg is uniform over the wavefront)
+    constexpr int HALF = FM / 2;
+    v4i fin[HALF][FN];
+    int lrows[HALF];
 #pragma unroll
-    for (int ii = 0; ii < FM / 2; ++ii) {
-        const int i = kg == 0 ? ii : ii + FM / 2;
-        const int row = m0 + wm * WTM + i * 16 + lr;
-        const bool row_ok = row < p.m;
-        const int rs = row_ok ? p.a_sum[row] : 0;
-        const float as = (PJ.out && row_ok) ? p.a_scale[row] : 1.0f;
-        const float as_recip = f32_div(1.0f, as);
-        const bool row_fast = ws_fast && invariant_divisor_ok(as);
-        const bool wave_fast = __builtin_amdgcn_ballot_w64(!row_fast) == 0;
-        if (!row_ok) continue;
+    for (int ii = 0; ii < HALF; ++ii) {
+        lrows[ii] = wm * WTM + (ii + kg * HALF) * 16 + lr;
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const int col = n0 + wn * WTN + j * 16 + lg * 4;
-            if (col >= PJ.n) continue;
-            const size_t o = (size_t)row * PJ.n + col;
-            const v4i a4 = kg == 0 ? acc[ii][j] : acc[ii + FM / 2][j];
-            int tot[4];
-            float v[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                tot[r] = a4[r] - rs;
-                const float scaled = f32_mul((float)tot[r], ws);
-                v[r] = wave_fast ? div_by_invariant_unchecked(scaled, as, as_recip) : f32_div(scaled, as);
-            }
-            if (vec_ok) {
-                if (PJ.acc) *reinterpret_cast<int4 *>(PJ.acc + o) = make_int4(tot[0], tot[1], tot[2], tot[3]);
-                if (PJ.out) {
-                    if (PJ.bias) {
-                        const float4 b = *reinterpret_cast<const float4 *>(PJ.bias + col);
-                        v[0] = f32_add(v[0], b.x); v[1] = f32_add(v[1], b.y); v[2] = f32_add(v[2], b.z); v[3] = f32_add(v[3], b.w);
-                    }
-                    if (PJ.residual) {
-                        const float4 q = *reinterpret_cast<const float4 *>(PJ.residual + o);
-                        v[0] = f32_add(v[0], q.x); v[1] = f32_add(v[1], q.y); v[2] = f32_add(v[2], q.z); v[3] = f32_add(v[3], q.w);
-                    }
-                    *reinterpret_cast<float4 *>(PJ.out + o) = make_float4(v[0], v[1], v[2], v[3]);
-                }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if (col + r >= PJ.n) continue;
-                    if (PJ.acc) PJ.acc[o + r] = tot[r];
-                    if (PJ.out) {
-                        float y = v[r];
-                        if (PJ.bias) y = f32_add(y, PJ.bias[col + r]);
-                        if (PJ.residual) y = f32_add(y, PJ.residual[o + r]);
-                        PJ.out[o + r] = y;
-                    }
-                }
-            }
-        }
+        for (int j = 0; j < FN; ++j) fin[ii][j] = kg == 0 ? acc[ii][j] : acc[ii + HALF][j];
     }
+    finish_fragments<BM, HALF, FN>(fin, lrows, m0, n0 + wn * WTN + lg * 4, m0 + BM <= p.m && n0 + BN <= PJ.n, lds + ROWP, PJ, p);
 }
 
 template <int BM, int BN>

@@ -352,6 +352,27 @@ def test_gemm_ragged_shapes_both_kernels(m, n, k):
         assert np.array_equal(host(out), out_ref)
 
 
+@pytest.mark.parametrize("m,n,k", [(100, 172, 512), (257, 2560, 768), (1600, 2564, 512), (1990, 6900, 768),
+                                   (2048, 6912, 512), (1990, 6902, 512), (4100, 5000, 512)])
+@pytest.mark.parametrize("extras", [False, True], ids=["plain", "bias_residual"])
+def test_gemm_f32_only_epilogue_ragged(m, n, k, extras):
+    """f32 output without the int32 accumulators: the straight-line epilogue of the LDS-direct kernels (64 x 160,
+    eight-wavefront 128 x 160 and four-wavefront 128 x 160 workgroups), tiles cut by m and n, n not a multiple of 4 (general epilogue), and one activation scale outside the short division's
+    range (whole wavefronts fall back to the plain division)."""
+    rng = np.random.default_rng(7 * m + 3 * n + k + int(extras))
+    packed, ws, a, a_scale = make_problem(rng, m, n, k, full_range=True)
+    a_scale = a_scale.copy()
+    a_scale[m // 2] = np.float32(2.0) ** 100  # invariant_divisor_ok fails for this row
+    tiled = bh.retile_weights(dev(packed), n, k)
+    bias = rng.standard_normal(n, dtype=f32) if extras else None
+    res = rng.standard_normal((m, n), dtype=f32) if extras else None
+    out_ref = orc.epilogue(orc.gemm_w2a8(packed, a, n), ws, a_scale, bias, res)
+    a_sum = dev(a.astype(np.int32).sum(axis=1).astype(np.int32))
+    _, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale),
+                            dev(bias) if extras else None, dev(res) if extras else None, want_acc=False, a_sum=a_sum)
+    assert np.array_equal(host(out), out_ref)
+
+
 def test_bitlinear_forward_prefill_uses_quantiser_row_sums():
     """BitLinear.forward at a prefill token count: quantiser -> row sums -> LDS-direct GEMM, bit-exact."""
     rng = np.random.default_rng(77)
