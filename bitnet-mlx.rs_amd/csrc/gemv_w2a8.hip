@@ -430,7 +430,9 @@ struct GemvMfmaParams {
 // FAST: k is a multiple of 256 and the activations are 16-byte aligned.  Every load is then unconditional
 // (indices past the end are clamped, the values discarded), so the compiler can count the loads in flight
 // and the next batch of tiles really stays outstanding while the current one is multiplied.
-template <int RB, int MT, bool FAST>
+// ONE: the wavefront's k-tiles (at most 8: k <= 8192) form a single batch, requested as a whole at the start: one
+// memory latency instead of one per batch (RB = MT = 1 only, where the registers allow it).
+template <int RB, int MT, bool FAST, bool ONE = false>
 __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 {
     __shared__ int red[3][RB][MT][64][4];  // partial accumulators of wavefronts 1..3
@@ -503,6 +505,19 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
             e_scale[g][i] = (P.out && t < p.m) ? p.a_scale[t] : 1.0f;
         }
 
+    // bias and residual of the rows wavefront 0 will store (clamped indices; unused values are discarded)
+    float e_bias[RB], e_res[RB][MT][4];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+        const int n = min((rb0 + r) * TILE_ROWS + lr, P.n - 1);
+        e_bias[r] = (wave == 0 && P.bias) ? P.bias[n] : 0.0f;
+#pragma unroll
+        for (int g = 0; g < MT; ++g)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                e_res[r][g][i] = (wave == 0 && P.residual) ? P.residual[(size_t)min(16 * g + lg * 4 + i, p.m - 1) * P.n + n] : 0.0f;
+    }
+
     v4i acc[RB][MT];
     int rowsum[MT];
 #pragma unroll
@@ -512,11 +527,12 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         for (int r = 0; r < RB; ++r) acc[r][g] = (v4i){0, 0, 0, 0};
     }
 
-    constexpr int PF = RB * MT == 1 ? 4 : (RB * MT == 2 ? 3 : (MT <= 2 ? 2 : 1));  // bounded by the register file
+    static_assert(!ONE || RB * MT == 1, "single batch: one row block, one token group");
+    constexpr int PF = ONE ? 8 : (RB * MT == 1 ? 4 : (RB * MT == 2 ? 3 : (MT <= 2 ? 2 : 1)));  // bounded by the register file
     // All loads of a batch of PF k-tiles are issued before the first MFMA of the batch, and the next
     // batch is requested while the current one is computed: the weight stream is what the kernel waits for.
-    uint4 wcur[PF][RB], wnxt[PF][RB];
-    v4i acur[PF][MT][4], anxt[PF][MT][4];
+    uint4 wcur[PF][RB], wnxt[ONE ? 1 : PF][RB];
+    v4i acur[PF][MT][4], anxt[ONE ? 1 : PF][MT][4];
     auto load_batch = [&](int kt0, uint4 (&w)[PF][RB], v4i (&a)[PF][MT][4]) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
@@ -561,22 +577,27 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         }
     };
     load_batch(wave, wcur, acur);
+    if constexpr (ONE) {
+        compute_batch(wave);
+    } else
     for (int kt0 = wave; kt0 < p.kt_count; kt0 += 4 * PF) {
         // two straight-line bodies, so that the wait before the MFMAs is for this batch only in both of them
-        if (kt0 + 4 * PF < p.kt_count) {  // uniform over the wavefront
-            load_batch(kt0 + 4 * PF, wnxt, anxt);
-            compute_batch(kt0);
+        if constexpr (!ONE) {
+            if (kt0 + 4 * PF < p.kt_count) {  // uniform over the wavefront
+                load_batch(kt0 + 4 * PF, wnxt, anxt);
+                compute_batch(kt0);
 #pragma unroll
-            for (int u = 0; u < PF; ++u) {
+                for (int u = 0; u < PF; ++u) {
 #pragma unroll
-                for (int r = 0; r < RB; ++r) wcur[u][r] = wnxt[u][r];
+                    for (int r = 0; r < RB; ++r) wcur[u][r] = wnxt[u][r];
 #pragma unroll
-                for (int g = 0; g < MT; ++g)
+                    for (int g = 0; g < MT; ++g)
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) acur[u][g][t] = anxt[u][g][t];
+                        for (int t = 0; t < 4; ++t) acur[u][g][t] = anxt[u][g][t];
+                }
+            } else {
+                compute_batch(kt0);
             }
-        } else {
-            compute_batch(kt0);
         }
     }
 
@@ -612,8 +633,8 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
                         if (P.acc) P.acc[o] = total;
                         if (P.out) {
                             float v = f32_div(f32_mul((float)total, ws), e_scale[g][i]);
-                            if (P.bias) v = f32_add(v, P.bias[n]);
-                            if (P.residual) v = f32_add(v, P.residual[o]);
+                            if (P.bias) v = f32_add(v, e_bias[r]);
+                            if (P.residual) v = f32_add(v, e_res[r][g][i]);
                             P.out[o] = v;
                         }
                     }
@@ -732,7 +753,15 @@ int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const floa
     for (int j = nproj; j < GEMV_MAX_PROJ; ++j) p.proj[j] = p.proj[nproj - 1];
     p.nproj = nproj; p.a = a; p.a_scale = a_scale; p.m = (int)m; p.k = (int)k; p.kt_count = (int)k_tiles(k);
     if (end == 0) return BITNET_HIP_OK;
-    if (k % TILE_K == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0)
+    const bool fast = k % TILE_K == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0;
+    if constexpr (RB * MT == 1) {
+        if (fast && p.kt_count > 16 && p.kt_count <= 32) {  // more than one batch of 4 tiles per wavefront, at most one of 8
+            hipLaunchKernelGGL((gemv_mfma_kernel<1, 1, true, true>), dim3((unsigned)end), dim3(256), 0, stream, p);
+            BITNET_HIP_CHECK_LAUNCH("gemv_mfma_kernel");
+            return BITNET_HIP_OK;
+        }
+    }
+    if (fast)
         hipLaunchKernelGGL((gemv_mfma_kernel<RB, MT, true>), dim3((unsigned)end), dim3(256), 0, stream, p);
     else
         hipLaunchKernelGGL((gemv_mfma_kernel<RB, MT, false>), dim3((unsigned)end), dim3(256), 0, stream, p);
