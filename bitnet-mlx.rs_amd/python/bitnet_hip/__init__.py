@@ -375,8 +375,10 @@ class BitLinear:
         return buf, s.value
 
     def forward(self, x: torch.Tensor, gamma: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None,
-                debug: bool = False, stream=None):
-        """BitLinearForward::forward (forward.rs:55-92).  x: [m,in] or [b,s,in] f32 on the GPU."""
+                debug: bool = False, stream=None, out: Optional[torch.Tensor] = None,
+                workspace: Optional[torch.Tensor] = None):
+        """BitLinearForward::forward (forward.rs:55-92).  x: [m,in] or [b,s,in] f32 on the GPU.  out and workspace
+        (uint8, at least workspace_size(m) bytes) may be supplied by callers that must not allocate per call."""
         _dev(x, torch.float32, "input")
         lib = load_library()
         dims = (C.c_size_t * max(x.dim(), 1))(*x.shape)
@@ -385,7 +387,12 @@ class BitLinear:
         m = 1
         for d in x.shape[:-1]:
             m *= d
-        out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
+        if out is None:
+            out = torch.empty(out_shape, dtype=torch.float32, device=x.device)
+        else:
+            _dev(out, torch.float32, "out")
+            if tuple(out.shape) != tuple(out_shape) or not out.is_contiguous():
+                raise BitLinearError(SHAPE_MISMATCH, "out", list(out_shape), list(out.shape))
         q = a_scale = acc = None
         if debug and x.dim() in (2, 3) and x.shape[-1] == self.config.in_features:
             q = torch.empty((m, self.config.in_features), dtype=torch.int8, device=x.device)
@@ -394,13 +401,21 @@ class BitLinear:
         # scratch for the quantised activations comes from torch's caching allocator (the library would otherwise
         # allocate stream-ordered memory itself on every call)
         ws_bytes = lib.bitnet_hip_bitlinear_workspace_size(self._h, m) if m > 0 else 0
-        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=x.device) if ws_bytes else None
+        if workspace is not None:
+            _dev(workspace, torch.uint8, "workspace")
+            ws, ws_bytes = workspace, workspace.numel()  # the library checks the size
+        else:
+            ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=x.device) if ws_bytes else None
         _check(lib.bitnet_hip_bitlinear_forward(self._h, _ptr(x), dims, x.dim(), _ptr(gamma), self.config.rms_norm_eps,
                                                 self.config.sum_order, _ptr(residual), _ptr(out), _ptr(ws), ws_bytes,
                                                 _ptr(q), _ptr(a_scale), _ptr(acc), _stream(stream)))
         if debug:
             return out, q, a_scale, acc
         return out
+
+    def workspace_size(self, m: int) -> int:
+        """Bytes of scratch forward() needs for m token rows."""
+        return int(load_library().bitnet_hip_bitlinear_workspace_size(self._h, m)) if m > 0 else 0
 
     def matmul_quantized(self, a: torch.Tensor, a_scale: torch.Tensor, residual: Optional[torch.Tensor] = None,
                          want_acc: bool = False, out: Optional[torch.Tensor] = None, stream=None,

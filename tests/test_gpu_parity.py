@@ -373,6 +373,44 @@ def test_gemm_f32_only_epilogue_ragged(m, n, k, extras):
     assert np.array_equal(host(out), out_ref)
 
 
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_forward_in_hip_graph_replays_match_eager(m):
+    """forward() with caller-supplied output and workspace allocates nothing and records no memset, so a caller may
+    capture it into a HIP graph: three replays, with eager work and synchronisations between them, each bit-equal
+    to the eager result and to the oracle."""
+    rng = np.random.default_rng(900 + m)
+    n, k = 2560, 6912
+    w = synth_weights(rng, n, k)
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "graph")
+    layer.update_weights(dev(w))
+    qw, ws_ = orc.quantize_weights_absmean(w)
+    x = synth_activations(rng, m, k, outliers=True)
+    ref = orc.bitlinear_forward(x, orc.pack_2bit(qw), n, ws_)[0]
+    xd = dev(x)
+    y = torch.empty((m, n), device="cuda", dtype=torch.float32)
+    scratch = torch.empty((max(layer.workspace_size(m), 16),), device="cuda", dtype=torch.uint8)
+    layer.forward(xd, out=y, workspace=scratch)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(y), ref)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer.forward(xd, out=y, workspace=scratch)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        layer.forward(xd, out=y, workspace=scratch)
+        layer.forward(xd, out=y, workspace=scratch)
+    for _ in range(3):
+        y.zero_()
+        other = layer.forward(xd)  # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(y), ref)
+        assert np.array_equal(host(other), ref)
+
+
 def test_bitlinear_forward_prefill_uses_quantiser_row_sums():
     """BitLinear.forward at a prefill token count: quantiser -> row sums -> LDS-direct GEMM, bit-exact."""
     rng = np.random.default_rng(77)
