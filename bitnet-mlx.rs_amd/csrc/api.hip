@@ -272,6 +272,22 @@ int bitnet_hip_unpack_ternary_2bit(const uint8_t *packed, size_t count, int8_t *
     return launch_unpack_2bit(packed, count, q, as_stream(stream));
 }
 
+size_t bitnet_hip_base3_packed_size(size_t count) { return (count + 4) / 5; }
+
+int bitnet_hip_pack_ternary_base3(const int8_t *q, size_t count, uint8_t *packed, void *stream)
+{
+    if (count == 0) return BITNET_HIP_OK;
+    if (!q || !packed) return fail(BITNET_HIP_NULL_POINTER, "pack_ternary_base3: null buffer");
+    return launch_pack_base3(q, count, packed, as_stream(stream));
+}
+
+int bitnet_hip_unpack_ternary_base3(const uint8_t *packed, size_t count, int8_t *q, void *stream)
+{
+    if (count == 0) return BITNET_HIP_OK;
+    if (!q || !packed) return fail(BITNET_HIP_NULL_POINTER, "unpack_ternary_base3: null buffer");
+    return launch_unpack_base3(packed, count, q, as_stream(stream));
+}
+
 int bitnet_hip_quantize_weights(const float *w, size_t n, size_t k, int method, float threshold_factor,
                                 uint8_t *packed, float *w_scale, int8_t *q_i8, void *stream)
 {
@@ -443,6 +459,35 @@ int bitnet_hip_bitlinear_set_weights_packed(bitnet_hip_bitlinear *layer, const u
     int rc = launch_retile(layer->packed, n, k, BITNET_HIP_LAYOUT_OUT_IN, layer->tiled, s);
     if (rc != BITNET_HIP_OK) return rc;
     BITNET_HIP_TRY(hipStreamSynchronize(s));  // w_scale is read from the caller's stack
+    layer->has_weights = true;
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_bitlinear_set_weights_base3(bitnet_hip_bitlinear *layer, const uint8_t *packed, size_t packed_len,
+                                           float w_scale, int on_device, void *stream)
+{
+    if (!layer || !packed) return fail(BITNET_HIP_NULL_POINTER, "set_weights_base3: null argument");
+    const size_t n = layer->out_features, k = layer->in_features, need = (n * k + 4) / 5;
+    if (packed_len < need) {
+        size_t e[1] = {need}, a[1] = {packed_len};
+        return fail_shape(e, 1, a, 1, "base-3 packed weight bytes");
+    }
+    hipStream_t s = as_stream(stream);
+    DeviceTemp staged;  // the base-3 bytes on the device
+    const uint8_t *src = packed;
+    if (!on_device) {
+        int rc = staged.alloc(need);
+        if (rc != BITNET_HIP_OK) return rc;
+        BITNET_HIP_TRY(hipMemcpyAsync(staged.ptr, packed, need, hipMemcpyHostToDevice, s));
+        src = static_cast<const uint8_t *>(staged.ptr);
+    }
+    std::unique_lock<std::shared_mutex> guard(layer->lock);
+    int rc = launch_base3_to_2bit(src, n * k, layer->packed, s);
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipMemcpyAsync(layer->w_scale, &w_scale, sizeof(float), hipMemcpyHostToDevice, s));
+    rc = launch_retile(layer->packed, n, k, BITNET_HIP_LAYOUT_OUT_IN, layer->tiled, s);
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipStreamSynchronize(s));  // w_scale is read from the caller's stack; `staged` is freed on return
     layer->has_weights = true;
     return BITNET_HIP_OK;
 }

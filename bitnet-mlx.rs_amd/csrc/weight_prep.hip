@@ -45,6 +45,46 @@ __global__ __launch_bounds__(256) void unpack_2bit_kernel(const uint8_t *packed,
     q[i] = code == 0 ? -1 : (code == 2 ? 1 : 0);
 }
 
+// Base-3 bytes: value j of byte b is digit j of b in base 3 (bitnet-quant/src/quantization/packing.rs:424-501).
+__device__ __forceinline__ unsigned base3_digit(unsigned byte, unsigned j)
+{
+    const unsigned div = j == 0 ? 1u : (j == 1 ? 3u : (j == 2 ? 9u : (j == 3 ? 27u : 81u)));
+    return (byte / div) % 3u;
+}
+
+__global__ __launch_bounds__(256) void pack_base3_kernel(const int8_t *q, size_t count, uint8_t *packed, size_t nbytes)
+{
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nbytes) return;
+    unsigned byte = 0, mult = 1;
+    for (int j = 0; j < 5; ++j) {
+        size_t i = 5 * b + j;
+        if (i < count) byte += (unsigned)(uint8_t)(q[i] + 1) * mult;
+        mult *= 3;
+    }
+    packed[b] = (uint8_t)byte;
+}
+
+__global__ __launch_bounds__(256) void unpack_base3_kernel(const uint8_t *packed, size_t count, int8_t *q)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    q[i] = (int8_t)base3_digit(packed[i / 5], (unsigned)(i % 5)) - 1;
+}
+
+// One 2-bit byte (elements 4b .. 4b+3) per thread: both formats use the code w + 1.
+__global__ __launch_bounds__(256) void base3_to_2bit_kernel(const uint8_t *base3, size_t count, uint8_t *packed, size_t nbytes)
+{
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nbytes) return;
+    unsigned byte = 0;
+    for (int j = 0; j < 4; ++j) {
+        size_t i = 4 * b + j;
+        if (i < count) byte |= base3_digit(base3[i / 5], (unsigned)(i % 5)) << (2 * j);
+    }
+    packed[b] = (uint8_t)byte;
+}
+
 __device__ __forceinline__ double wave_sum_f64(double p)
 {
 #pragma unroll
@@ -180,6 +220,32 @@ int launch_unpack_2bit(const uint8_t *packed, size_t count, int8_t *q, hipStream
     if (count == 0) return BITNET_HIP_OK;
     hipLaunchKernelGGL(unpack_2bit_kernel, dim3(blocks_for(count, 256)), dim3(256), 0, stream, packed, count, q);
     BITNET_HIP_CHECK_LAUNCH("unpack_2bit_kernel");
+    return BITNET_HIP_OK;
+}
+
+int launch_pack_base3(const int8_t *q, size_t count, uint8_t *packed, hipStream_t stream)
+{
+    size_t nbytes = (count + 4) / 5;
+    if (nbytes == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL(pack_base3_kernel, dim3(blocks_for(nbytes, 256)), dim3(256), 0, stream, q, count, packed, nbytes);
+    BITNET_HIP_CHECK_LAUNCH("pack_base3_kernel");
+    return BITNET_HIP_OK;
+}
+
+int launch_unpack_base3(const uint8_t *packed, size_t count, int8_t *q, hipStream_t stream)
+{
+    if (count == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL(unpack_base3_kernel, dim3(blocks_for(count, 256)), dim3(256), 0, stream, packed, count, q);
+    BITNET_HIP_CHECK_LAUNCH("unpack_base3_kernel");
+    return BITNET_HIP_OK;
+}
+
+int launch_base3_to_2bit(const uint8_t *base3, size_t count, uint8_t *packed, hipStream_t stream)
+{
+    size_t nbytes = (count + 3) / 4;
+    if (nbytes == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL(base3_to_2bit_kernel, dim3(blocks_for(nbytes, 256)), dim3(256), 0, stream, base3, count, packed, nbytes);
+    BITNET_HIP_CHECK_LAUNCH("base3_to_2bit_kernel");
     return BITNET_HIP_OK;
 }
 

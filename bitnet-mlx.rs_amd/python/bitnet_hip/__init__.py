@@ -87,6 +87,9 @@ def load_library() -> C.CDLL:
         "bitnet_hip_packed_size": (sz, [sz]),
         "bitnet_hip_pack_ternary_2bit": (i32, [vp, sz, vp, vp]),
         "bitnet_hip_unpack_ternary_2bit": (i32, [vp, sz, vp, vp]),
+        "bitnet_hip_base3_packed_size": (sz, [sz]),
+        "bitnet_hip_pack_ternary_base3": (i32, [vp, sz, vp, vp]),
+        "bitnet_hip_unpack_ternary_base3": (i32, [vp, sz, vp, vp]),
         "bitnet_hip_quantize_weights": (i32, [vp, sz, sz, i32, f32, vp, vp, vp, vp]),
         "bitnet_hip_tiled_size": (sz, [sz, sz]),
         "bitnet_hip_retile_weights": (i32, [vp, sz, sz, i32, vp, vp]),
@@ -98,6 +101,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_bitlinear_destroy": (None, [vp]),
         "bitnet_hip_bitlinear_set_weights_f32": (i32, [vp, vp, sz, sz, i32, i32, i32, f32, vp]),
         "bitnet_hip_bitlinear_set_weights_packed": (i32, [vp, vp, sz, f32, i32, vp]),
+        "bitnet_hip_bitlinear_set_weights_base3": (i32, [vp, vp, sz, f32, i32, vp]),
         "bitnet_hip_bitlinear_set_weights_gguf": (i32, [vp, vp, sz, sz, sz, i32, i32, C.POINTER(C.c_float),
                                                   C.POINTER(C.c_float), vp]),
         "bitnet_hip_bitlinear_set_bias": (i32, [vp, vp, sz, i32, vp]),
@@ -221,6 +225,26 @@ def unpack_ternary_2bit(packed: torch.Tensor, count: int, stream=None) -> torch.
     return out
 
 
+def base3_packed_size(count: int) -> int:
+    return (count + 4) // 5
+
+
+def pack_ternary_base3(q: torch.Tensor, stream=None) -> torch.Tensor:
+    _dev(q, torch.int8, "q")
+    out = torch.empty((base3_packed_size(q.numel()),), dtype=torch.uint8, device=q.device)
+    _check(load_library().bitnet_hip_pack_ternary_base3(_ptr(q), q.numel(), _ptr(out), _stream(stream)))
+    return out
+
+
+def unpack_ternary_base3(packed: torch.Tensor, count: int, stream=None) -> torch.Tensor:
+    _dev(packed, torch.uint8, "packed")
+    if packed.numel() < base3_packed_size(count):
+        raise BitLinearError(SHAPE_MISMATCH, "packed buffer too short", [base3_packed_size(count)], [packed.numel()])
+    out = torch.empty((count,), dtype=torch.int8, device=packed.device)
+    _check(load_library().bitnet_hip_unpack_ternary_base3(_ptr(packed), count, _ptr(out), _stream(stream)))
+    return out
+
+
 def quantize_weights(w: torch.Tensor, method: int = TERNARY_ABSMEAN_ROUNDCLIP, threshold_factor: float = 0.5,
                      want_i8: bool = False, stream=None):
     """Ternarise + pack an [n, k] f32 matrix on the GPU.  Returns (packed u8, w_scale f32[1], q i8 or None)."""
@@ -290,6 +314,16 @@ class BitPacked2BitPacker:
         return unpack_ternary_2bit(packed, element_count)
 
 
+class Base3PackedPacker:
+    """Mirror of Base3PackedPacker (bitnet-quant/src/quantization/packing.rs:421-501): 5 values per byte."""
+
+    def pack(self, weights: torch.Tensor) -> torch.Tensor:
+        return pack_ternary_base3(weights.reshape(-1))
+
+    def unpack(self, packed: torch.Tensor, element_count: int) -> torch.Tensor:
+        return unpack_ternary_base3(packed, element_count)
+
+
 class TernaryProcessor:
     """Mirror of TernaryProcessor (bitnet-inference/src/engine/ternary_operations.rs:56-172), int8 kept."""
 
@@ -346,6 +380,14 @@ class BitLinear:
             raise BitLinearError(INVALID_CONFIG, "packed weights must be contiguous u8")
         _check(load_library().bitnet_hip_bitlinear_set_weights_packed(self._h, _ptr(packed), packed.numel(), w_scale,
                                                                       int(packed.is_cuda), _stream(stream)))
+
+    def set_base3_weights(self, packed: torch.Tensor, w_scale: float, stream=None):
+        """Weights in the reference's base-3 byte format (Base3PackedPacker, packing.rs:421-501), [out, in] flat,
+        host or device; re-coded once into the 2-bit tiles."""
+        if packed.dtype != torch.uint8 or not packed.is_contiguous():
+            raise BitLinearError(INVALID_CONFIG, "packed weights must be contiguous u8")
+        _check(load_library().bitnet_hip_bitlinear_set_weights_base3(self._h, _ptr(packed), packed.numel(), w_scale,
+                                                                     int(packed.is_cuda), _stream(stream)))
 
     def load_gguf_ternary(self, data: torch.Tensor, layout: int = LAYOUT_OUT_IN, stream=None):
         """A GGUF BitnetB158 tensor (8-byte scale/offset header + 2-bit codes, GgufLoader::decode_ternary_weights,

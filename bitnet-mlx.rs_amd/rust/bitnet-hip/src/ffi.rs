@@ -46,6 +46,9 @@ extern "C" {
     pub fn bitnet_hip_packed_size(count: usize) -> usize;
     pub fn bitnet_hip_pack_ternary_2bit(q: *const i8, count: usize, packed: *mut u8, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_unpack_ternary_2bit(packed: *const u8, count: usize, q: *mut i8, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_base3_packed_size(count: usize) -> usize;
+    pub fn bitnet_hip_pack_ternary_base3(q: *const i8, count: usize, packed: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_unpack_ternary_base3(packed: *const u8, count: usize, q: *mut i8, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_quantize_weights(w: *const f32, n: usize, k: usize, method: c_int, threshold_factor: f32,
                                        packed: *mut u8, w_scale: *mut f32, q_i8: *mut i8, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_tiled_size(n: usize, k: usize) -> usize;
@@ -69,6 +72,9 @@ extern "C" {
     pub fn bitnet_hip_bitlinear_set_weights_packed(layer: *mut bitnet_hip_bitlinear, packed: *const u8,
                                                    packed_len: usize, w_scale: f32, on_device: c_int,
                                                    stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_bitlinear_set_weights_base3(layer: *mut bitnet_hip_bitlinear, packed: *const u8,
+                                                  packed_len: usize, w_scale: f32, on_device: c_int,
+                                                  stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_bitlinear_set_weights_gguf(layer: *mut bitnet_hip_bitlinear, data: *const u8, len: usize,
                                                  rows: usize, cols: usize, layout: c_int, on_device: c_int,
                                                  scale_out: *mut f32, offset_out: *mut f32,

@@ -110,6 +110,14 @@ size_t bitnet_hip_packed_size(size_t count);
 int bitnet_hip_pack_ternary_2bit(const int8_t *q, size_t count, uint8_t *packed, void *stream);
 int bitnet_hip_unpack_ternary_2bit(const uint8_t *packed, size_t count, int8_t *q, void *stream);
 
+/* Base-3 pack / unpack, 5 ternary values per byte: byte = sum_{j<5} (w[5b+j] + 1) * 3^j; value j of a byte is
+ * (byte / 3^j) % 3 - 1 (bytes above 242 decode by the same divisions).  bitnet_hip_base3_packed_size(count) =
+ * (count + 4) / 5 bytes.
+ *   replaces Base3PackedPacker::{pack,unpack} (bitnet-quant/src/quantization/packing.rs:424-501). */
+size_t bitnet_hip_base3_packed_size(size_t count);
+int bitnet_hip_pack_ternary_base3(const int8_t *q, size_t count, uint8_t *packed, void *stream);
+int bitnet_hip_unpack_ternary_base3(const uint8_t *packed, size_t count, int8_t *q, void *stream);
+
 /* Ternarise an f32 weight matrix [n, k] (row-major) and pack it in the reference's byte format.
  *   replaces SimdTernaryOps::{compute_absmean, quantize_batch} (bitnet-quant/src/simd/ternary.rs:27-66)
  *   / BitNetWeightQuantizer::quantize (bitnet-quant/src/quantization/weights.rs:568-611) + the packer.
@@ -189,6 +197,11 @@ int bitnet_hip_bitlinear_set_weights_packed(bitnet_hip_bitlinear *layer, const u
 int bitnet_hip_bitlinear_set_weights_gguf(bitnet_hip_bitlinear *layer, const uint8_t *data, size_t len, size_t rows,
                                           size_t cols, int layout, int on_device, float *scale_out,
                                           float *offset_out, void *stream);
+/* Pre-quantised weights in the reference's base-3 byte format (TernaryPackingStrategy::Base3Packed,
+ * packing.rs:424-501: 1.6 bits per weight on disk), [out,in] flat, plus their scale.  The bytes are re-coded once into
+ * the 2-bit tiles the kernels stream; a buffer shorter than ceil(out*in/5) bytes is a SHAPE_MISMATCH. */
+int bitnet_hip_bitlinear_set_weights_base3(bitnet_hip_bitlinear *layer, const uint8_t *packed, size_t packed_len,
+                                           float w_scale, int on_device, void *stream);
 /* BitLinear::update_bias (layer.rs:329-352): INVALID_CONFIG if the layer was created without bias. */
 int bitnet_hip_bitlinear_set_bias(bitnet_hip_bitlinear *layer, const float *bias, size_t len, int on_device,
                                   void *stream);

@@ -13,6 +13,8 @@
  * Parity status of each function (what pins it besides this restatement):
  *   orc_pack_2bit / orc_unpack_2bit      pinned: byte fixtures and round trips held by the reference's tests
  *   orc_gguf_decode_ternary              pinned: the reference's own decode test (header + 0x24 -> [-1,0,1,-1])
+ *   orc_pack_base3 / orc_unpack_base3    pinned: the reference's four encoding fixtures (140, 0, 242, 121) and
+ *                                        its round-trip test
  *   orc_round_clip, orc_ternarize_*      pinned: reference tables (round_clip ties, strict '>' threshold)
  *   orc_absmean                          pinned: reference vector [1,-2,3,-4] -> 2.5; order declared here
  *   orc_gemv_w2a8 / orc_gemm_w2a8        pinned: reference 3x4 GEMV / 2x3x2 GEMM vectors + brute force
@@ -340,6 +342,33 @@ size_t orc_gguf_decode_ternary(const uint8_t *data, size_t len, size_t count, in
     for (size_t b = start; b < len && produced < count; ++b)
         for (int j = 0; j < 4 && produced < count; ++j) q[produced++] = lut[(data[b] >> (2 * j)) & 3u];
     return produced;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Base-3 packing, 5 ternary values per byte.   reference: bitnet-quant/src/quantization/packing.rs:424-501
+ *   pack:   byte = sum_{j<5} (w[5b+j] + 1) * 3^j, elements past the end left out (:436-447)
+ *   unpack: value j of a byte = (byte / 3^j) % 3 - 1, for as many elements as were packed (:486-497);
+ *           bytes above 242 are decoded by the same divisions (their digits are still in 0..2)
+ * ---------------------------------------------------------------------------------------------- */
+void orc_pack_base3(const int8_t *q, size_t n, uint8_t *packed)
+{
+    for (size_t b = 0; 5 * b < n; ++b) {
+        unsigned byte = 0, mult = 1;
+        for (size_t j = 0; j < 5 && 5 * b + j < n; ++j) {
+            byte += (unsigned)(uint8_t)(q[5 * b + j] + 1) * mult;
+            mult *= 3;
+        }
+        packed[b] = (uint8_t)byte;
+    }
+}
+
+void orc_unpack_base3(const uint8_t *packed, size_t n, int8_t *q)
+{
+    for (size_t i = 0; i < n; ++i) {
+        unsigned rem = packed[i / 5];
+        for (size_t j = 0; j < i % 5; ++j) rem /= 3;
+        q[i] = (int8_t)(rem % 3) - 1;
+    }
 }
 
 /* ------------------------------------------------------------------------------------------------

@@ -162,6 +162,23 @@ def unpack_2bit(packed, n):
     return q
 
 
+def pack_base3(q):
+    """Base3PackedPacker::pack (packing.rs:424-447): 5 values per byte, value j weighs 3^j."""
+    q = np.ascontiguousarray(q, dtype=np.int8).ravel()
+    out = np.zeros((q.size + 4) // 5, dtype=np.uint8)
+    lib().orc_pack_base3(_p(q), _sz(q.size), _p(out))
+    return out
+
+
+def unpack_base3(packed, count):
+    """Base3PackedPacker::unpack (packing.rs:480-501)."""
+    packed = np.ascontiguousarray(packed, dtype=np.uint8).ravel()
+    assert packed.size * 5 >= count
+    q = np.empty(count, dtype=np.int8)
+    lib().orc_unpack_base3(_p(packed), _sz(count), _p(q))
+    return q
+
+
 def gguf_decode_ternary(data, count):
     """GgufLoader::decode_ternary_weights (gguf.rs:1089-1165): returns (q int8 [produced], scale, offset), or None
     where the reference reports "Insufficient packed data"."""

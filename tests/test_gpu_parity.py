@@ -411,6 +411,46 @@ def test_forward_in_hip_graph_replays_match_eager(m):
         assert np.array_equal(host(other), ref)
 
 
+@pytest.mark.parametrize("n", [1, 4, 5, 6, 1000, 10001, 2560 * 640])
+def test_base3_pack_unpack_bit_exact(n):
+    """Base3PackedPacker on the GPU against the oracle, ragged tails included; decoding every byte value."""
+    rng = np.random.default_rng(n)
+    q = rng.integers(-1, 2, size=n).astype(np.int8)
+    packed = bh.pack_ternary_base3(dev(q))
+    assert np.array_equal(host(packed), orc.pack_base3(q))
+    assert np.array_equal(host(bh.unpack_ternary_base3(packed, n)), q)
+    raw = rng.integers(0, 256, size=(n + 4) // 5).astype(np.uint8)  # any byte, also above 242
+    assert np.array_equal(host(bh.unpack_ternary_base3(dev(raw), n)), orc.unpack_base3(raw, n))
+
+
+@pytest.mark.parametrize("n,k", [(1, 4), (48, 300), (33, 7), (640, 2560)])
+@pytest.mark.parametrize("on_device", [False, True])
+def test_bitlinear_base3_weights_match_2bit_weights(n, k, on_device):
+    """A layer loaded from base-3 bytes holds the same canonical 2-bit bytes and computes the same forward as a
+    layer loaded from the 2-bit bytes of the same ternary matrix; short buffers are a shape mismatch."""
+    rng = np.random.default_rng(31 * n + k)
+    q = rng.integers(-1, 2, size=(n, k)).astype(np.int8)
+    ws = np.float32(0.0173)
+    b3 = torch.from_numpy(orc.pack_base3(q.ravel()))
+    a = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "b3")
+    a.set_base3_weights(b3.cuda() if on_device else b3, float(ws))
+    b = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), "b2")
+    b.set_quantized_weights(dev(orc.pack_2bit(q.ravel())), float(ws))
+    pa, sa = a.get_quantized_weights()
+    pb, sb = b.get_quantized_weights()
+    assert sa == sb == float(ws)
+    assert np.array_equal(pa.numpy(), pb.numpy())
+    assert np.array_equal(pa.numpy(), orc.pack_2bit(q.ravel()))
+    x = synth_activations(rng, 3, k)
+    ya, yb = host(a.forward(dev(x))), host(b.forward(dev(x)))
+    assert np.array_equal(ya, yb)
+    assert np.array_equal(ya, orc.bitlinear_forward(x, orc.pack_2bit(q.ravel()), n, ws)[0])
+    if b3.numel() > 1:
+        with pytest.raises(bh.BitLinearError) as err:
+            a.set_base3_weights(b3[:-1].contiguous(), float(ws))
+        assert err.value.status == bh.SHAPE_MISMATCH
+
+
 def test_bitlinear_forward_prefill_uses_quantiser_row_sums():
     """BitLinear.forward at a prefill token count: quantiser -> row sums -> LDS-direct GEMM, bit-exact."""
     rng = np.random.default_rng(77)

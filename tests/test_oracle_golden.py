@@ -462,3 +462,35 @@ def test_cpu_baselines_compute_the_same_product():
     orc.cpu_ref_simd_gemv(qw, x, y, ws)
     assert np.max(np.abs(y - want)) < 1e-4 * np.max(np.abs(want))
     assert orc.cpu_threads() >= 1 and orc.cpu_isa() in ("scalar", "avx2+fma", "avx512f")
+
+
+@pytest.mark.parametrize("case", G["base3_encoding"], ids=lambda c: str(c["byte"]))
+def test_base3_encoding_fixtures(case):
+    """Base3PackedPacker: the reference's four encoding patterns, byte for byte, and back."""
+    w = np.array(case["weights"], dtype=np.int8)
+    packed = orc.pack_base3(w)
+    assert packed.tolist() == [case["byte"]]
+    assert np.array_equal(orc.unpack_base3(packed, w.size), w)
+
+
+def test_base3_roundtrip_and_closed_forms():
+    """The reference's round-trip vector; every byte 0..242 is the base-3 numeral of its five values (checked
+    against numpy's own digits); ragged tails leave the missing digits at zero; bytes above 242 still decode by
+    the same divisions (packing.rs:486-497)."""
+    w = np.array(G["base3_roundtrip"]["weights"], dtype=np.int8)
+    assert np.array_equal(orc.unpack_base3(orc.pack_base3(w), w.size), w)
+    allbytes = np.arange(243, dtype=np.uint8)
+    digits = np.stack([(allbytes.astype(np.int64) // 3 ** j) % 3 for j in range(5)], axis=1) - 1
+    assert np.array_equal(orc.unpack_base3(allbytes, 243 * 5).reshape(243, 5), digits.astype(np.int8))
+    assert np.array_equal(orc.pack_base3(digits.astype(np.int8).ravel()), allbytes)
+    rng = np.random.default_rng(5)
+    for n in (1, 2, 3, 4, 6, 9, 1000, 10001):
+        q = rng.integers(-1, 2, size=n).astype(np.int8)
+        packed = orc.pack_base3(q)
+        assert packed.size == (n + 4) // 5
+        assert np.array_equal(orc.unpack_base3(packed, n), q)
+        if n % 5:
+            assert packed[-1] < 3 ** (n % 5)  # nothing above the last packed digit
+    high = np.array([255, 243, 250], dtype=np.uint8)
+    want = np.stack([(high.astype(np.int64) // 3 ** j) % 3 for j in range(5)], axis=1).ravel() - 1
+    assert np.array_equal(orc.unpack_base3(high, 15), want.astype(np.int8))
