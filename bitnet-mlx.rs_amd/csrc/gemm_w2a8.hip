@@ -25,7 +25,10 @@
 // three or four workgroups per compute unit).  An LDS-direct load writes lane l's 16 bytes at base + 16*l, so the XOR swizzle
 // that keeps the fragment reads free of bank conflicts is applied to the global address each lane fetches.
 // The MFMA takes the weight fragment as its first operand, so a lane ends up with four consecutive output
-// columns of one token row and the epilogue stores 16 bytes per lane.
+// columns of one token row and the epilogue stores 16 bytes per lane.  The epilogue's per-row operands (a_sum,
+// a_scale) arrive by LDS-direct loads in the stage buffer that is free during the last stage; the usual case
+// (f32 output only, n % 4 == 0, scales within the short division's range) is straight-line code
+// (store_fragments_fast), everything else goes through store_fragments_general: same bits.
 //
 // gemm_dma8_kernel: the same data path with eight wavefronts per workgroup, for launches with about one tile
 // per compute unit (see its own comment).
