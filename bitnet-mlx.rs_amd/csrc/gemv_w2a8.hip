@@ -26,6 +26,7 @@
 //   * up to three projections that share the input row (q, k, v or gate, up): the grid is the
 //     concatenation of their row blocks.
 // HBM traffic per call: n*k/4 weight bytes; the input row (K or 4K bytes per workgroup) comes from L2.
+// gemv_fused16_kernel is this launch with 16 wavefronts per workgroup (the default for one token; see its comment).
 //
 // gemv_mfma_kernel is the same weight-streaming scheme for 2..16 token rows: the 16 x 16 x 64 int8 MFMA takes
 // the place of the dot-product chain (its A operand is 16 token rows x 64 columns, loaded straight from the
@@ -414,6 +415,149 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
     }
 }
 
+// The same launch with 16 wavefronts per workgroup.  The prologue of gemv_fused_kernel is redundant arithmetic on
+// one wavefront per SIMD (normalise, absmax, quantise: about half of the dependent work of a launch); 1024 threads
+// do the element-wise part four times faster.  Thread t owns chunks t, t + 1024 (NCHB of them); the sum of squares
+// keeps the declared order: chunk c belongs to virtual lane c % 256, whose chain runs over its chunks in ascending
+// order, so every thread parks the four squares of its chunks in LDS and threads 0..255 (one per virtual lane) add
+// them up in that order: 4 * ceil(k / 1024) dependent additions, then the four 64-lane butterflies as before.
+// The (row block, k-tile) pairs of the workgroup are dealt out to the wavefronts round-robin, U per wavefront.
+constexpr int FUSED16_MAX_RB = 4;
+
+template <int MODE, bool NORM, int NCHB, int U>
+__global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p, int rbw)
+{
+    extern __shared__ uint4 lds_a[];  // int8 activations (zero past K), then (NORM) the squares: float4 per chunk
+    __shared__ float red_f[2][16];
+    __shared__ int red_i[16];
+    __shared__ int tot[FUSED16_MAX_RB][TILE_ROWS];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int chunks = p.k >> 2, lds_words = p.kt_count * 64;
+
+    int pj = 0;
+#pragma unroll
+    for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
+        if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
+    const GemvProjDev &P = p.proj[pj];
+    const int rb0 = ((int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0)) * rbw;  // rb_end counts groups of rbw row blocks
+    const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
+    const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + lane;
+    const int pairs = rbw * p.kt_count;
+
+    // every load is unconditional (clamped indices, values discarded), in the order in which the data is needed
+    float4 v[NCHB], gm[NORM ? NCHB : 1];
+    uint4 wt[U];
+#pragma unroll
+    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(p.src, 0, min(tid + 1024 * i, chunks - 1));
+    const int e_n = min((rb0 + (tid >> 4)) * TILE_ROWS + (tid & 15), P.n - 1);  // meaningful for tid < 16 * rbw
+    const float e_ws = P.out ? *P.w_scale : 0.0f;
+    const float e_bias = P.bias ? P.bias[e_n] : 0.0f;
+    const float e_res = P.residual ? P.residual[e_n] : 0.0f;
+    if constexpr (NORM) {
+#pragma unroll
+        for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(p.src, min(tid + 1024 * i, chunks - 1), true);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {  // pairs past the end repeat the last one; their results are not added
+        const int pidx = min(wave + 16 * u, pairs - 1);
+        const int r = pidx / p.kt_count, kt = pidx - r * p.kt_count;
+        wt[u] = tiles[((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + kt) * 64];
+    }
+    if (tid < FUSED16_MAX_RB * TILE_ROWS) tot[tid >> 4][tid & 15] = 0;
+#pragma unroll
+    for (int i = 0; i < NCHB; ++i)
+        if (tid + 1024 * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+    if constexpr (NORM) {
+        float4 *sq = reinterpret_cast<float4 *>(lds_a + p.kt_count * 16);
+#pragma unroll
+        for (int i = 0; i < NCHB; ++i) {
+            const int c = tid + 1024 * i;
+            if (c < chunks)
+                sq[c] = make_float4(f32_mul(v[i].x, v[i].x), f32_mul(v[i].y, v[i].y), f32_mul(v[i].z, v[i].z), f32_mul(v[i].w, v[i].w));
+        }
+        lds_barrier();
+        if (tid < 256) {  // wavefronts 0..3: thread tid is virtual lane tid
+            float part = 0.0f;
+            for (int c = tid; c < chunks; c += 256) {
+                const float4 e = sq[c];
+                part = f32_add(f32_add(f32_add(f32_add(part, e.x), e.y), e.z), e.w);
+            }
+            part = wave_sum_f32(part);
+            if (lane == 0) red_f[0][wave] = part;
+        }
+        lds_barrier();
+        const float ss = f32_add(f32_add(f32_add(red_f[0][0], red_f[0][1]), red_f[0][2]), red_f[0][3]);
+        const RowDivisor rdiv = make_row_divisor(rms_from_ss(ss, p.k, p.src.eps));
+#pragma unroll
+        for (int i = 0; i < NCHB; ++i)
+            if (tid + 1024 * i < chunks) v[i] = normalize4(v[i], rdiv, gm[i]);
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCHB; ++i) amax = absmax4(amax, v[i]);
+    amax = wave_max_f32(amax);
+    if (lane == 0) red_f[1][wave] = amax;
+    lds_barrier();
+    amax = red_f[1][0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) amax = fmaxf(amax, red_f[1][w]);
+    const float scale = scale_from_absmax(amax);
+    uint32_t *lds_w = reinterpret_cast<uint32_t *>(lds_a);
+    int isum = 0;
+#pragma unroll
+    for (int i = 0; i < NCHB; ++i) {
+        const int c = tid + 1024 * i;
+        if (c < chunks) {
+            const uint32_t packed = quant4_packed(v[i], scale, &isum);
+            lds_w[c] = packed;
+            if (p.q_out && blockIdx.x == 0) reinterpret_cast<uint32_t *>(p.q_out)[c] = packed;
+        } else if (c < lds_words) {
+            lds_w[c] = 0;
+        }
+    }
+    isum = wave_sum_i32(isum);
+    if (lane == 0) red_i[wave] = isum;
+    lds_barrier();
+
+    const int kq = lane >> 4;  // lane group: columns 64t + 16kq .. +15 of each tile, t = 0..3
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int pidx = wave + 16 * u;
+        if (pidx < pairs) {  // uniform over the wavefront
+            const int r = pidx / p.kt_count, kt = pidx - r * p.kt_count;
+            int acc = dot64(wt[u], lds_a + kt * 16 + kq, 0);
+            acc = sum_over_lane_groups(acc);  // lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
+            if (lane < TILE_ROWS) atomicAdd(&tot[r][lane], acc);  // int32: any order gives the same sum
+        }
+    }
+    lds_barrier();
+
+    if (tid < TILE_ROWS * rbw) {
+        const int r = tid >> 4, row = tid & 15;
+        const int n = (rb0 + r) * TILE_ROWS + row;
+        int asum = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) asum += red_i[w];
+        if (blockIdx.x == 0 && tid == 0) {
+            if (p.a_scale_out) p.a_scale_out[0] = scale;
+            if (p.a_sum_out) p.a_sum_out[0] = asum;
+        }
+        if (n < P.n) {
+            const int total = tot[r][row] - asum;
+            if (P.acc) P.acc[n] = total;
+            if (P.out) {
+                float y = f32_mul((float)total, e_ws);
+                y = f32_div(y, scale);
+                if (P.bias) y = f32_add(y, e_bias);
+                if (P.residual) y = f32_add(y, e_res);
+                P.out[n] = y;
+            }
+        }
+    }
+}
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 struct GemvMfmaParams {
@@ -715,6 +859,29 @@ int launch_fused_mode(const GemvParams &p, hipStream_t stream)
     return BITNET_HIP_OK;
 }
 
+template <int MODE>
+int launch_fused16_mode(const GemvParams &p, int rbw, hipStream_t stream)
+{
+    const bool norm = p.src.gamma != nullptr;
+    const int chunks = p.k >> 2;
+    const size_t lds = (size_t)p.kt_count * 16 * sizeof(uint4) + (norm ? (size_t)chunks * sizeof(float4) : 0);
+    const dim3 grid((unsigned)p.proj[p.nproj - 1].rb_end);
+    const int u = (rbw * p.kt_count + 15) / 16;
+    const bool one = chunks <= 1024;
+#define BITNET_F16(NORM_, NCHB_, U_) \
+    hipLaunchKernelGGL((gemv_fused16_kernel<MODE, NORM_, NCHB_, U_>), grid, dim3(1024), lds, stream, p, rbw)
+    if (norm) {
+        if (one) { if (u == 1) BITNET_F16(true, 1, 1); else if (u == 2) BITNET_F16(true, 1, 2); else BITNET_F16(true, 1, 3); }
+        else { if (u == 1) BITNET_F16(true, 2, 1); else if (u == 2) BITNET_F16(true, 2, 2); else BITNET_F16(true, 2, 3); }
+    } else {
+        if (one) { if (u == 1) BITNET_F16(false, 1, 1); else if (u == 2) BITNET_F16(false, 1, 2); else BITNET_F16(false, 1, 3); }
+        else { if (u == 1) BITNET_F16(false, 2, 1); else if (u == 2) BITNET_F16(false, 2, 2); else BITNET_F16(false, 2, 3); }
+    }
+#undef BITNET_F16
+    BITNET_HIP_CHECK_LAUNCH("gemv_fused16_kernel");
+    return BITNET_HIP_OK;
+}
+
 // rbw: row blocks per workgroup (rb_end then counts groups of rbw row blocks, per projection)
 int fill_projs(GemvParams &p, const GemvProj *projs, int nproj, size_t t0, size_t k, int rbw = 1)
 {
@@ -841,6 +1008,25 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
     // workgroup two (short rows only: the tiles of both must fit its registers).
     size_t blocks = 0;
     for (int j = 0; j < nproj; ++j) blocks += row_blocks(projs[j].n);
+    // 16 wavefronts per workgroup (the declared summation order only; k <= 8192; at most 48 (row block, k-tile) pairs)
+    const bool wide = (gamma == nullptr || sum_order == BITNET_HIP_SUM_BLOCK256) && k <= 8192;
+    if (wide) {
+        const int rbw16 = (blocks > 512 && k_tiles(k) * 4 <= 48) ? 4 : 1;
+        if (rbw16 * k_tiles(k) <= 48) {
+            GemvParams p = {};
+            if (fill_projs(p, projs, nproj, 0, k, rbw16) == 0) return BITNET_HIP_OK;
+            p.m = (int)m;
+            p.src.x = x; p.src.x2 = x2; p.src.gamma = gamma; p.src.ldx = ldx; p.src.k = (int)k;
+            p.src.head_dim = (int)(head_dim ? head_dim : 1); p.src.gqa_group = (int)(gqa_group ? gqa_group : 1);
+            p.src.sum_order = sum_order; p.src.eps = eps;
+            p.q_out = q_out; p.a_scale_out = a_scale_out; p.a_sum_out = a_sum_out;
+            switch (input_mode) {
+                case BITNET_HIP_INPUT_PLAIN: return launch_fused16_mode<BITNET_HIP_INPUT_PLAIN>(p, rbw16, stream);
+                case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused16_mode<BITNET_HIP_INPUT_RELU2_MUL>(p, rbw16, stream);
+                default: return launch_fused16_mode<BITNET_HIP_INPUT_GQA_BROADCAST>(p, rbw16, stream);
+            }
+        }
+    }
     const int rbw = (blocks > 512 && k <= 3 * 1024) ? 2 : 1;
     GemvParams p = {};
     if (fill_projs(p, projs, nproj, 0, k, rbw) == 0) return BITNET_HIP_OK;
