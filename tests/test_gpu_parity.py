@@ -604,6 +604,27 @@ def test_bitlinear_forward_decode_debug_outputs(m):
     assert np.array_equal(host(layer.forward(dev(x), gamma=dev(g))), out_ref)
 
 
+@pytest.mark.parametrize("k,ns", [(2560, (640,)), (6912, (2560,)), (2560, (6912, 6912))], ids=["short", "long_row", "two_row_blocks"])
+def test_decode_sequential_sum_order_four_wavefront_kernel(k, ns):
+    """One token with RMSNorm in the reference's literal (sequential) summation order: the launch shape that keeps four
+    wavefronts per workgroup (every thread runs the whole chain), with short and long rows, one and two row blocks per
+    workgroup, one and two projections per launch."""
+    rng = np.random.default_rng(k + len(ns))
+    g = (1 + 0.1 * rng.standard_normal(k, dtype=f32)).astype(f32)
+    x = synth_activations(rng, 1, k, outliers=True)
+    layers, refs = [], []
+    for i, n in enumerate(ns):
+        w = synth_weights(rng, n, k)
+        layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n, sum_order=bh.SUM_SEQUENTIAL), f"seq{i}")
+        layer.update_weights(dev(w))
+        layers.append(layer)
+        qw, ws = orc.quantize_weights_absmean(w)
+        refs.append(orc.bitlinear_forward(x, orc.pack_2bit(qw), n, ws, g=g, eps=1e-5, order=orc.SUM_SEQUENTIAL)[0])
+    outs = bh.forward_multi(layers, dev(x), gamma=dev(g)) if len(ns) > 1 else [layers[0].forward(dev(x), gamma=dev(g))]
+    for out, ref in zip(outs, refs):
+        assert np.array_equal(host(out), ref)
+
+
 def test_forward_from_several_threads_and_streams():
     """BitLinear is Send + Sync in the reference (layer.rs:427-428): forward on one layer object from several host
     threads, each on a stream of its own, at decode and prefill token counts, while nothing is shared but the
