@@ -58,12 +58,12 @@ def time_events(torch, fn):
     return start.elapsed_time(stop)
 
 
-LAUNCHES_PER_STEP = 4  # q+k+v | o | gate+up | down, each one gemv_fused16_kernel<MODE, NORM, NCHB, U> launch
+LAUNCHES_PER_STEP = 4  # q+k+v | o | gate+up | down, each one gemv_fused16_kernel<MODE, NORM, NCHB, RBW> launch
 # HBM bytes per launch of that kernel from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (two runs of this
 # script with --no-extras --calibration-copy), each scaled by what the same counter reads for the plain
 # 256 MiB copy: FETCH_SIZE reads 0.5 KiB per KiB fetched (factor 2.0), WRITE_SIZE 1.0 (factor 1.0).
 # Summary: profiles/decode_layer_b1_gemv_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_687_718
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_684_913
 
 
 def decode_roofline(event_ms, steps):
@@ -73,7 +73,7 @@ def decode_roofline(event_ms, steps):
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-        "kernel": "gemv_fused16_kernel<MODE, NORM, NCHB, U> (decode GEMV, activation quantiser in the prologue)",
+        "kernel": "gemv_fused16_kernel<MODE, NORM, NCHB, RBW> (decode GEMV, activation quantiser in the prologue)",
         "launches": launches, "avg_launch_us": round(event_ms * 1e3 / launches, 3),
         "bytes_per_launch": LAYER_BYTES // LAUNCHES_PER_STEP,
         "how": "HIP events on the launch stream around the timed region, which holds only this kernel "

@@ -419,18 +419,19 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
 // one wavefront per SIMD (normalise, absmax, quantise: about half of the dependent work of a launch); 1024 threads
 // do the element-wise part four times faster.  Thread t owns chunks t, t + 1024 (NCHB of them); the sum of squares
 // keeps the declared order: chunk c belongs to virtual lane c % 256, whose chain runs over its chunks in ascending
-// order, so every thread parks the four squares of its chunks in LDS and threads 0..255 (one per virtual lane) add
-// them up in that order: 4 * ceil(k / 1024) dependent additions, then the four 64-lane butterflies as before.
-// The (row block, k-tile) pairs of the workgroup are dealt out to the wavefronts round-robin, U per wavefront.
-constexpr int FUSED16_MAX_RB = 4;
+// order, so threads 0..255 (one per virtual lane) also fetch their lane's chunks (from L2, with the first loads of the
+// kernel) and add the squares up in that order, then the four 64-lane butterflies as before.
+// A 256-column k-tile is the 64 chunks one wavefront quantises, so every wavefront multiplies the tiles of its own
+// chunks (for each of the workgroup's RBW row blocks) straight after writing them to LDS, without a workgroup barrier
+// between quantiser and dot products; the partial sums of a row meet in LDS atomics.
 
-template <int MODE, bool NORM, int NCHB, int U>
-__global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p, int rbw)
+template <int MODE, bool NORM, int NCHB, int RBW>
+__global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p)
 {
-    extern __shared__ uint4 lds_a[];  // int8 activations (zero past K), then (NORM) the squares: float4 per chunk
+    extern __shared__ uint4 lds_a[];  // int8 activations, zero past K
     __shared__ float red_f[2][16];
     __shared__ int red_i[16];
-    __shared__ int tot[FUSED16_MAX_RB][TILE_ROWS];
+    __shared__ int tot[RBW][TILE_ROWS];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int chunks = p.k >> 2, lds_words = p.kt_count * 64;
@@ -440,17 +441,24 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p, int rb
     for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
         if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
     const GemvProjDev &P = p.proj[pj];
-    const int rb0 = ((int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0)) * rbw;  // rb_end counts groups of rbw row blocks
+    const int rb0 = ((int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0)) * RBW;  // rb_end counts groups of RBW row blocks
     const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
     const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + lane;
-    const int pairs = rbw * p.kt_count;
 
     // every load is unconditional (clamped indices, values discarded), in the order in which the data is needed
     float4 v[NCHB], gm[NORM ? NCHB : 1];
-    uint4 wt[U];
+    constexpr int NSS = NORM ? 4 * NCHB : 1;  // chunks per virtual lane of the summation order
+    float4 vs[NSS];
+    uint4 wt[RBW][NCHB];
 #pragma unroll
     for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(p.src, 0, min(tid + 1024 * i, chunks - 1));
-    const int e_n = min((rb0 + (tid >> 4)) * TILE_ROWS + (tid & 15), P.n - 1);  // meaningful for tid < 16 * rbw
+    if constexpr (NORM) {
+        if (wave < 4) {  // thread tid < 256 is virtual lane tid: it fetches the lane's chunks itself (from L2)
+#pragma unroll
+            for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(p.src, 0, min(tid + 256 * i, chunks - 1));
+        }
+    }
+    const int e_n = min((rb0 + (tid >> 4)) * TILE_ROWS + (tid & 15), P.n - 1);  // meaningful for tid < 16 * RBW
     const float e_ws = P.out ? *P.w_scale : 0.0f;
     const float e_bias = P.bias ? P.bias[e_n] : 0.0f;
     const float e_res = P.residual ? P.residual[e_n] : 0.0f;
@@ -458,32 +466,24 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p, int rb
 #pragma unroll
         for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(p.src, min(tid + 1024 * i, chunks - 1), true);
     }
+    // k-tile kt holds chunks 64*kt .. 64*kt + 63: exactly what wavefront kt % 16 quantises, so a wavefront multiplies
+    // the tiles of its own chunks (tiles and row blocks past the end repeat the last one; their results are not added)
 #pragma unroll
-    for (int u = 0; u < U; ++u) {  // pairs past the end repeat the last one; their results are not added
-        const int pidx = min(wave + 16 * u, pairs - 1);
-        const int r = pidx / p.kt_count, kt = pidx - r * p.kt_count;
-        wt[u] = tiles[((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + kt) * 64];
-    }
-    if (tid < FUSED16_MAX_RB * TILE_ROWS) tot[tid >> 4][tid & 15] = 0;
+    for (int r = 0; r < RBW; ++r)
+#pragma unroll
+        for (int i = 0; i < NCHB; ++i)
+            wt[r][i] = tiles[((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 16 * i, p.kt_count - 1)) * 64];
+    if (tid < RBW * TILE_ROWS) tot[tid >> 4][tid & 15] = 0;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i)
         if (tid + 1024 * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     if constexpr (NORM) {
-        float4 *sq = reinterpret_cast<float4 *>(lds_a + p.kt_count * 16);
-#pragma unroll
-        for (int i = 0; i < NCHB; ++i) {
-            const int c = tid + 1024 * i;
-            if (c < chunks)
-                sq[c] = make_float4(f32_mul(v[i].x, v[i].x), f32_mul(v[i].y, v[i].y), f32_mul(v[i].z, v[i].z), f32_mul(v[i].w, v[i].w));
-        }
-        lds_barrier();
-        if (tid < 256) {  // wavefronts 0..3: thread tid is virtual lane tid
+        if (wave < 4) {  // wavefronts 0..3: thread tid is virtual lane tid
             float part = 0.0f;
-            for (int c = tid; c < chunks; c += 256) {
-                const float4 e = sq[c];
-                part = f32_add(f32_add(f32_add(f32_add(part, e.x), e.y), e.z), e.w);
-            }
+#pragma unroll
+            for (int i = 0; i < NSS; ++i)
+                if (tid + 256 * i < chunks) part = sum_squares4(part, vs[i]);  // chunks past the end would add +0
             part = wave_sum_f32(part);
             if (lane == 0) red_f[0][wave] = part;
         }
@@ -519,22 +519,26 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p, int rb
     }
     isum = wave_sum_i32(isum);
     if (lane == 0) red_i[wave] = isum;
-    lds_barrier();
+    // the int8 values this wavefront reads back below are its own: no workgroup barrier, only the LDS queue of the wavefront
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
 
     const int kq = lane >> 4;  // lane group: columns 64t + 16kq .. +15 of each tile, t = 0..3
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const int pidx = wave + 16 * u;
-        if (pidx < pairs) {  // uniform over the wavefront
-            const int r = pidx / p.kt_count, kt = pidx - r * p.kt_count;
-            int acc = dot64(wt[u], lds_a + kt * 16 + kq, 0);
-            acc = sum_over_lane_groups(acc);  // lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
-            if (lane < TILE_ROWS) atomicAdd(&tot[r][lane], acc);  // int32: any order gives the same sum
+    for (int i = 0; i < NCHB; ++i) {
+        const int kt = wave + 16 * i;
+        if (kt < p.kt_count) {  // uniform over the wavefront
+#pragma unroll
+            for (int r = 0; r < RBW; ++r) {
+                int acc = dot64(wt[r][i], lds_a + kt * 16 + kq, 0);
+                acc = sum_over_lane_groups(acc);  // lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
+                if (lane < TILE_ROWS) atomicAdd(&tot[r][lane], acc);  // int32: any order gives the same sum
+            }
         }
     }
     lds_barrier();
 
-    if (tid < TILE_ROWS * rbw) {
+    if (tid < TILE_ROWS * RBW) {
         const int r = tid >> 4, row = tid & 15;
         const int n = (rb0 + r) * TILE_ROWS + row;
         int asum = 0;
@@ -859,25 +863,16 @@ int launch_fused_mode(const GemvParams &p, hipStream_t stream)
     return BITNET_HIP_OK;
 }
 
-template <int MODE>
-int launch_fused16_mode(const GemvParams &p, int rbw, hipStream_t stream)
+template <int MODE, int RBW>
+int launch_fused16_mode(const GemvParams &p, hipStream_t stream)
 {
-    const bool norm = p.src.gamma != nullptr;
-    const int chunks = p.k >> 2;
-    const size_t lds = (size_t)p.kt_count * 16 * sizeof(uint4) + (norm ? (size_t)chunks * sizeof(float4) : 0);
+    const bool norm = p.src.gamma != nullptr, one = (p.k >> 2) <= 1024;
+    const size_t lds = (size_t)p.kt_count * 16 * sizeof(uint4);
     const dim3 grid((unsigned)p.proj[p.nproj - 1].rb_end);
-    const int u = (rbw * p.kt_count + 15) / 16;
-    const bool one = chunks <= 1024;
-#define BITNET_F16(NORM_, NCHB_, U_) \
-    hipLaunchKernelGGL((gemv_fused16_kernel<MODE, NORM_, NCHB_, U_>), grid, dim3(1024), lds, stream, p, rbw)
-    if (norm) {
-        if (one) { if (u == 1) BITNET_F16(true, 1, 1); else if (u == 2) BITNET_F16(true, 1, 2); else BITNET_F16(true, 1, 3); }
-        else { if (u == 1) BITNET_F16(true, 2, 1); else if (u == 2) BITNET_F16(true, 2, 2); else BITNET_F16(true, 2, 3); }
-    } else {
-        if (one) { if (u == 1) BITNET_F16(false, 1, 1); else if (u == 2) BITNET_F16(false, 1, 2); else BITNET_F16(false, 1, 3); }
-        else { if (u == 1) BITNET_F16(false, 2, 1); else if (u == 2) BITNET_F16(false, 2, 2); else BITNET_F16(false, 2, 3); }
-    }
-#undef BITNET_F16
+    if (norm && one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 1, RBW>), grid, dim3(1024), lds, stream, p);
+    else if (norm) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 2, RBW>), grid, dim3(1024), lds, stream, p);
+    else if (one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, 1, RBW>), grid, dim3(1024), lds, stream, p);
+    else hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, 2, RBW>), grid, dim3(1024), lds, stream, p);
     BITNET_HIP_CHECK_LAUNCH("gemv_fused16_kernel");
     return BITNET_HIP_OK;
 }
@@ -1008,23 +1003,27 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
     // workgroup two (short rows only: the tiles of both must fit its registers).
     size_t blocks = 0;
     for (int j = 0; j < nproj; ++j) blocks += row_blocks(projs[j].n);
-    // 16 wavefronts per workgroup (the declared summation order only; k <= 8192; at most 48 (row block, k-tile) pairs)
-    const bool wide = (gamma == nullptr || sum_order == BITNET_HIP_SUM_BLOCK256) && k <= 8192;
-    if (wide) {
-        const int rbw16 = (blocks > 512 && k_tiles(k) * 4 <= 48) ? 4 : 1;
-        if (rbw16 * k_tiles(k) <= 48) {
-            GemvParams p = {};
-            if (fill_projs(p, projs, nproj, 0, k, rbw16) == 0) return BITNET_HIP_OK;
-            p.m = (int)m;
-            p.src.x = x; p.src.x2 = x2; p.src.gamma = gamma; p.src.ldx = ldx; p.src.k = (int)k;
-            p.src.head_dim = (int)(head_dim ? head_dim : 1); p.src.gqa_group = (int)(gqa_group ? gqa_group : 1);
-            p.src.sum_order = sum_order; p.src.eps = eps;
-            p.q_out = q_out; p.a_scale_out = a_scale_out; p.a_sum_out = a_sum_out;
+    // 16 wavefronts per workgroup (the declared summation order only; k <= 8192: two chunks per thread, 32 k-tiles)
+    if ((gamma == nullptr || sum_order == BITNET_HIP_SUM_BLOCK256) && k <= 8192) {
+        const int rbw16 = (blocks > 512 && k <= 4096) ? 4 : 1;
+        GemvParams p = {};
+        if (fill_projs(p, projs, nproj, 0, k, rbw16) == 0) return BITNET_HIP_OK;
+        p.m = (int)m;
+        p.src.x = x; p.src.x2 = x2; p.src.gamma = gamma; p.src.ldx = ldx; p.src.k = (int)k;
+        p.src.head_dim = (int)(head_dim ? head_dim : 1); p.src.gqa_group = (int)(gqa_group ? gqa_group : 1);
+        p.src.sum_order = sum_order; p.src.eps = eps;
+        p.q_out = q_out; p.a_scale_out = a_scale_out; p.a_sum_out = a_sum_out;
+        if (rbw16 == 4) {
             switch (input_mode) {
-                case BITNET_HIP_INPUT_PLAIN: return launch_fused16_mode<BITNET_HIP_INPUT_PLAIN>(p, rbw16, stream);
-                case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused16_mode<BITNET_HIP_INPUT_RELU2_MUL>(p, rbw16, stream);
-                default: return launch_fused16_mode<BITNET_HIP_INPUT_GQA_BROADCAST>(p, rbw16, stream);
+                case BITNET_HIP_INPUT_PLAIN: return launch_fused16_mode<BITNET_HIP_INPUT_PLAIN, 4>(p, stream);
+                case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused16_mode<BITNET_HIP_INPUT_RELU2_MUL, 4>(p, stream);
+                default: return launch_fused16_mode<BITNET_HIP_INPUT_GQA_BROADCAST, 4>(p, stream);
             }
+        }
+        switch (input_mode) {
+            case BITNET_HIP_INPUT_PLAIN: return launch_fused16_mode<BITNET_HIP_INPUT_PLAIN, 1>(p, stream);
+            case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused16_mode<BITNET_HIP_INPUT_RELU2_MUL, 1>(p, stream);
+            default: return launch_fused16_mode<BITNET_HIP_INPUT_GQA_BROADCAST, 1>(p, stream);
         }
     }
     const int rbw = (blocks > 512 && k <= 3 * 1024) ? 2 : 1;
