@@ -583,7 +583,7 @@ struct GemvMfmaParams {
 template <int RB, int MT, bool FAST, bool ONE = false>
 __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 {
-    __shared__ int red[3][RB][MT][64][4];  // partial accumulators of wavefronts 1..3
+    __shared__ int red[4][RB][MT][64][4];  // partial accumulators of the four wavefronts
     __shared__ int red_sum[4][MT][16];     // per wavefront: sum_k a[t, k] over its k-tiles
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -643,27 +643,21 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 
     // scales the epilogue will need (result register i of a lane belongs to token 16g + 4*(lane/16) + i): requested
     // now, so that their latency is not paid at the end
+    // The RB * MT <= 4 fragments (row block, token group) are finished by one wavefront each: fragment
+    // (fr, fg) = (wave / MT, wave % MT).  Its scale, bias and residual are requested now (clamped indices; unused
+    // values are discarded).
+    static_assert(RB * MT <= 4, "one wavefront per fragment");
     const float ws = P.out ? *P.w_scale : 0.0f;
-    float e_scale[MT][4];
+    const int fr = min(wave / MT, RB - 1), fg = wave % MT;
+    const bool finisher = wave < RB * MT;
+    const int e_n = min((rb0 + fr) * TILE_ROWS + lr, P.n - 1);
+    const float e_bias = (finisher && P.bias) ? P.bias[e_n] : 0.0f;
+    float e_scale[4], e_res[4];
 #pragma unroll
-    for (int g = 0; g < MT; ++g)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int t = 16 * g + lg * 4 + i;
-            e_scale[g][i] = (P.out && t < p.m) ? p.a_scale[t] : 1.0f;
-        }
-
-    // bias and residual of the rows wavefront 0 will store (clamped indices; unused values are discarded)
-    float e_bias[RB], e_res[RB][MT][4];
-#pragma unroll
-    for (int r = 0; r < RB; ++r) {
-        const int n = min((rb0 + r) * TILE_ROWS + lr, P.n - 1);
-        e_bias[r] = (wave == 0 && P.bias) ? P.bias[n] : 0.0f;
-#pragma unroll
-        for (int g = 0; g < MT; ++g)
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                e_res[r][g][i] = (wave == 0 && P.residual) ? P.residual[(size_t)min(16 * g + lg * 4 + i, p.m - 1) * P.n + n] : 0.0f;
+    for (int i = 0; i < 4; ++i) {
+        const int t = min(16 * fg + lg * 4 + i, p.m - 1);
+        e_scale[i] = (finisher && P.out) ? p.a_scale[t] : 1.0f;
+        e_res[i] = (finisher && P.residual) ? P.residual[(size_t)t * P.n + e_n] : 0.0f;
     }
 
     v4i acc[RB][MT];
@@ -675,8 +669,9 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         for (int r = 0; r < RB; ++r) acc[r][g] = (v4i){0, 0, 0, 0};
     }
 
-    static_assert(!ONE || RB * MT == 1, "single batch: one row block, one token group");
-    constexpr int PF = ONE ? 8 : (RB * MT == 1 ? 4 : (RB * MT == 2 ? 3 : (MT <= 2 ? 2 : 1)));  // bounded by the register file
+    static_assert(!ONE || MT == 1, "single batch: one token group");
+    constexpr int PF = ONE ? (RB == 1 ? 8 : (RB == 2 ? 4 : 3))
+                           : (RB * MT == 1 ? 4 : (RB * MT == 2 ? 3 : (MT <= 2 ? 2 : 1)));  // bounded by the register file
     // All loads of a batch of PF k-tiles are issued before the first MFMA of the batch, and the next
     // batch is requested while the current one is computed: the weight stream is what the kernel waits for.
     uint4 wcur[PF][RB], wnxt[ONE ? 1 : PF][RB];
@@ -755,37 +750,30 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         rowsum[g] = sum_over_lane_groups(rowsum[g]);
         if (lane < 16) red_sum[wave][g][lane] = rowsum[g];
     }
-    if (wave > 0) {
 #pragma unroll
-        for (int r = 0; r < RB; ++r)
+    for (int r = 0; r < RB; ++r)
 #pragma unroll
-            for (int g = 0; g < MT; ++g)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) red[wave - 1][r][g][lane][i] = acc[r][g][i];
-    }
+        for (int g = 0; g < MT; ++g)
+            *reinterpret_cast<v4i *>(&red[wave][r][g][lane][0]) = acc[r][g];
     lds_barrier();
-    if (wave == 0) {
+    if (finisher) {  // uniform over the wavefront
+        const int n = (rb0 + fr) * TILE_ROWS + lr;  // result register i of lane l is C[4*(l/16) + i][l mod 16]
+        const v4i s0 = *reinterpret_cast<const v4i *>(&red[0][fr][fg][lane][0]), s1 = *reinterpret_cast<const v4i *>(&red[1][fr][fg][lane][0]);
+        const v4i s2 = *reinterpret_cast<const v4i *>(&red[2][fr][fg][lane][0]), s3 = *reinterpret_cast<const v4i *>(&red[3][fr][fg][lane][0]);
+        const v4i sum = s0 + s1 + s2 + s3;
 #pragma unroll
-        for (int r = 0; r < RB; ++r) {
-            const int n = (rb0 + r) * TILE_ROWS + lr;  // result register i of lane l is C[4*(l/16) + i][l mod 16]
-#pragma unroll
-            for (int g = 0; g < MT; ++g) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int tl = lg * 4 + i, t = 16 * g + tl;
-                    if (n < P.n && t < p.m) {
-                        const int asum = red_sum[0][g][tl] + red_sum[1][g][tl] + red_sum[2][g][tl] + red_sum[3][g][tl];
-                        const int total = acc[r][g][i] + red[0][r][g][lane][i] + red[1][r][g][lane][i] +
-                                          red[2][r][g][lane][i] - asum;
-                        const size_t o = (size_t)t * P.n + n;
-                        if (P.acc) P.acc[o] = total;
-                        if (P.out) {
-                            float v = f32_div(f32_mul((float)total, ws), e_scale[g][i]);
-                            if (P.bias) v = f32_add(v, e_bias[r]);
-                            if (P.residual) v = f32_add(v, e_res[r][g][i]);
-                            P.out[o] = v;
-                        }
-                    }
+        for (int i = 0; i < 4; ++i) {
+            const int tl = lg * 4 + i, t = 16 * fg + tl;
+            if (n < P.n && t < p.m) {
+                const int asum = red_sum[0][fg][tl] + red_sum[1][fg][tl] + red_sum[2][fg][tl] + red_sum[3][fg][tl];
+                const int total = sum[i] - asum;
+                const size_t o = (size_t)t * P.n + n;
+                if (P.acc) P.acc[o] = total;
+                if (P.out) {
+                    float v = f32_div(f32_mul((float)total, ws), e_scale[i]);
+                    if (P.bias) v = f32_add(v, e_bias);
+                    if (P.residual) v = f32_add(v, e_res[i]);
+                    P.out[o] = v;
                 }
             }
         }
@@ -916,9 +904,11 @@ int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const floa
     p.nproj = nproj; p.a = a; p.a_scale = a_scale; p.m = (int)m; p.k = (int)k; p.kt_count = (int)k_tiles(k);
     if (end == 0) return BITNET_HIP_OK;
     const bool fast = k % TILE_K == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0;
-    if constexpr (RB * MT == 1) {
-        if (fast && p.kt_count > 16 && p.kt_count <= 32) {  // more than one batch of 4 tiles per wavefront, at most one of 8
-            hipLaunchKernelGGL((gemv_mfma_kernel<1, 1, true, true>), dim3((unsigned)end), dim3(256), 0, stream, p);
+    if constexpr (MT == 1) {
+        // more than one double-buffered batch per wavefront, but few enough k-tiles for one batch without the second buffer
+        constexpr int PF2 = RB == 1 ? 4 : (RB == 2 ? 3 : 2), PF1 = RB == 1 ? 8 : (RB == 2 ? 4 : 3);
+        if (fast && p.kt_count > 4 * PF2 && p.kt_count <= 4 * PF1) {
+            hipLaunchKernelGGL((gemv_mfma_kernel<RB, 1, true, true>), dim3((unsigned)end), dim3(256), 0, stream, p);
             BITNET_HIP_CHECK_LAUNCH("gemv_mfma_kernel");
             return BITNET_HIP_OK;
         }
