@@ -1,11 +1,13 @@
 // Stand-alone fused RMSNorm + per-token absmax int8 activation quantiser for gfx950 (the arithmetic and the
 // declared summation order are in rowquant.hpp; the decode GEMV runs the same code inside its prologue).
 //
-// Two launch shapes, same bits:
-//   act_quant_block_kernel  one 256-thread workgroup per token row, the row held in registers between the three
-//                           passes (sum of squares, absmax, quantise): 4*K bytes read once, K + 8 bytes written.
-//                           The usual shape (k <= 7168 with aligned rows), for one row or thousands.
-//   act_quant_wave_kernel   one wavefront per token row: many rows of any length or alignment.
+// Three launch shapes, same bits:
+//   act_quant_block_kernel    one 256-thread workgroup per token row, the row held in registers between the three
+//                             passes (sum of squares, absmax, quantise): 4*K bytes read once, K + 8 bytes written.
+//                             The usual shape (k <= 7168 with aligned rows), for one row or thousands.
+//   act_quant_block16_kernel  one 1024-thread workgroup per token row: up to 16 rows (a decode batch), where the
+//                             launch is as long as one row takes.
+//   act_quant_wave_kernel     one wavefront per token row: many rows of any length or alignment.
 #include "kernels.hpp"
 #include "rowquant.hpp"
 
@@ -216,6 +218,96 @@ __global__ __launch_bounds__(256) void act_quant_block_kernel(ActQuantParams p)
     }
 }
 
+// One workgroup of 16 wavefronts per row, for the few rows of a decode batch: a row is then one workgroup's whole
+// work, so its time is the row's arithmetic divided by the threads that share it.  Thread t owns chunks t, t + 1024
+// (NCHB of them; k <= 4096 * NCHB, 16-byte aligned rows).  The sum of squares keeps the declared order: chunk c belongs
+// to virtual lane c % 256, so threads 0..255 also fetch the chunks of their lane and run its chain, then the four 64-lane
+// butterflies.  Same bits as the other two kernels.
+template <int MODE, int NCHB>
+__global__ __launch_bounds__(1024) void act_quant_block16_kernel(ActQuantParams p)
+{
+    __shared__ float red_f[2][16];
+    __shared__ int red_i[16];
+    const RowSource &src = p.src;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const size_t row = blockIdx.x;
+    const int k = src.k, chunks = k >> 2;
+    const bool norm = src.gamma != nullptr;
+    const bool chain = norm && src.sum_order != BITNET_HIP_SUM_SEQUENTIAL && wave < 4;
+    constexpr int NSS = 4 * NCHB;
+
+    // all loads up front, unconditional (clamped indices, values discarded)
+    float4 v[NCHB], gm[NCHB], vs[NSS];
+#pragma unroll
+    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(src, row, min(tid + 1024 * i, chunks - 1));
+    if (chain) {
+#pragma unroll
+        for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(src, row, min(tid + 256 * i, chunks - 1));
+    }
+    if (norm) {
+#pragma unroll
+        for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(src, min(tid + 1024 * i, chunks - 1), true);
+    }
+#pragma unroll
+    for (int i = 0; i < NCHB; ++i)
+        if (tid + 1024 * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+    if (norm) {
+        float ss;
+        if (src.sum_order == BITNET_HIP_SUM_SEQUENTIAL) {
+            ss = sum_squares_sequential<MODE>(src, row);
+        } else {
+            if (chain) {  // thread tid < 256 is virtual lane tid
+                float part = 0.0f;
+#pragma unroll
+                for (int i = 0; i < NSS; ++i)
+                    if (tid + 256 * i < chunks) part = sum_squares4(part, vs[i]);  // chunks past the end would add +0
+                part = wave_sum_f32(part);
+                if (lane == 0) red_f[0][wave] = part;
+            }
+            lds_barrier();
+            ss = f32_add(f32_add(f32_add(red_f[0][0], red_f[0][1]), red_f[0][2]), red_f[0][3]);
+        }
+        const RowDivisor rdiv = make_row_divisor(rms_from_ss(ss, k, src.eps));
+#pragma unroll
+        for (int i = 0; i < NCHB; ++i)
+            if (tid + 1024 * i < chunks) v[i] = normalize4(v[i], rdiv, gm[i]);
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCHB; ++i) amax = absmax4(amax, v[i]);
+    amax = wave_max_f32(amax);
+    if (lane == 0) red_f[1][wave] = amax;
+    lds_barrier();
+    amax = red_f[1][0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) amax = fmaxf(amax, red_f[1][w]);
+    const float scale = scale_from_absmax(amax);
+
+    int isum = 0;
+#pragma unroll
+    for (int i = 0; i < NCHB; ++i) {
+        const int c = tid + 1024 * i;
+        if (c < chunks) {
+            const size_t base = row * (size_t)k + 4 * (size_t)c;
+            *reinterpret_cast<uint32_t *>(p.q + base) = quant4_packed(v[i], scale, &isum);
+            if (p.y) *reinterpret_cast<float4 *>(p.y + base) = v[i];
+        }
+    }
+    isum = wave_sum_i32(isum);
+    if (lane == 0) red_i[wave] = isum;
+    lds_barrier();
+    if (tid == 0) {
+        p.a_scale[row] = scale;
+        if (p.a_sum) {
+            int total = 0;
+#pragma unroll
+            for (int w = 0; w < 16; ++w) total += red_i[w];
+            p.a_sum[row] = total;
+        }
+    }
+}
+
 template <int MODE, int NCH, bool VEC>
 void launch_wave(const ActQuantParams &p, hipStream_t s)
 {
@@ -235,6 +327,12 @@ template <int MODE>
 void launch_mode(const ActQuantParams &p, bool vec, hipStream_t s)
 {
     const int chunks = (p.src.k + 3) >> 2;
+    // Few rows (a decode batch): 16 wavefronts per row.
+    if (p.m <= 16 && vec && chunks <= 2048) {
+        if (chunks <= 1024) hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 1>), dim3((unsigned)p.m), dim3(1024), 0, s, p);
+        else hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 2>), dim3((unsigned)p.m), dim3(1024), 0, s, p);
+        return;
+    }
     // A workgroup per row for few rows, and for any number of rows whose chunks fit the threads' registers: with
     // more, shorter-lived workgroups in flight the load latency of one overlaps the arithmetic of others (measured
     // at 2048 rows: 8.0 us against 9.0 us at k = 2560, 16.9 us against 23.1 us at k = 6912).
