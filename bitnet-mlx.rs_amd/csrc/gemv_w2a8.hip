@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
 #pragma unroll
     for (int u = 0; u < GEMV_PREFETCH; ++u) {
         int kt = wave + 4 * u;
-        wbuf[u] = tiles[(size_t)min(kt, p.kt_count - 1) * 64 + lane];  // unconditional: the waits can be counted
+        wbuf[u] = load_weight_slot(tiles + (size_t)min(kt, p.kt_count - 1) * 64 + lane);  // unconditional: the waits can be counted
     }
 
     if constexpr (MODE == MODE_PREQUANT) {
@@ -242,7 +242,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(GemvParams p)
             uint4 wnext[GEMV_PREFETCH];
 #pragma unroll
             for (int u = 0; u < GEMV_PREFETCH; ++u)
-                wnext[u] = tiles[(size_t)min(kt0 + 4 * (GEMV_PREFETCH + u), p.kt_count - 1) * 64 + lane];
+                wnext[u] = load_weight_slot(tiles + (size_t)min(kt0 + 4 * (GEMV_PREFETCH + u), p.kt_count - 1) * 64 + lane);
             dot_batch(kt0);
 #pragma unroll
             for (int u = 0; u < GEMV_PREFETCH; ++u) wbuf[u] = wnext[u];
@@ -328,7 +328,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
     for (int r = 0; r < RBW; ++r)
 #pragma unroll
         for (int u = 0; u < NCH; ++u)  // row blocks past the end repeat the last one; their results are not stored
-            wt[r][u] = tiles[((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 4 * u, p.kt_count - 1)) * 64];
+            wt[r][u] = load_weight_slot(tiles + ((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 4 * u, p.kt_count - 1)) * 64);
 #pragma unroll
     for (int i = 0; i < NCH; ++i)
         if (tid + 256 * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -472,7 +472,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p)
     for (int r = 0; r < RBW; ++r)
 #pragma unroll
         for (int i = 0; i < NCHB; ++i)
-            wt[r][i] = tiles[((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 16 * i, p.kt_count - 1)) * 64];
+            wt[r][i] = load_weight_slot(tiles + ((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 16 * i, p.kt_count - 1)) * 64);
     if (tid < RBW * TILE_ROWS) tot[tid >> 4][tid & 15] = 0;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i)
@@ -634,9 +634,9 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         for (int r = 0; r < RB; ++r) {
             const int rb = rb0 + r;
             if constexpr (FAST)  // results of row blocks past the end are never stored
-                w[r] = wbase[((size_t)min(rb, rb_count - 1) * p.kt_count + min(kt, p.kt_count - 1)) * 64];
+                w[r] = load_weight_slot(wbase + ((size_t)min(rb, rb_count - 1) * p.kt_count + min(kt, p.kt_count - 1)) * 64);
             else
-                w[r] = rb < rb_count ? wbase[((size_t)rb * p.kt_count + kt) * 64]
+                w[r] = rb < rb_count ? load_weight_slot(wbase + ((size_t)rb * p.kt_count + kt) * 64)
                                      : make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
         }
     };

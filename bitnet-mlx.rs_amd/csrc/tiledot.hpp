@@ -4,6 +4,15 @@
 
 namespace bitnet {
 
+// A slot of a weight tile (16 bytes per lane).  The weights of a GEMV are read once per call and never again, so the
+// load is non-temporal (no cache line kept for them): measured 5.1 -> 5.7 TB/s on a 128 MiB weight matrix.
+__device__ __forceinline__ uint4 load_weight_slot(const uint4 *ptr)
+{
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    const v4u v = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(ptr));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
 __device__ __forceinline__ int dot4(uint32_t a, uint32_t c, int acc)
 {
     return __builtin_amdgcn_sdot4((int)a, (int)c, acc, false);
