@@ -254,6 +254,20 @@ int bitnet_hip_quantize_activations_i8(const float *x, const float *x2, size_t l
                             a_sum, y_f32, as_stream(stream));
 }
 
+// ---- lookup-table kernels ----------------------------------------------------------------------------
+
+int bitnet_hip_lookup_compute(int kind, const int8_t *weights, size_t n_weights, const float *inputs, size_t n_inputs,
+                              float *output, size_t n_output, void *stream)
+{
+    if (kind != BITNET_HIP_LOOKUP_TERNARY && kind != BITNET_HIP_LOOKUP_I2S)
+        return fail(BITNET_HIP_INVALID_CONFIG, "lookup_compute: unknown kind %d", kind);
+    if (n_weights == 0 || n_inputs == 0 || n_output == 0) return fail(BITNET_HIP_INVALID_CONFIG, "Empty input arrays");
+    if (!weights || !inputs || !output) return fail(BITNET_HIP_NULL_POINTER, "lookup_compute: null buffer");
+    size_t n = n_weights < n_inputs ? n_weights : n_inputs;
+    if (n_output < n) n = n_output;
+    return launch_lookup_compute(kind, weights, inputs, output, n, as_stream(stream));
+}
+
 // ---- weight side -----------------------------------------------------------------------------------
 
 size_t bitnet_hip_packed_size(size_t count) { return (count + 3) / 4; }

@@ -22,6 +22,7 @@ int launch_act_quant(const float *x, const float *x2, size_t ldx, size_t m, size
 // weight_prep.hip
 int launch_pack_2bit(const int8_t *q, size_t count, uint8_t *packed, hipStream_t stream);
 int launch_unpack_2bit(const uint8_t *packed, size_t count, int8_t *q, hipStream_t stream);
+int launch_lookup_compute(int kind, const int8_t *w, const float *x, float *out, size_t n, hipStream_t stream);
 // base-3 bytes (5 values each): pack, unpack, and re-code into the 2-bit bytes (4 values each)
 int launch_pack_base3(const int8_t *q, size_t count, uint8_t *packed, hipStream_t stream);
 int launch_unpack_base3(const uint8_t *packed, size_t count, int8_t *q, hipStream_t stream);

@@ -85,6 +85,18 @@ __global__ __launch_bounds__(256) void base3_to_2bit_kernel(const uint8_t *base3
     packed[b] = (uint8_t)byte;
 }
 
+// TernaryLookupKernel / I2SLookupKernel::compute (bitnet-core/src/cpu/kernels/generic.rs:54-75,118-139).
+__global__ __launch_bounds__(256) void lookup_compute_kernel(int kind, const int8_t *w, const float *x, float *out, size_t n)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int v = w[i];
+    float l;
+    if (kind == BITNET_HIP_LOOKUP_TERNARY) l = v == -1 ? -1.0f : (v == 1 ? 1.0f : 0.0f);
+    else l = v == -2 ? -2.0f : (v == -1 ? -1.0f : (v == 1 ? 1.0f : 0.0f));
+    out[i] = f32_mul(x[i], l);
+}
+
 __device__ __forceinline__ double wave_sum_f64(double p)
 {
 #pragma unroll
@@ -220,6 +232,14 @@ int launch_unpack_2bit(const uint8_t *packed, size_t count, int8_t *q, hipStream
     if (count == 0) return BITNET_HIP_OK;
     hipLaunchKernelGGL(unpack_2bit_kernel, dim3(blocks_for(count, 256)), dim3(256), 0, stream, packed, count, q);
     BITNET_HIP_CHECK_LAUNCH("unpack_2bit_kernel");
+    return BITNET_HIP_OK;
+}
+
+int launch_lookup_compute(int kind, const int8_t *w, const float *x, float *out, size_t n, hipStream_t stream)
+{
+    if (n == 0) return BITNET_HIP_OK;
+    hipLaunchKernelGGL(lookup_compute_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, kind, w, x, out, n);
+    BITNET_HIP_CHECK_LAUNCH("lookup_compute_kernel");
     return BITNET_HIP_OK;
 }
 

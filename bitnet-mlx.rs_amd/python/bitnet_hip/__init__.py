@@ -84,6 +84,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_init": (i32, [i32]),
         "bitnet_hip_device_info": (i32, [C.c_char_p, sz, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz)]),
         "bitnet_hip_quantize_activations_i8": (i32, [vp, vp, sz, sz, sz, i32, sz, sz, vp, f32, i32, vp, vp, vp, vp, vp]),
+        "bitnet_hip_lookup_compute": (i32, [i32, vp, sz, vp, sz, vp, sz, vp]),
         "bitnet_hip_packed_size": (sz, [sz]),
         "bitnet_hip_pack_ternary_2bit": (i32, [vp, sz, vp, vp]),
         "bitnet_hip_unpack_ternary_2bit": (i32, [vp, sz, vp, vp]),
@@ -312,6 +313,40 @@ class BitPacked2BitPacker:
 
     def unpack(self, packed: torch.Tensor, element_count: int) -> torch.Tensor:
         return unpack_ternary_2bit(packed, element_count)
+
+
+LOOKUP_TERNARY, LOOKUP_I2S = 0, 1
+
+
+class _HipLookupKernel:
+    """compute(weights i8, inputs f32, output f32) on device tensors: output[i] = inputs[i] * lut[weights[i]] over the
+    shortest of the three; any empty tensor is an error (bitnet-core/src/cpu/kernels/generic.rs:54-75,118-139)."""
+    _kind = LOOKUP_TERNARY
+    _name = ""
+
+    def compute(self, weights: torch.Tensor, inputs: torch.Tensor, output: torch.Tensor, stream=None):
+        for t, dt, nm in ((weights, torch.int8, "weights"), (inputs, torch.float32, "inputs"), (output, torch.float32, "output")):
+            if t.numel():
+                _dev(t, dt, nm)
+        _check(load_library().bitnet_hip_lookup_compute(self._kind, _ptr(weights) if weights.numel() else None, weights.numel(),
+                                                        _ptr(inputs) if inputs.numel() else None, inputs.numel(),
+                                                        _ptr(output) if output.numel() else None, output.numel(), _stream(stream)))
+
+    def name(self) -> str:
+        return self._name
+
+    def optimal_batch_size(self) -> int:
+        return 1 << 20  # elements per call from which the launch cost is small beside the 9 bytes per element moved
+
+
+class HipTernaryLookupKernel(_HipLookupKernel):
+    """Mirror of TernaryLookupKernel (bitnet-core/src/cpu/mod.rs:132-149): weights in {-1, 0, +1}."""
+    _kind, _name = LOOKUP_TERNARY, "HIP-gfx950-Ternary"
+
+
+class HipI2SLookupKernel(_HipLookupKernel):
+    """Mirror of I2SLookupKernel (bitnet-core/src/cpu/mod.rs:151-169): weights in {-2, -1, 0, +1}."""
+    _kind, _name = LOOKUP_I2S, "HIP-gfx950-I2S"
 
 
 class Base3PackedPacker:

@@ -32,6 +32,8 @@ pub const BITNET_HIP_TERNARY_MEAN_THRESHOLD: c_int = 1;
 pub const BITNET_HIP_INPUT_PLAIN: c_int = 0;
 pub const BITNET_HIP_INPUT_RELU2_MUL: c_int = 1;
 pub const BITNET_HIP_INPUT_GQA_BROADCAST: c_int = 2;
+pub const BITNET_HIP_LOOKUP_TERNARY: c_int = 0;
+pub const BITNET_HIP_LOOKUP_I2S: c_int = 1;
 
 extern "C" {
     pub fn bitnet_hip_last_error() -> *const c_char;
@@ -43,6 +45,8 @@ extern "C" {
                                               input_mode: c_int, gqa_group: usize, head_dim: usize, gamma: *const f32,
                                               eps: f32, sum_order: c_int, q: *mut i8, a_scale: *mut f32,
                                               a_sum: *mut i32, y_f32: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_lookup_compute(kind: c_int, weights: *const i8, n_weights: usize, inputs: *const f32,
+                                     n_inputs: usize, output: *mut f32, n_output: usize, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_packed_size(count: usize) -> usize;
     pub fn bitnet_hip_pack_ternary_2bit(q: *const i8, count: usize, packed: *mut u8, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_unpack_ternary_2bit(packed: *const u8, count: usize, q: *mut i8, stream: *mut c_void) -> c_int;

@@ -158,3 +158,26 @@ impl HipBackend {
         })
     }
 }
+
+/// Device-side stand-in for the kernels `KernelSelector` hands out (bitnet-core/src/cpu/mod.rs:107-127): the
+/// arithmetic of `TernaryLookupKernel::compute` / `I2SLookupKernel::compute` (bitnet-core/src/cpu/mod.rs:132-169,
+/// kernels/generic.rs:54-75,118-139) on device slices (pointer, length).  A crate that owns the trait definitions
+/// implements them for this type by staging its host slices through device buffers.
+pub struct HipLookupKernel {
+    kind: c_int,
+    stream: *mut c_void,
+}
+impl HipLookupKernel {
+    pub fn ternary() -> Self { Self { kind: ffi::BITNET_HIP_LOOKUP_TERNARY, stream: ptr::null_mut() } }
+    pub fn i2s() -> Self { Self { kind: ffi::BITNET_HIP_LOOKUP_I2S, stream: ptr::null_mut() } }
+    /// `output[i] = inputs[i] * lut[weights[i]]` over the shortest of the three; an empty slice is an error.
+    pub fn compute(&self, weights: (*const i8, usize), inputs: (*const f32, usize), output: (*mut f32, usize)) -> HipResult<()> {
+        check(unsafe {
+            ffi::bitnet_hip_lookup_compute(self.kind, weights.0, weights.1, inputs.0, inputs.1, output.0, output.1, self.stream)
+        })
+    }
+    pub fn name(&self) -> &'static str {
+        if self.kind == ffi::BITNET_HIP_LOOKUP_TERNARY { "HIP-gfx950-Ternary" } else { "HIP-gfx950-I2S" }
+    }
+    pub fn optimal_batch_size(&self) -> usize { 1 << 20 }
+}

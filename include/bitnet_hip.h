@@ -96,6 +96,20 @@ int bitnet_hip_quantize_activations_i8(const float *x, const float *x2, size_t l
                                        const float *gamma, float eps, int sum_order, int8_t *q,
                                        float *a_scale, int32_t *a_sum, float *y_f32, void *stream);
 
+/* ---- lookup-table kernels --------------------------------------------------------------------- */
+
+#define BITNET_HIP_LOOKUP_TERNARY 0 /* weights {-1,0,+1}, anything else counts as 0 */
+#define BITNET_HIP_LOOKUP_I2S 1     /* weights {-2,-1,0,+1}, anything else counts as 0 */
+
+/* output[i] = inputs[i] * lut[weights[i]] over min(n_weights, n_inputs, n_output) elements, device buffers.
+ * INVALID_CONFIG ("Empty input arrays") when one of the three lengths is 0.
+ *   replaces TernaryLookupKernel::compute and I2SLookupKernel::compute (bitnet-core/src/cpu/mod.rs:132-169) as
+ *   GenericTernaryKernel / GenericI2SKernel implement them (bitnet-core/src/cpu/kernels/generic.rs:54-75,118-139),
+ *   the kernels KernelSelector hands out (bitnet-core/src/cpu/mod.rs:107-127).  Element-wise and memory-bound
+ *   (9 bytes per element); it is not on the BitLinear path, which never expands weights to f32. */
+int bitnet_hip_lookup_compute(int kind, const int8_t *weights, size_t n_weights, const float *inputs, size_t n_inputs,
+                              float *output, size_t n_output, void *stream);
+
 /* ---- weight side ------------------------------------------------------------------------------ */
 
 /* Bytes of `count` ternary values in the reference's 2-bit format: (count + 3) / 4

@@ -13,6 +13,7 @@
  * Parity status of each function (what pins it besides this restatement):
  *   orc_pack_2bit / orc_unpack_2bit      pinned: byte fixtures and round trips held by the reference's tests
  *   orc_gguf_decode_ternary              pinned: the reference's own decode test (header + 0x24 -> [-1,0,1,-1])
+ *   orc_lookup_compute                   pinned: the reference's two compute fixtures and its index tables (generic.rs tests)
  *   orc_pack_base3 / orc_unpack_base3    pinned: the reference's four encoding fixtures (140, 0, 242, 121) and
  *                                        its round-trip test
  *   orc_round_clip, orc_ternarize_*      pinned: reference tables (round_clip ties, strict '>' threshold)
@@ -369,6 +370,27 @@ void orc_unpack_base3(const uint8_t *packed, size_t n, int8_t *q)
         for (size_t j = 0; j < i % 5; ++j) rem /= 3;
         q[i] = (int8_t)(rem % 3) - 1;
     }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Lookup-table kernels.   reference: bitnet-core/src/cpu/mod.rs:132-169 (traits), kernels/generic.rs:28-75,95-148
+ *   ternary: output[i] = inputs[i] * lut[idx(w[i])], lut = {-1, 0, +1, 0}, idx(-1,0,1,other) = 0,1,2,3
+ *   i2s:     lut = {-2, -1, 0, +1, 0}, idx(-2,-1,0,1,other) = 0,1,2,3,4
+ *   over min(len) elements; any empty array is an error (returns -1).  The product is a real f32
+ *   multiplication (0 * inf = NaN, as in the reference).
+ * ---------------------------------------------------------------------------------------------- */
+int orc_lookup_compute(int kind, const int8_t *w, size_t nw, const float *x, size_t nx, float *out, size_t nout)
+{
+    if (nw == 0 || nx == 0 || nout == 0) return -1;
+    size_t n = nw < nx ? nw : nx;
+    if (nout < n) n = nout;
+    for (size_t i = 0; i < n; ++i) {
+        float l;
+        if (kind == 0) l = w[i] == -1 ? -1.0f : (w[i] == 1 ? 1.0f : 0.0f);
+        else l = w[i] == -2 ? -2.0f : (w[i] == -1 ? -1.0f : (w[i] == 1 ? 1.0f : 0.0f));
+        out[i] = x[i] * l;
+    }
+    return 0;
 }
 
 /* ------------------------------------------------------------------------------------------------

@@ -162,6 +162,17 @@ def unpack_2bit(packed, n):
     return q
 
 
+def lookup_compute(kind, w, x, nout=None):
+    """TernaryLookupKernel / I2SLookupKernel::compute (bitnet-core/src/cpu/kernels/generic.rs:54-75,118-139);
+    kind 0 = ternary, 1 = i2s.  Returns the output array (length nout, elements past min(len) left at zero) or None."""
+    w = np.ascontiguousarray(w, dtype=np.int8).ravel()
+    x = _f32(np.asarray(x).ravel())
+    nout = min(w.size, x.size) if nout is None else nout
+    out = np.zeros(nout, dtype=np.float32)
+    rc = lib().orc_lookup_compute(C.c_int(kind), _p(w), _sz(w.size), _p(x), _sz(x.size), _p(out), _sz(nout))
+    return None if rc != 0 else out
+
+
 def pack_base3(q):
     """Base3PackedPacker::pack (packing.rs:424-447): 5 values per byte, value j weighs 3^j."""
     q = np.ascontiguousarray(q, dtype=np.int8).ravel()

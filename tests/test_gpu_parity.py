@@ -451,6 +451,34 @@ def test_bitlinear_base3_weights_match_2bit_weights(n, k, on_device):
         assert err.value.status == bh.SHAPE_MISMATCH
 
 
+@pytest.mark.parametrize("kind,cls", [(bh.LOOKUP_TERNARY, bh.HipTernaryLookupKernel), (bh.LOOKUP_I2S, bh.HipI2SLookupKernel)],
+                         ids=["ternary", "i2s"])
+def test_lookup_kernels_bit_exact(kind, cls):
+    """TernaryLookupKernel / I2SLookupKernel::compute on the GPU: bit-identical to the oracle, out-of-table weights,
+    non-finite inputs and signed zeros included; the shortest buffer decides the length; empty buffers are errors."""
+    rng = np.random.default_rng(kind)
+    kernel = cls()
+    for n in (1, 5, 1000, 100003):
+        w = rng.integers(-3, 4, size=n).astype(np.int8)
+        x = rng.standard_normal(n, dtype=f32)
+        x[rng.integers(0, n, size=max(1, n // 50))] = np.inf
+        x[rng.integers(0, n, size=max(1, n // 50))] = np.nan
+        out = torch.zeros((n,), device="cuda", dtype=torch.float32)
+        kernel.compute(dev(w), dev(x), out)
+        ref = orc.lookup_compute(kind, w, x)
+        assert np.array_equal(host(out).view(np.uint32), ref.view(np.uint32))
+    out = torch.full((6,), 7.0, device="cuda", dtype=torch.float32)
+    kernel.compute(dev(np.array([1, -1, 1, 1], np.int8)), dev(np.array([2.0, 3.0, 4.0], f32)), out)
+    assert host(out).tolist() == [2.0, -3.0, 4.0, 7.0, 7.0, 7.0]
+    empty_w, empty_x = torch.empty((0,), dtype=torch.int8, device="cuda"), torch.empty((0,), dtype=torch.float32, device="cuda")
+    for args in ((empty_w, dev(np.ones(2, f32)), out), (dev(np.ones(2, np.int8)), empty_x, out),
+                 (dev(np.ones(2, np.int8)), dev(np.ones(2, f32)), empty_x)):
+        with pytest.raises(bh.BitLinearError) as err:
+            kernel.compute(*args)
+        assert err.value.status == bh.INVALID_CONFIG
+    assert kernel.name() and kernel.optimal_batch_size() > 0
+
+
 def test_bitlinear_forward_prefill_uses_quantiser_row_sums():
     """BitLinear.forward at a prefill token count: quantiser -> row sums -> LDS-direct GEMM, bit-exact."""
     rng = np.random.default_rng(77)

@@ -494,3 +494,26 @@ def test_base3_roundtrip_and_closed_forms():
     high = np.array([255, 243, 250], dtype=np.uint8)
     want = np.stack([(high.astype(np.int64) // 3 ** j) % 3 for j in range(5)], axis=1).ravel() - 1
     assert np.array_equal(orc.unpack_base3(high, 15), want.astype(np.int8))
+
+
+@pytest.mark.parametrize("case", G["lookup_compute"], ids=lambda c: "i2s" if c["kind"] else "ternary")
+def test_lookup_kernel_fixtures(case):
+    """GenericTernaryKernel / GenericI2SKernel::compute: the reference's two compute vectors."""
+    out = orc.lookup_compute(case["kind"], case["weights"], case["inputs"])
+    assert out.tolist() == case["expected"]
+
+
+def test_lookup_kernel_edges():
+    """Values outside a table count as 0 (the reference's index fallback); the shortest array decides the length;
+    an empty array is an error; 0 * inf is NaN, as a real multiplication gives."""
+    bad = G["lookup_index_fallback"]["weight"]
+    for kind in (0, 1):
+        assert orc.lookup_compute(kind, [bad, -128, 127], [1.0, 2.0, 3.0]).tolist() == [0.0, 0.0, 0.0]
+        assert orc.lookup_compute(kind, [1, 1, 1], [5.0, 6.0], nout=4).tolist() == [5.0, 6.0, 0.0, 0.0]
+        assert orc.lookup_compute(kind, [], [1.0]) is None
+        assert orc.lookup_compute(kind, [1], []) is None
+        assert orc.lookup_compute(kind, [1], [1.0], nout=0) is None
+    out = orc.lookup_compute(0, [0, 1, -1], [np.inf, np.inf, np.nan])
+    assert np.isnan(out[0]) and out[1] == np.inf and np.isnan(out[2])
+    assert orc.lookup_compute(0, [-2], [3.0]).tolist() == [0.0] and orc.lookup_compute(1, [-2], [3.0]).tolist() == [-6.0]
+    assert np.signbit(orc.lookup_compute(0, [0], [-3.0])[0])  # -3 * 0 = -0
