@@ -643,21 +643,24 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 
     // scales the epilogue will need (result register i of a lane belongs to token 16g + 4*(lane/16) + i): requested
     // now, so that their latency is not paid at the end
-    // The RB * MT <= 4 fragments (row block, token group) are finished by one wavefront each: fragment
-    // (fr, fg) = (wave / MT, wave % MT).  Its scale, bias and residual are requested now (clamped indices; unused
-    // values are discarded).
-    static_assert(RB * MT <= 4, "one wavefront per fragment");
+    // The RB * MT fragments (row block, token group) are finished by the wavefronts in turn: fragment
+    // q = wave + 4 * f is (row block q / MT, token group q % MT).  Scales, bias and residuals are requested now
+    // (clamped indices; unused values are discarded).
+    constexpr int NFRAG = RB * MT, FPW = (NFRAG + 3) / 4;  // fragments, fragments per wavefront
     const float ws = P.out ? *P.w_scale : 0.0f;
-    const int fr = min(wave / MT, RB - 1), fg = wave % MT;
-    const bool finisher = wave < RB * MT;
-    const int e_n = min((rb0 + fr) * TILE_ROWS + lr, P.n - 1);
-    const float e_bias = (finisher && P.bias) ? P.bias[e_n] : 0.0f;
-    float e_scale[4], e_res[4];
+    float e_bias[FPW], e_scale[FPW][4], e_res[FPW][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int t = min(16 * fg + lg * 4 + i, p.m - 1);
-        e_scale[i] = (finisher && P.out) ? p.a_scale[t] : 1.0f;
-        e_res[i] = (finisher && P.residual) ? P.residual[(size_t)t * P.n + e_n] : 0.0f;
+    for (int f = 0; f < FPW; ++f) {
+        const int q = min(wave + 4 * f, NFRAG - 1), fr = q / MT, fg = q % MT;
+        const bool mine = wave + 4 * f < NFRAG;
+        const int e_n = min((rb0 + fr) * TILE_ROWS + lr, P.n - 1);
+        e_bias[f] = (mine && P.bias) ? P.bias[e_n] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = min(16 * fg + lg * 4 + i, p.m - 1);
+            e_scale[f][i] = (mine && P.out) ? p.a_scale[t] : 1.0f;
+            e_res[f][i] = (mine && P.residual) ? P.residual[(size_t)t * P.n + e_n] : 0.0f;
+        }
     }
 
     v4i acc[RB][MT];
@@ -756,7 +759,10 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         for (int g = 0; g < MT; ++g)
             *reinterpret_cast<v4i *>(&red[wave][r][g][lane][0]) = acc[r][g];
     lds_barrier();
-    if (finisher) {  // uniform over the wavefront
+#pragma unroll
+    for (int f = 0; f < FPW; ++f) {
+        if (wave + 4 * f >= NFRAG) break;  // uniform over the wavefront
+        const int q = wave + 4 * f, fr = q / MT, fg = q % MT;
         const int n = (rb0 + fr) * TILE_ROWS + lr;  // result register i of lane l is C[4*(l/16) + i][l mod 16]
         const v4i s0 = *reinterpret_cast<const v4i *>(&red[0][fr][fg][lane][0]), s1 = *reinterpret_cast<const v4i *>(&red[1][fr][fg][lane][0]);
         const v4i s2 = *reinterpret_cast<const v4i *>(&red[2][fr][fg][lane][0]), s3 = *reinterpret_cast<const v4i *>(&red[3][fr][fg][lane][0]);
@@ -770,9 +776,9 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
                 const size_t o = (size_t)t * P.n + n;
                 if (P.acc) P.acc[o] = total;
                 if (P.out) {
-                    float v = f32_div(f32_mul((float)total, ws), e_scale[i]);
-                    if (P.bias) v = f32_add(v, e_bias);
-                    if (P.residual) v = f32_add(v, e_res[i]);
+                    float v = f32_div(f32_mul((float)total, ws), e_scale[f][i]);
+                    if (P.bias) v = f32_add(v, e_bias[f]);
+                    if (P.residual) v = f32_add(v, e_res[f][i]);
                     P.out[o] = v;
                 }
             }
@@ -954,8 +960,10 @@ int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const f
             const int8_t *a0 = a + t0 * k;
             const float *s0 = a_scale ? a_scale + t0 : nullptr;
             int rc;
-            if (rows > 32) rc = launch_mfma_rb<1, 4>(sub, nproj, a0, s0, rows, k, stream);
-            else if (rows > 16) rc = launch_mfma_rb<1, 2>(sub, nproj, a0, s0, rows, k, stream);
+            if (rows > 32) rc = blocks >= 400 ? launch_mfma_rb<2, 4>(sub, nproj, a0, s0, rows, k, stream)
+                                              : launch_mfma_rb<1, 4>(sub, nproj, a0, s0, rows, k, stream);
+            else if (rows > 16) rc = blocks >= 400 ? launch_mfma_rb<2, 2>(sub, nproj, a0, s0, rows, k, stream)
+                                                   : launch_mfma_rb<1, 2>(sub, nproj, a0, s0, rows, k, stream);
             else if (blocks >= 800) rc = launch_mfma_rb<4, 1>(sub, nproj, a0, s0, rows, k, stream);
             else if (blocks >= 400) rc = launch_mfma_rb<2, 1>(sub, nproj, a0, s0, rows, k, stream);
             else rc = launch_mfma_rb<1, 1>(sub, nproj, a0, s0, rows, k, stream);
