@@ -426,15 +426,22 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
 // between quantiser and dot products; the partial sums of a row meet in LDS atomics.
 
 template <int MODE, bool NORM, int NCHB, int RBW>
-__global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p)
+__global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, const float *hot_x2, const float *hot_gamma, int hot_k, int hot_head_dim,
+                                                           int hot_gqa_group, GemvParams p)
 {
+    // The leading scalar arguments repeat what the first loads need (input row, RMSNorm weights, k): the file is
+    // compiled with kernel-argument preloading, so they arrive in registers with the wavefront instead of through a
+    // load from the argument buffer that the first address computation would have to wait for.
+    RowSource hot;
+    hot.x = hot_x; hot.x2 = hot_x2; hot.gamma = hot_gamma; hot.ldx = 0; hot.k = hot_k; hot.head_dim = hot_head_dim;
+    hot.gqa_group = hot_gqa_group; hot.sum_order = BITNET_HIP_SUM_BLOCK256; hot.eps = 0.0f;  // row 0 only: ldx unused
     extern __shared__ uint4 lds_a[];  // int8 activations, zero past K
     __shared__ float red_f[2][16];
     __shared__ int red_i[16];
     __shared__ int tot[RBW][TILE_ROWS];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int chunks = p.k >> 2, lds_words = p.kt_count * 64;
+    const int chunks = hot_k >> 2, lds_words = p.kt_count * 64;
 
     int pj = 0;
 #pragma unroll
@@ -451,11 +458,11 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p)
     float4 vs[NSS];
     uint4 wt[RBW][NCHB];
 #pragma unroll
-    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(p.src, 0, min(tid + 1024 * i, chunks - 1));
+    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(hot, 0, min(tid + 1024 * i, chunks - 1));
     if constexpr (NORM) {
         if (wave < 4) {  // thread tid < 256 is virtual lane tid: it fetches the lane's chunks itself (from L2)
 #pragma unroll
-            for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(p.src, 0, min(tid + 256 * i, chunks - 1));
+            for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(hot, 0, min(tid + 256 * i, chunks - 1));
         }
     }
     const int e_n = min((rb0 + (tid >> 4)) * TILE_ROWS + (tid & 15), P.n - 1);  // meaningful for tid < 16 * RBW
@@ -464,7 +471,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(GemvParams p)
     const float e_res = P.residual ? P.residual[e_n] : 0.0f;
     if constexpr (NORM) {
 #pragma unroll
-        for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(p.src, min(tid + 1024 * i, chunks - 1), true);
+        for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(hot, min(tid + 1024 * i, chunks - 1), true);
     }
     // k-tile kt holds chunks 64*kt .. 64*kt + 63: exactly what wavefront kt % 16 quantises, so a wavefront multiplies
     // the tiles of its own chunks (tiles and row blocks past the end repeat the last one; their results are not added)
@@ -863,10 +870,12 @@ int launch_fused16_mode(const GemvParams &p, hipStream_t stream)
     const bool norm = p.src.gamma != nullptr, one = (p.k >> 2) <= 1024;
     const size_t lds = (size_t)p.kt_count * 16 * sizeof(uint4);
     const dim3 grid((unsigned)p.proj[p.nproj - 1].rb_end);
-    if (norm && one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 1, RBW>), grid, dim3(1024), lds, stream, p);
-    else if (norm) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 2, RBW>), grid, dim3(1024), lds, stream, p);
-    else if (one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, 1, RBW>), grid, dim3(1024), lds, stream, p);
-    else hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, 2, RBW>), grid, dim3(1024), lds, stream, p);
+#define BITNET_HOT_ARGS p.src.x, p.src.x2, p.src.gamma, p.src.k, p.src.head_dim, p.src.gqa_group
+    if (norm && one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 1, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
+    else if (norm) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 2, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
+    else if (one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, 1, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
+    else hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, 2, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
+#undef BITNET_HOT_ARGS
     BITNET_HIP_CHECK_LAUNCH("gemv_fused16_kernel");
     return BITNET_HIP_OK;
 }

@@ -24,7 +24,8 @@ fn main() {
         let status = Command::new(&hipcc)
             .args(["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
                    "-fhip-fp32-correctly-rounded-divide-sqrt",
-                   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-c"])
+                   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                   "-mllvm", "-amdgpu-kernarg-preload-count=9", "-c"])
             .arg(csrc.join(k))
             .arg("-o")
             .arg(&obj)

@@ -50,5 +50,6 @@ def test_rust_build_script_compiles_the_same_sources_with_the_same_flags():
     makefile = (ROOT / "bitnet-mlx.rs_amd" / "Makefile").read_text()
     for src in re.findall(r"csrc/([a-z0-9_]+\.hip)", makefile):
         assert f'"{src}"' in build_rs, src
-    for flag in ("--offload-arch=gfx950", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-packed-fp32-ops"):
+    for flag in ("--offload-arch=gfx950", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-packed-fp32-ops",
+                 "-amdgpu-kernarg-preload-count=9"):
         assert flag in build_rs and flag.lstrip("-") in makefile.replace("$(ARCH)", "gfx950")
