@@ -224,11 +224,16 @@ __global__ __launch_bounds__(256) void act_quant_block_kernel(ActQuantParams p)
 // to virtual lane c % 256, so threads 0..255 also fetch the chunks of their lane and run its chain, then the four 64-lane
 // butterflies.  Same bits as the other two kernels.
 template <int MODE, int NCHB>
-__global__ __launch_bounds__(1024) void act_quant_block16_kernel(ActQuantParams p)
+__global__ __launch_bounds__(1024) void act_quant_block16_kernel(const float *hot_x, int hot_ldx, int hot_k, const float *hot_x2,
+                                                                const float *hot_gamma, int hot_head_dim, int hot_gqa_group,
+                                                                ActQuantParams p)
 {
     __shared__ float red_f[2][16];
     __shared__ int red_i[16];
-    const RowSource &src = p.src;
+    // the leading scalar arguments repeat what the first loads need; they are preloaded into registers (see the Makefile)
+    RowSource src = p.src;
+    src.x = hot_x; src.ldx = (size_t)hot_ldx; src.k = hot_k; src.x2 = hot_x2; src.gamma = hot_gamma;
+    src.head_dim = hot_head_dim; src.gqa_group = hot_gqa_group;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const size_t row = blockIdx.x;
     const int k = src.k, chunks = k >> 2;
@@ -328,9 +333,11 @@ void launch_mode(const ActQuantParams &p, bool vec, hipStream_t s)
 {
     const int chunks = (p.src.k + 3) >> 2;
     // Few rows (a decode batch): 16 wavefronts per row.
-    if (p.m <= 16 && vec && chunks <= 2048) {
-        if (chunks <= 1024) hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 1>), dim3((unsigned)p.m), dim3(1024), 0, s, p);
-        else hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 2>), dim3((unsigned)p.m), dim3(1024), 0, s, p);
+    if (p.m <= 16 && vec && chunks <= 2048 && p.src.ldx < (1u << 31)) {
+#define BITNET_HOT_ARGS p.src.x, (int)p.src.ldx, p.src.k, p.src.x2, p.src.gamma, p.src.head_dim, p.src.gqa_group
+        if (chunks <= 1024) hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 1>), dim3((unsigned)p.m), dim3(1024), 0, s, BITNET_HOT_ARGS, p);
+        else hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 2>), dim3((unsigned)p.m), dim3(1024), 0, s, BITNET_HOT_ARGS, p);
+#undef BITNET_HOT_ARGS
         return;
     }
     // A workgroup per row for few rows, and for any number of rows whose chunks fit the threads' registers: with

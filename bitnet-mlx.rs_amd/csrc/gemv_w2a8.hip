@@ -588,8 +588,10 @@ struct GemvMfmaParams {
 // ONE: the wavefront's k-tiles (at most 8: k <= 8192) form a single batch, requested as a whole at the start: one
 // memory latency instead of one per batch (RB = MT = 1 only, where the registers allow it).
 template <int RB, int MT, bool FAST, bool ONE = false>
-__global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
+__global__ __launch_bounds__(256) void gemv_mfma_kernel(const int8_t *hot_a, int hot_k, int hot_m, int hot_kt_count, GemvMfmaParams p)
 {
+    // the leading scalar arguments repeat the fields a, k, m and kt_count of p, which the first address computations need;
+    // they are preloaded into registers (see the Makefile) and used in place of the fields throughout
     __shared__ int red[4][RB][MT][64][4];  // partial accumulators of the four wavefronts
     __shared__ int red_sum[4][MT][16];     // per wavefront: sum_k a[t, k] over its k-tiles
 
@@ -608,29 +610,29 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 
     // A operand of this lane in token group g: token row 16g + lr, the 16 columns 64t + 16lg of each k-tile
     // (rows past m read as zero)
-    const bool a_vec = (p.k % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0);
+    const bool a_vec = (hot_k % 16 == 0) && ((reinterpret_cast<uintptr_t>(hot_a) & 15) == 0);
     bool row_ok[MT];
     const int8_t *arow[MT];
 #pragma unroll
     for (int g = 0; g < MT; ++g) {
-        row_ok[g] = 16 * g + lr < p.m;
-        arow[g] = p.a + (size_t)(row_ok[g] ? 16 * g + lr : 0) * p.k + lg * 16;
+        row_ok[g] = 16 * g + lr < hot_m;
+        arow[g] = hot_a + (size_t)(row_ok[g] ? 16 * g + lr : 0) * hot_k + lg * 16;
     }
     auto load_a = [&](int g, int kt, int t) -> v4i {
         if constexpr (FAST) {
-            const v4i v = *reinterpret_cast<const v4i *>(arow[g] + min(kt, p.kt_count - 1) * TILE_K + t * 64);
+            const v4i v = *reinterpret_cast<const v4i *>(arow[g] + min(kt, hot_kt_count - 1) * TILE_K + t * 64);
             return row_ok[g] ? v : (v4i){0, 0, 0, 0};
         }
         v4i v = (v4i){0, 0, 0, 0};
         const int col = kt * TILE_K + t * 64 + lg * 16;
-        if (row_ok[g] && col < p.k) {
+        if (row_ok[g] && col < hot_k) {
             const int8_t *src = arow[g] + kt * TILE_K + t * 64;
             if (a_vec) {
                 v = *reinterpret_cast<const v4i *>(src);
             } else {
                 int d[4] = {0, 0, 0, 0};
                 for (int j = 0; j < 16; ++j)
-                    if (col + j < p.k) d[j >> 2] |= (int)((uint32_t)(uint8_t)src[j] << (8 * (j & 3)));
+                    if (col + j < hot_k) d[j >> 2] |= (int)((uint32_t)(uint8_t)src[j] << (8 * (j & 3)));
                 v = (v4i){d[0], d[1], d[2], d[3]};
             }
         }
@@ -641,9 +643,9 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         for (int r = 0; r < RB; ++r) {
             const int rb = rb0 + r;
             if constexpr (FAST)  // results of row blocks past the end are never stored
-                w[r] = load_weight_slot(wbase + ((size_t)min(rb, rb_count - 1) * p.kt_count + min(kt, p.kt_count - 1)) * 64);
+                w[r] = load_weight_slot(wbase + ((size_t)min(rb, rb_count - 1) * hot_kt_count + min(kt, hot_kt_count - 1)) * 64);
             else
-                w[r] = rb < rb_count ? load_weight_slot(wbase + ((size_t)rb * p.kt_count + kt) * 64)
+                w[r] = rb < rb_count ? load_weight_slot(wbase + ((size_t)rb * hot_kt_count + kt) * 64)
                                      : make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
         }
     };
@@ -664,7 +666,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
         e_bias[f] = (mine && P.bias) ? P.bias[e_n] : 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int t = min(16 * fg + lg * 4 + i, p.m - 1);
+            const int t = min(16 * fg + lg * 4 + i, hot_m - 1);
             e_scale[f][i] = (mine && P.out) ? p.a_scale[t] : 1.0f;
             e_res[f][i] = (mine && P.residual) ? P.residual[(size_t)t * P.n + e_n] : 0.0f;
         }
@@ -690,7 +692,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
             const int kt = kt0 + 4 * u;
-            if (FAST || kt < p.kt_count) {
+            if (FAST || kt < hot_kt_count) {
                 load_w(kt, w[u]);
 #pragma unroll
                 for (int g = 0; g < MT; ++g)
@@ -702,7 +704,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
     auto compute_batch = [&](int kt0) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
-            if (kt0 + 4 * u >= p.kt_count) continue;
+            if (kt0 + 4 * u >= hot_kt_count) continue;
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
 #pragma unroll
@@ -733,10 +735,10 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
     if constexpr (ONE) {
         compute_batch(wave);
     } else
-    for (int kt0 = wave; kt0 < p.kt_count; kt0 += 4 * PF) {
+    for (int kt0 = wave; kt0 < hot_kt_count; kt0 += 4 * PF) {
         // two straight-line bodies, so that the wait before the MFMAs is for this batch only in both of them
         if constexpr (!ONE) {
-            if (kt0 + 4 * PF < p.kt_count) {  // uniform over the wavefront
+            if (kt0 + 4 * PF < hot_kt_count) {  // uniform over the wavefront
                 load_batch(kt0 + 4 * PF, wnxt, anxt);
                 compute_batch(kt0);
 #pragma unroll
@@ -777,7 +779,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int tl = lg * 4 + i, t = 16 * fg + tl;
-            if (n < P.n && t < p.m) {
+            if (n < P.n && t < hot_m) {
                 const int asum = red_sum[0][fg][tl] + red_sum[1][fg][tl] + red_sum[2][fg][tl] + red_sum[3][fg][tl];
                 const int total = sum[i] - asum;
                 const size_t o = (size_t)t * P.n + n;
@@ -923,15 +925,15 @@ int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const floa
         // more than one double-buffered batch per wavefront, but few enough k-tiles for one batch without the second buffer
         constexpr int PF2 = RB == 1 ? 4 : (RB == 2 ? 3 : 2), PF1 = RB == 1 ? 8 : (RB == 2 ? 4 : 3);
         if (fast && p.kt_count > 4 * PF2 && p.kt_count <= 4 * PF1) {
-            hipLaunchKernelGGL((gemv_mfma_kernel<RB, 1, true, true>), dim3((unsigned)end), dim3(256), 0, stream, p);
+            hipLaunchKernelGGL((gemv_mfma_kernel<RB, 1, true, true>), dim3((unsigned)end), dim3(256), 0, stream, p.a, p.k, p.m, p.kt_count, p);
             BITNET_HIP_CHECK_LAUNCH("gemv_mfma_kernel");
             return BITNET_HIP_OK;
         }
     }
     if (fast)
-        hipLaunchKernelGGL((gemv_mfma_kernel<RB, MT, true>), dim3((unsigned)end), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((gemv_mfma_kernel<RB, MT, true>), dim3((unsigned)end), dim3(256), 0, stream, p.a, p.k, p.m, p.kt_count, p);
     else
-        hipLaunchKernelGGL((gemv_mfma_kernel<RB, MT, false>), dim3((unsigned)end), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((gemv_mfma_kernel<RB, MT, false>), dim3((unsigned)end), dim3(256), 0, stream, p.a, p.k, p.m, p.kt_count, p);
     BITNET_HIP_CHECK_LAUNCH("gemv_mfma_kernel");
     return BITNET_HIP_OK;
 }

@@ -25,7 +25,7 @@ fn main() {
             .args(["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
                    "-fhip-fp32-correctly-rounded-divide-sqrt",
                    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                   "-mllvm", "-amdgpu-kernarg-preload-count=9", "-c"])
+                   "-mllvm", "-amdgpu-kernarg-preload-count=10", "-c"])
             .arg(csrc.join(k))
             .arg("-o")
             .arg(&obj)

@@ -51,5 +51,5 @@ def test_rust_build_script_compiles_the_same_sources_with_the_same_flags():
     for src in re.findall(r"csrc/([a-z0-9_]+\.hip)", makefile):
         assert f'"{src}"' in build_rs, src
     for flag in ("--offload-arch=gfx950", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-packed-fp32-ops",
-                 "-amdgpu-kernarg-preload-count=9"):
+                 "-amdgpu-kernarg-preload-count=10"):
         assert flag in build_rs and flag.lstrip("-") in makefile.replace("$(ARCH)", "gfx950")
