@@ -441,8 +441,36 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     __shared__ int tot[RBW][TILE_ROWS];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int chunks = hot_k >> 2, lds_words = p.kt_count * 64;
+    const int chunks = hot_k >> 2;
 
+    // Every load is unconditional (clamped indices, values discarded), in the order in which the data is needed.
+    // First what the preloaded arguments alone address: the input row and the RMSNorm weights.  The argument buffer is
+    // read only after these loads are on their way and after the wavefronts of the summation order have added up
+    // their squares, so that its latency hides behind theirs.
+    float4 v[NCHB], gm[NORM ? NCHB : 1];
+    constexpr int NSS = NORM ? 4 * NCHB : 1;  // chunks per virtual lane of the summation order
+#pragma unroll
+    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(hot, 0, min(tid + 1024 * i, chunks - 1));
+    if constexpr (NORM) {
+        float4 vs[NSS];
+        if (wave < 4) {  // thread tid < 256 is virtual lane tid: it fetches the lane's chunks itself (from L2)
+#pragma unroll
+            for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(hot, 0, min(tid + 256 * i, chunks - 1));
+        }
+#pragma unroll
+        for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(hot, min(tid + 1024 * i, chunks - 1), true);
+        if (wave < 4) {
+            float part = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NSS; ++i)
+                if (tid + 256 * i < chunks) part = sum_squares4(part, vs[i]);  // chunks past the end would add +0
+            part = wave_sum_f32(part);
+            if (lane == 0) red_f[0][wave] = part;
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // nothing below moves above: the first wait for the argument buffer comes here
+
+    const int lds_words = p.kt_count * 64;
     int pj = 0;
 #pragma unroll
     for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
@@ -451,49 +479,28 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     const int rb0 = ((int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0)) * RBW;  // rb_end counts groups of RBW row blocks
     const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
     const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + lane;
-
-    // every load is unconditional (clamped indices, values discarded), in the order in which the data is needed
-    float4 v[NCHB], gm[NORM ? NCHB : 1];
-    constexpr int NSS = NORM ? 4 * NCHB : 1;  // chunks per virtual lane of the summation order
-    float4 vs[NSS];
-    uint4 wt[RBW][NCHB];
-#pragma unroll
-    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(hot, 0, min(tid + 1024 * i, chunks - 1));
-    if constexpr (NORM) {
-        if (wave < 4) {  // thread tid < 256 is virtual lane tid: it fetches the lane's chunks itself (from L2)
-#pragma unroll
-            for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(hot, 0, min(tid + 256 * i, chunks - 1));
-        }
-    }
-    const int e_n = min((rb0 + (tid >> 4)) * TILE_ROWS + (tid & 15), P.n - 1);  // meaningful for tid < 16 * RBW
-    const float e_ws = P.out ? *P.w_scale : 0.0f;
-    const float e_bias = P.bias ? P.bias[e_n] : 0.0f;
-    const float e_res = P.residual ? P.residual[e_n] : 0.0f;
-    if constexpr (NORM) {
-#pragma unroll
-        for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(hot, min(tid + 1024 * i, chunks - 1), true);
-    }
     // k-tile kt holds chunks 64*kt .. 64*kt + 63: exactly what wavefront kt % 16 quantises, so a wavefront multiplies
     // the tiles of its own chunks (tiles and row blocks past the end repeat the last one; their results are not added)
+    uint4 wt[RBW][NCHB];
 #pragma unroll
     for (int r = 0; r < RBW; ++r)
 #pragma unroll
         for (int i = 0; i < NCHB; ++i)
             wt[r][i] = load_weight_slot(tiles + ((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 16 * i, p.kt_count - 1)) * 64);
+    // epilogue operands: absent ones read the input row instead (always there) and are not used; the weight scale goes
+    // through a per-lane address so that it is a vector load, which nothing waits for before the epilogue
+    const int e_n = min((rb0 + (tid >> 4)) * TILE_ROWS + (tid & 15), P.n - 1);  // meaningful for tid < 16 * RBW
+    int lane_zero = 0;
+    asm volatile("" : "+v"(lane_zero));
+    const float e_ws = (P.out ? P.w_scale : hot_x)[lane_zero];
+    const float e_bias = *(P.bias ? P.bias + e_n : hot_x);
+    const float e_res = *(P.residual ? P.residual + e_n : hot_x);
     if (tid < RBW * TILE_ROWS) tot[tid >> 4][tid & 15] = 0;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i)
         if (tid + 1024 * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     if constexpr (NORM) {
-        if (wave < 4) {  // wavefronts 0..3: thread tid is virtual lane tid
-            float part = 0.0f;
-#pragma unroll
-            for (int i = 0; i < NSS; ++i)
-                if (tid + 256 * i < chunks) part = sum_squares4(part, vs[i]);  // chunks past the end would add +0
-            part = wave_sum_f32(part);
-            if (lane == 0) red_f[0][wave] = part;
-        }
         lds_barrier();
         const float ss = f32_add(f32_add(f32_add(red_f[0][0], red_f[0][1]), red_f[0][2]), red_f[0][3]);
         const RowDivisor rdiv = make_row_divisor(rms_from_ss(ss, p.k, p.src.eps));
