@@ -238,14 +238,15 @@ __global__ __launch_bounds__(1024) void act_quant_block16_kernel(const float *ho
     const size_t row = blockIdx.x;
     const int k = src.k, chunks = k >> 2;
     const bool norm = src.gamma != nullptr;
-    const bool chain = norm && src.sum_order != BITNET_HIP_SUM_SEQUENTIAL && wave < 4;
     constexpr int NSS = 4 * NCHB;
 
-    // all loads up front, unconditional (clamped indices, values discarded)
+    // all loads up front, unconditional (clamped indices, values discarded), addressed by the preloaded arguments alone:
+    // the argument buffer is read only once they are on their way (wavefronts 0..3 fetch their lanes' chunks whatever
+    // the summation order turns out to be)
     float4 v[NCHB], gm[NCHB], vs[NSS];
 #pragma unroll
     for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(src, row, min(tid + 1024 * i, chunks - 1));
-    if (chain) {
+    if (norm && wave < 4) {
 #pragma unroll
         for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(src, row, min(tid + 256 * i, chunks - 1));
     }
@@ -253,6 +254,8 @@ __global__ __launch_bounds__(1024) void act_quant_block16_kernel(const float *ho
 #pragma unroll
         for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(src, min(tid + 1024 * i, chunks - 1), true);
     }
+    __builtin_amdgcn_sched_barrier(0);  // nothing below moves above: the first wait for the argument buffer comes here
+    const bool chain = norm && src.sum_order != BITNET_HIP_SUM_SEQUENTIAL && wave < 4;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i)
         if (tid + 1024 * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);

@@ -605,16 +605,6 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const int8_t *hot_a, int
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 15, lg = lane >> 4;
 
-    int pj = 0;
-#pragma unroll
-    for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
-        if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
-    const GemvProjDev &P = p.proj[pj];
-    const int grp = (int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0);
-    const int rb0 = grp * RB;
-    const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
-    const uint4 *wbase = reinterpret_cast<const uint4 *>(P.w) + lane;
-
     // A operand of this lane in token group g: token row 16g + lr, the 16 columns 64t + 16lg of each k-tile
     // (rows past m read as zero)
     const bool a_vec = (hot_k % 16 == 0) && ((reinterpret_cast<uintptr_t>(hot_a) & 15) == 0);
@@ -645,6 +635,36 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const int8_t *hot_a, int
         }
         return v;
     };
+    static_assert(!ONE || MT == 1, "single batch: one token group");
+    constexpr int PF = ONE ? (RB == 1 ? 8 : (RB == 2 ? 4 : 3))
+                           : (RB * MT == 1 ? 4 : (RB * MT == 2 ? 3 : (MT <= 2 ? 2 : 1)));  // bounded by the register file
+    // All loads of a batch of PF k-tiles are issued before the first MFMA of the batch, and the next
+    // batch is requested while the current one is computed: the weight stream is what the kernel waits for.
+    uint4 wcur[PF][RB], wnxt[ONE ? 1 : PF][RB];
+    v4i acur[PF][MT][4], anxt[ONE ? 1 : PF][MT][4];
+    // The first batch: the activations are addressed by the preloaded arguments alone, so with FAST they are requested
+    // before anything reads the argument buffer (the weights' address comes from there).
+    if constexpr (FAST) {
+#pragma unroll
+        for (int u = 0; u < PF; ++u)
+#pragma unroll
+            for (int g = 0; g < MT; ++g)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acur[u][g][t] = load_a(g, wave + 4 * u, t);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // nothing below moves above: the first wait for the argument buffer comes here
+
+    int pj = 0;
+#pragma unroll
+    for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
+        if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
+    const GemvProjDev &P = p.proj[pj];
+    const int grp = (int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0);
+    const int rb0 = grp * RB;
+    const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
+    const uint4 *wbase = reinterpret_cast<const uint4 *>(P.w) + lane;
+
+
     auto load_w = [&](int kt, uint4 (&w)[RB]) {
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
@@ -657,28 +677,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const int8_t *hot_a, int
         }
     };
 
-    // scales the epilogue will need (result register i of a lane belongs to token 16g + 4*(lane/16) + i): requested
-    // now, so that their latency is not paid at the end
-    // The RB * MT fragments (row block, token group) are finished by the wavefronts in turn: fragment
-    // q = wave + 4 * f is (row block q / MT, token group q % MT).  Scales, bias and residuals are requested now
-    // (clamped indices; unused values are discarded).
     constexpr int NFRAG = RB * MT, FPW = (NFRAG + 3) / 4;  // fragments, fragments per wavefront
-    const float ws = P.out ? *P.w_scale : 0.0f;
-    float e_bias[FPW], e_scale[FPW][4], e_res[FPW][4];
-#pragma unroll
-    for (int f = 0; f < FPW; ++f) {
-        const int q = min(wave + 4 * f, NFRAG - 1), fr = q / MT, fg = q % MT;
-        const bool mine = wave + 4 * f < NFRAG;
-        const int e_n = min((rb0 + fr) * TILE_ROWS + lr, P.n - 1);
-        e_bias[f] = (mine && P.bias) ? P.bias[e_n] : 0.0f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int t = min(16 * fg + lg * 4 + i, hot_m - 1);
-            e_scale[f][i] = (mine && P.out) ? p.a_scale[t] : 1.0f;
-            e_res[f][i] = (mine && P.residual) ? P.residual[(size_t)t * P.n + e_n] : 0.0f;
-        }
-    }
-
     v4i acc[RB][MT];
     int rowsum[MT];
 #pragma unroll
@@ -688,13 +687,6 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const int8_t *hot_a, int
         for (int r = 0; r < RB; ++r) acc[r][g] = (v4i){0, 0, 0, 0};
     }
 
-    static_assert(!ONE || MT == 1, "single batch: one token group");
-    constexpr int PF = ONE ? (RB == 1 ? 8 : (RB == 2 ? 4 : 3))
-                           : (RB * MT == 1 ? 4 : (RB * MT == 2 ? 3 : (MT <= 2 ? 2 : 1)));  // bounded by the register file
-    // All loads of a batch of PF k-tiles are issued before the first MFMA of the batch, and the next
-    // batch is requested while the current one is computed: the weight stream is what the kernel waits for.
-    uint4 wcur[PF][RB], wnxt[ONE ? 1 : PF][RB];
-    v4i acur[PF][MT][4], anxt[ONE ? 1 : PF][MT][4];
     auto load_batch = [&](int kt0, uint4 (&w)[PF][RB], v4i (&a)[PF][MT][4]) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
@@ -708,6 +700,14 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const int8_t *hot_a, int
             }
         }
     };
+    if constexpr (FAST) {  // the activations of the first batch are on their way already
+#pragma unroll
+        for (int u = 0; u < PF; ++u) load_w(wave + 4 * u, wcur[u]);
+    } else {
+        load_batch(wave, wcur, acur);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
     auto compute_batch = [&](int kt0) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
@@ -738,7 +738,30 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const int8_t *hot_a, int
             }
         }
     };
-    load_batch(wave, wcur, acur);
+    // The RB * MT fragments (row block, token group) are finished by the wavefronts in turn: fragment
+    // q = wave + 4 * f is (row block q / MT, token group q % MT); result register i of a lane belongs to token
+    // 16g + 4*(lane/16) + i.  Scales, bias and residuals are requested now, behind the first batch of the main loads, so
+    // that their latency is not paid at the end.  Absent operands read the weight tiles instead (always there; the
+    // values are not used), which keeps this part free of branches, and the weight scale goes through a per-lane address:
+    // a vector load, which nothing waits for before the epilogue.
+    const float *absent = reinterpret_cast<const float *>(P.w);
+    int lane_zero = 0;
+    asm volatile("" : "+v"(lane_zero));
+    const float ws = (P.out ? P.w_scale : absent)[lane_zero];
+    float e_bias[FPW], e_scale[FPW][4], e_res[FPW][4];
+#pragma unroll
+    for (int f = 0; f < FPW; ++f) {
+        const int q = min(wave + 4 * f, NFRAG - 1), fr = q / MT, fg = q % MT;
+        const int e_n = min((rb0 + fr) * TILE_ROWS + lr, P.n - 1);
+        e_bias[f] = *(P.bias ? P.bias + e_n : absent);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = min(16 * fg + lg * 4 + i, hot_m - 1);
+            e_scale[f][i] = *(P.out ? p.a_scale + t : absent);
+            e_res[f][i] = *(P.residual ? P.residual + ((size_t)t * P.n + e_n) : absent);
+        }
+    }
+
     if constexpr (ONE) {
         compute_batch(wave);
     } else
