@@ -480,13 +480,20 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
     const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + lane;
     // k-tile kt holds chunks 64*kt .. 64*kt + 63: exactly what wavefront kt % 16 quantises, so a wavefront multiplies
-    // the tiles of its own chunks (tiles and row blocks past the end repeat the last one; their results are not added)
+    // the tiles of its own chunks (tiles and row blocks past the end repeat the last one; their results are not added).
+    // The tiles are requested right after the first workgroup barrier, not here: the chain of reductions that starts
+    // from the input row is what the kernel's duration hangs on, and a weight stream requested before the row has
+    // been reduced once holds that chain up (in the memory system and in the L1 that every wavefront's loads share).
     uint4 wt[RBW][NCHB];
+    auto request_weight_tiles = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int r = 0; r < RBW; ++r)
+        for (int r = 0; r < RBW; ++r)
 #pragma unroll
-        for (int i = 0; i < NCHB; ++i)
-            wt[r][i] = load_weight_slot(tiles + ((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 16 * i, p.kt_count - 1)) * 64);
+            for (int i = 0; i < NCHB; ++i)
+                wt[r][i] = load_weight_slot(tiles + ((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 16 * i, p.kt_count - 1)) * 64);
+        __builtin_amdgcn_sched_barrier(0);
+    };
     // epilogue operands: absent ones read the input row instead (always there) and are not used; the weight scale goes
     // through a per-lane address so that it is a vector load, which nothing waits for before the epilogue
     const int e_n = min((rb0 + (tid >> 4)) * TILE_ROWS + (tid & 15), P.n - 1);  // meaningful for tid < 16 * RBW
@@ -502,6 +509,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
 
     if constexpr (NORM) {
         lds_barrier();
+        request_weight_tiles();
         const float ss = f32_add(f32_add(f32_add(red_f[0][0], red_f[0][1]), red_f[0][2]), red_f[0][3]);
         const RowDivisor rdiv = make_row_divisor(rms_from_ss(ss, p.k, p.src.eps));
 #pragma unroll
@@ -514,6 +522,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     amax = wave_max_f32(amax);
     if (lane == 0) red_f[1][wave] = amax;
     lds_barrier();
+    if constexpr (!NORM) request_weight_tiles();
     amax = red_f[1][0];
 #pragma unroll
     for (int w = 1; w < 16; ++w) amax = fmaxf(amax, red_f[1][w]);
