@@ -546,17 +546,39 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
 
-    const int kq = lane >> 4;  // lane group: columns 64t + 16kq .. +15 of each tile, t = 0..3
+    // Dot products on the matrix unit: the tile's 16 rows are the B operand of v_mfma_i32_16x16x64_i8 (lane l: row l mod 16,
+    // columns 64t + 16kq .. +15 for dword t, kq = l / 16), the activations are row 0 of the A operand (lanes 0, 16, 32, 48
+    // hold the four column groups; the other 15 rows are zero), so result register 0 of lanes 0..15 is the sum over the
+    // 64 columns of step t for rows 0..15.  Against dot4 this leaves only the unpacking of the 2-bit codes on the VALU.
+    typedef int v4i_t __attribute__((ext_vector_type(4)));
+    const int kq = lane >> 4;
+    const bool row0 = (lane & 15) == 0;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i) {
         const int kt = wave + 16 * i;
         if (kt < p.kt_count) {  // uniform over the wavefront
+            v4i_t acc[RBW];
 #pragma unroll
-            for (int r = 0; r < RBW; ++r) {
-                int acc = dot64(wt[r][i], lds_a + kt * 16 + kq, 0);
-                acc = sum_over_lane_groups(acc);  // lanes l, l+16, l+32, l+48 hold the four column groups of row l mod 16
-                if (lane < TILE_ROWS) atomicAdd(&tot[r][lane], acc);  // int32: any order gives the same sum
+            for (int r = 0; r < RBW; ++r) acc[r] = (v4i_t){0, 0, 0, 0};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                v4i_t af = (v4i_t){0, 0, 0, 0};
+                if (row0) af = *reinterpret_cast<const v4i_t *>(lds_a + kt * 16 + 4 * t + kq);
+#pragma unroll
+                for (int r = 0; r < RBW; ++r) {
+                    const uint4 w4 = wt[r][i];
+                    const uint32_t wd = t == 0 ? w4.x : (t == 1 ? w4.y : (t == 2 ? w4.z : w4.w));
+                    v4i_t bf;
+                    bf[0] = (int)(wd & 0x03030303u);
+                    bf[1] = (int)((wd >> 2) & 0x03030303u);
+                    bf[2] = (int)((wd >> 4) & 0x03030303u);
+                    bf[3] = (int)((wd >> 6) & 0x03030303u);
+                    acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf, acc[r], 0, 0, 0);
+                }
             }
+#pragma unroll
+            for (int r = 0; r < RBW; ++r)
+                if (lane < TILE_ROWS) atomicAdd(&tot[r][lane], acc[r][0]);  // int32: any order gives the same sum
         }
     }
     lds_barrier();
