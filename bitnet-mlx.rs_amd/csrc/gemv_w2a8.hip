@@ -856,6 +856,153 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(const int8_t *hot_a, int
     }
 }
 
+// gemv_mfma_kernel for up to 16 tokens with the activations staged through LDS.  There every wavefront gathers its A
+// fragments straight from memory: 16 bytes per lane from 16 different rows, four loads per k-tile, and the address
+// unit of the compute unit spends more time on those gathers than the weight stream needs.  Here the workgroup copies
+// the m rows into LDS once with dense loads (thread t takes the 16-byte chunks t, t + 256, .. of every row) and the
+// fragments are LDS reads.  Rows are k + 16 bytes apart in LDS.  KCLASS 0: k <= 3072 (one chunk column per thread,
+// three k-tiles per wavefront), KCLASS 1: k <= 8192 and m <= 8 (two chunk columns, eight k-tiles).  k % 256 == 0, the
+// activations 16-byte aligned, m * (k + 16) bytes of dynamic LDS.
+template <int RB, int KCLASS>
+__global__ __launch_bounds__(256) void gemv_mfma_lds_kernel(const int8_t *hot_a, int hot_k, int hot_m, int hot_kt_count, GemvMfmaParams p)
+{
+    constexpr int JN = KCLASS == 0 ? 1 : 2, NT = KCLASS == 0 ? 3 : 8;
+    extern __shared__ uint4 lds_act[];        // [m][k / 16 + 1] chunks of 16 int8
+    __shared__ int red[4][RB][64][4];         // partial accumulators of the four wavefronts
+    __shared__ int red_sum[4][16];            // per wavefront: sum_k a[t, k] over its k-tiles
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lr = lane & 15, lg = lane >> 4;
+    const int cpr = hot_k >> 4, stride = cpr + 1;  // chunks per row in memory and in LDS
+
+    // the copy's loads first: they are addressed by the preloaded arguments alone (unconditional: rows past m repeat
+    // the last row, chunks past the row its last chunk; those are not stored)
+    v4i stage[16];
+    const v4i *a_chunks = reinterpret_cast<const v4i *>(hot_a);
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        const int r = min(s / JN, hot_m - 1), cc = min(tid + 256 * (s % JN), cpr - 1);
+        stage[s] = a_chunks[(size_t)r * cpr + cc];
+    }
+    __builtin_amdgcn_sched_barrier(0);  // nothing below moves above: the first wait for the argument buffer comes here
+
+    int pj = 0;
+#pragma unroll
+    for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
+        if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
+    const GemvProjDev &P = p.proj[pj];
+    const int rb0 = ((int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0)) * RB;
+    const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
+    const uint4 *wbase = reinterpret_cast<const uint4 *>(P.w) + lane;
+    __builtin_amdgcn_sched_barrier(0);
+    // The copy's stores, then everyone may read the rows.  The weight stream is requested only now: megabytes from all
+    // workgroups at once, behind which the activations (and the argument buffers of workgroups that start a little
+    // later) would queue in the memory system; this way they arrive about as early as they can, and the weights about
+    // when they would have anyway.
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        const int r = s / JN, cc = tid + 256 * (s % JN);
+        if (r < hot_m && cc < cpr) reinterpret_cast<v4i *>(lds_act)[r * stride + cc] = stage[s];
+    }
+    lds_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // all k-tiles of this wavefront (kt = wave + 4u) in one batch; tiles and row blocks past the end repeat the last one
+    uint4 w[NT][RB];
+#pragma unroll
+    for (int u = 0; u < NT; ++u)
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+            w[u][r] = load_weight_slot(wbase + ((size_t)min(rb0 + r, rb_count - 1) * hot_kt_count + min(wave + 4 * u, hot_kt_count - 1)) * 64);
+
+    // Row block q = wave + 4f of the workgroup is finished by this wavefront; scales, bias and residuals are requested now
+    // (absent operands read the weight tiles instead, the values are not used; the weight scale goes through a per-lane
+    // address: a vector load, which nothing waits for before the epilogue).
+    constexpr int FPW = (RB + 3) / 4;
+    const float *absent = reinterpret_cast<const float *>(P.w);
+    int lane_zero = 0;
+    asm volatile("" : "+v"(lane_zero));
+    const float ws = (P.out ? P.w_scale : absent)[lane_zero];
+    float e_bias[FPW], e_scale[FPW][4], e_res[FPW][4];
+#pragma unroll
+    for (int f = 0; f < FPW; ++f) {
+        const int fr = min(wave + 4 * f, RB - 1);
+        const int e_n = min((rb0 + fr) * TILE_ROWS + lr, P.n - 1);
+        e_bias[f] = *(P.bias ? P.bias + e_n : absent);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = min(lg * 4 + i, hot_m - 1);
+            e_scale[f][i] = *(P.out ? p.a_scale + t : absent);
+            e_res[f][i] = *(P.residual ? P.residual + ((size_t)t * P.n + e_n) : absent);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    v4i acc[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) acc[r] = (v4i){0, 0, 0, 0};
+    int rowsum = 0;
+    const bool row_ok = lr < hot_m;
+    const uint4 *arow = lds_act + (row_ok ? lr : 0) * stride + lg;  // A operand: token row lr, columns 64t + 16lg .. +15 of a k-tile
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+        const int kt = wave + 4 * u;
+        if (kt < hot_kt_count) {  // uniform over the wavefront
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                v4i af = (v4i){0, 0, 0, 0};
+                if (row_ok) af = *reinterpret_cast<const v4i *>(arow + kt * 16 + t * 4);
+                rowsum = __builtin_amdgcn_sdot4(af[0], 0x01010101, rowsum, false);
+                rowsum = __builtin_amdgcn_sdot4(af[1], 0x01010101, rowsum, false);
+                rowsum = __builtin_amdgcn_sdot4(af[2], 0x01010101, rowsum, false);
+                rowsum = __builtin_amdgcn_sdot4(af[3], 0x01010101, rowsum, false);
+#pragma unroll
+                for (int r = 0; r < RB; ++r) {
+                    const uint4 w4 = w[u][r];
+                    const uint32_t wd = t == 0 ? w4.x : (t == 1 ? w4.y : (t == 2 ? w4.z : w4.w));
+                    v4i bf;
+                    bf[0] = (int)(wd & 0x03030303u);
+                    bf[1] = (int)((wd >> 2) & 0x03030303u);
+                    bf[2] = (int)((wd >> 4) & 0x03030303u);
+                    bf[3] = (int)((wd >> 6) & 0x03030303u);
+                    acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf, acc[r], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // sum_k a[row, k] over this wavefront's tiles: lanes lr, lr+16, lr+32, lr+48 hold the four column groups
+    rowsum = sum_over_lane_groups(rowsum);
+    if (lane < 16) red_sum[wave][lane] = rowsum;
+#pragma unroll
+    for (int r = 0; r < RB; ++r) *reinterpret_cast<v4i *>(&red[wave][r][lane][0]) = acc[r];
+    lds_barrier();
+#pragma unroll
+    for (int f = 0; f < FPW; ++f) {
+        if (wave + 4 * f >= RB) break;  // uniform over the wavefront
+        const int fr = wave + 4 * f;
+        const int n = (rb0 + fr) * TILE_ROWS + lr;  // result register i of lane l is C[4*(l/16) + i][l mod 16]
+        const v4i s0 = *reinterpret_cast<const v4i *>(&red[0][fr][lane][0]), s1 = *reinterpret_cast<const v4i *>(&red[1][fr][lane][0]);
+        const v4i s2 = *reinterpret_cast<const v4i *>(&red[2][fr][lane][0]), s3 = *reinterpret_cast<const v4i *>(&red[3][fr][lane][0]);
+        const v4i sum = s0 + s1 + s2 + s3;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = lg * 4 + i;
+            if (n < P.n && t < hot_m) {
+                const int asum = red_sum[0][t] + red_sum[1][t] + red_sum[2][t] + red_sum[3][t];
+                const int total = sum[i] - asum;
+                const size_t o = (size_t)t * P.n + n;
+                if (P.acc) P.acc[o] = total;
+                if (P.out) {
+                    float v = f32_div(f32_mul((float)total, ws), e_scale[f][i]);
+                    if (P.bias) v = f32_add(v, e_bias[f]);
+                    if (P.residual) v = f32_add(v, e_res[f][i]);
+                    P.out[o] = v;
+                }
+            }
+        }
+    }
+}
+
 // The reference's flat row-major packing, any n and k (rows need not start on a byte boundary).
 // One wavefront per output row; lane l takes columns 4l..4l+3, 4l+256.., gathers their codes one by one.
 __global__ __launch_bounds__(256) void gemv_rowmajor_kernel(const uint8_t *packed, const int8_t *a,
@@ -983,6 +1130,17 @@ int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const floa
     if (end == 0) return BITNET_HIP_OK;
     const bool fast = k % TILE_K == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0;
     if constexpr (MT == 1) {
+        // 5 to 16 tokens whose rows fit LDS: the variant that stages the activations there (with fewer rows the gathers
+        // of the other variant are cheap enough, and it is measurably ahead)
+        const size_t lds = m * (k + 16);
+        if (fast && m >= 5 && lds + 4096 * RB + 512 <= 64 * 1024 && (k <= 3072 || (k <= 8192 && m <= 8))) {  // + the kernel's static LDS
+            if (k <= 3072)
+                hipLaunchKernelGGL((gemv_mfma_lds_kernel<RB, 0>), dim3((unsigned)end), dim3(256), lds, stream, p.a, p.k, p.m, p.kt_count, p);
+            else
+                hipLaunchKernelGGL((gemv_mfma_lds_kernel<RB, 1>), dim3((unsigned)end), dim3(256), lds, stream, p.a, p.k, p.m, p.kt_count, p);
+            BITNET_HIP_CHECK_LAUNCH("gemv_mfma_lds_kernel");
+            return BITNET_HIP_OK;
+        }
         // more than one double-buffered batch per wavefront, but few enough k-tiles for one batch without the second buffer
         constexpr int PF2 = RB == 1 ? 4 : (RB == 2 ? 3 : 2), PF1 = RB == 1 ? 8 : (RB == 2 ? 4 : 3);
         if (fast && p.kt_count > 4 * PF2 && p.kt_count <= 4 * PF1) {

@@ -274,6 +274,27 @@ def test_decode_gemv_ragged_shapes(m, n, k):
     assert np.array_equal(host(out), orc.epilogue(acc_ref, ws, a_scale, bias, res))
 
 
+@pytest.mark.parametrize("m,n,k", [(5, 40, 256), (16, 33, 3072), (8, 100, 3328), (8, 17, 8192), (5, 6500, 512),
+                                   (16, 13000, 256), (7, 2560, 6912), (16, 6912, 2560), (9, 48, 3328), (4, 48, 2560)])
+def test_decode_gemv_lds_staged_activations(m, n, k):
+    """5..16 tokens with k a multiple of 256 whose rows fit LDS take the MFMA GEMV that copies the activations into
+    LDS first: k <= 3072 (one chunk column per thread) or k <= 8192 with at most 8 tokens (two); n selects 1, 2 or 4
+    row blocks per workgroup (400 / 800 row blocks), ragged n the partial last block.  The last two cases fall just
+    outside (9 tokens at k > 3072, 4 tokens) and take the gathering variant."""
+    rng = np.random.default_rng(m + 10 * n + 100 * k)
+    packed, ws, a, a_scale = make_problem(rng, m, n, k, full_range=True)
+    tiled = bh.retile_weights(dev(packed), n, k)
+    bias = rng.standard_normal(n, dtype=f32)
+    res = rng.standard_normal((m, n), dtype=f32)
+    acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale), dev(bias), dev(res))
+    acc_ref = orc.gemm_w2a8(packed, a, n)
+    assert np.array_equal(host(acc), acc_ref)
+    assert np.array_equal(host(out), orc.epilogue(acc_ref, ws, a_scale, bias, res))
+    acc2, out2 = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale))
+    assert np.array_equal(host(acc2), acc_ref)
+    assert np.array_equal(host(out2), orc.epilogue(acc_ref, ws, a_scale))
+
+
 def test_decode_gemv_extremes_and_identities():
     k, n = 6912, 32
     tiled_neg = bh.retile_weights(dev(orc.pack_2bit(-np.ones((n, k), np.int8))), n, k)
