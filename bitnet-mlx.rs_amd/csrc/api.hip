@@ -110,7 +110,7 @@ int run_projections(bitnet_hip_bitlinear *const *layers, int count, const float 
                        out[j], acc ? acc[j] : nullptr, bl->out_features};
         return pj;
     };
-    if (gemv_fused_supported(x, x2, ldx, m, k, input_mode, head_dim, gamma)) {
+    if (gemv_fused_supported(x, x2, ldx, m, k, input_mode, head_dim, gamma, sum_order)) {
         for (int j0 = 0; j0 < count; j0 += GEMV_MAX_PROJ) {
             GemvProj pjs[GEMV_MAX_PROJ];
             const int nj = count - j0 < GEMV_MAX_PROJ ? count - j0 : GEMV_MAX_PROJ;
@@ -614,7 +614,7 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
 
     hipStream_t s = as_stream(stream);
     const bool debug = dbg_q || dbg_a_scale || dbg_acc;
-    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma);
+    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma, sum_order);
     void *ws = workspace;
     bool own_ws = false;
     QuantScratch sc = {dbg_q, dbg_a_scale, nullptr};
@@ -665,7 +665,7 @@ int bitnet_hip_bitlinear_forward_multi(bitnet_hip_bitlinear *const *layers, size
     }
     const size_t in = layers[0]->in_features;
     hipStream_t s = as_stream(stream);
-    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma);
+    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma, sum_order);
     void *ws = workspace;
     bool own_ws = false;
     QuantScratch sc = {nullptr, nullptr, nullptr};

@@ -42,6 +42,7 @@ namespace bitnet {
 namespace {
 
 constexpr int MODE_PREQUANT = -1;
+constexpr int GEMV_FUSED_MAX_ROWS = 3;  // tokens per fused quantiser + GEMV launch
 constexpr int FUSED_NCH = 7;  // 16-byte f32 chunks per thread kept in registers: K <= 7168
 
 struct GemvProjDev {
@@ -427,14 +428,19 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
 
 template <int MODE, bool NORM, int NCHB, int RBW>
 __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, const float *hot_x2, const float *hot_gamma, int hot_k, int hot_head_dim,
-                                                           int hot_gqa_group, GemvParams p)
+                                                           int hot_gqa_group, int hot_ldx, GemvParams p)
 {
-    // The leading scalar arguments repeat what the first loads need (input row, RMSNorm weights, k): the file is
+    // A launch has one to three tokens (input rows), each with its own workgroups.  Workgroup (x, y) of the grid works on
+    // token x / 8 and on group 8y + x % 8 of row blocks: the workgroups of one group are neighbours in dispatch order and,
+    // workgroups going to the XCDs in turn, run on the same XCD, so its L2 fetches their weight tiles once.
+    // The leading scalar arguments repeat what the first loads need (input rows, RMSNorm weights, k): the file is
     // compiled with kernel-argument preloading, so they arrive in registers with the wavefront instead of through a
     // load from the argument buffer that the first address computation would have to wait for.
     RowSource hot;
-    hot.x = hot_x; hot.x2 = hot_x2; hot.gamma = hot_gamma; hot.ldx = 0; hot.k = hot_k; hot.head_dim = hot_head_dim;
-    hot.gqa_group = hot_gqa_group; hot.sum_order = BITNET_HIP_SUM_BLOCK256; hot.eps = 0.0f;  // row 0 only: ldx unused
+    hot.x = hot_x; hot.x2 = hot_x2; hot.gamma = hot_gamma; hot.ldx = (size_t)hot_ldx; hot.k = hot_k; hot.head_dim = hot_head_dim;
+    hot.gqa_group = hot_gqa_group; hot.sum_order = BITNET_HIP_SUM_BLOCK256; hot.eps = 0.0f;
+    const size_t tok = blockIdx.x >> 3;
+    const int group = (int)blockIdx.y * 8 + (int)(blockIdx.x & 7);  // may lie past the last group: such workgroups leave below
     extern __shared__ uint4 lds_a[];  // int8 activations, zero past K
     __shared__ float red_f[2][16];
     __shared__ int red_i[16];
@@ -450,12 +456,12 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     float4 v[NCHB], gm[NORM ? NCHB : 1];
     constexpr int NSS = NORM ? 4 * NCHB : 1;  // chunks per virtual lane of the summation order
 #pragma unroll
-    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(hot, 0, min(tid + 1024 * i, chunks - 1));
+    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(hot, tok, min(tid + 1024 * i, chunks - 1));
     if constexpr (NORM) {
         float4 vs[NSS];
         if (wave < 4) {  // thread tid < 256 is virtual lane tid: it fetches the lane's chunks itself (from L2)
 #pragma unroll
-            for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(hot, 0, min(tid + 256 * i, chunks - 1));
+            for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(hot, tok, min(tid + 256 * i, chunks - 1));
         }
 #pragma unroll
         for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(hot, min(tid + 1024 * i, chunks - 1), true);
@@ -474,9 +480,9 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     int pj = 0;
 #pragma unroll
     for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
-        if (j + 1 < p.nproj && (int)blockIdx.x >= p.proj[j].rb_end) pj = j + 1;
+        if (j + 1 < p.nproj && group >= p.proj[j].rb_end) pj = j + 1;
     const GemvProjDev &P = p.proj[pj];
-    const int rb0 = ((int)blockIdx.x - (pj ? p.proj[pj - 1].rb_end : 0)) * RBW;  // rb_end counts groups of RBW row blocks
+    const int rb0 = (group - (pj ? p.proj[pj - 1].rb_end : 0)) * RBW;  // rb_end counts groups of RBW row blocks
     const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
     const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + lane;
     // k-tile kt holds chunks 64*kt .. 64*kt + 63: exactly what wavefront kt % 16 quantises, so a wavefront multiplies
@@ -501,7 +507,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     asm volatile("" : "+v"(lane_zero));
     const float e_ws = (P.out ? P.w_scale : hot_x)[lane_zero];
     const float e_bias = *(P.bias ? P.bias + e_n : hot_x);
-    const float e_res = *(P.residual ? P.residual + e_n : hot_x);
+    const float e_res = *(P.residual ? P.residual + (tok * (size_t)P.n + e_n) : hot_x);
     if (tid < RBW * TILE_ROWS) tot[tid >> 4][tid & 15] = 0;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i)
@@ -535,7 +541,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
         if (c < chunks) {
             const uint32_t packed = quant4_packed(v[i], scale, &isum);
             lds_w[c] = packed;
-            if (p.q_out && blockIdx.x == 0) reinterpret_cast<uint32_t *>(p.q_out)[c] = packed;
+            if (p.q_out && group == 0) reinterpret_cast<uint32_t *>(p.q_out + tok * (size_t)hot_k)[c] = packed;
         } else if (c < lds_words) {
             lds_w[c] = 0;
         }
@@ -589,19 +595,19 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
         int asum = 0;
 #pragma unroll
         for (int w = 0; w < 16; ++w) asum += red_i[w];
-        if (blockIdx.x == 0 && tid == 0) {
-            if (p.a_scale_out) p.a_scale_out[0] = scale;
-            if (p.a_sum_out) p.a_sum_out[0] = asum;
+        if (group == 0 && tid == 0) {
+            if (p.a_scale_out) p.a_scale_out[tok] = scale;
+            if (p.a_sum_out) p.a_sum_out[tok] = asum;
         }
         if (n < P.n) {
             const int total = tot[r][row] - asum;
-            if (P.acc) P.acc[n] = total;
+            if (P.acc) P.acc[tok * (size_t)P.n + n] = total;
             if (P.out) {
                 float y = f32_mul((float)total, e_ws);
                 y = f32_div(y, scale);
                 if (P.bias) y = f32_add(y, e_bias);
                 if (P.residual) y = f32_add(y, e_res);
-                P.out[n] = y;
+                P.out[tok * (size_t)P.n + n] = y;
             }
         }
     }
@@ -1079,8 +1085,8 @@ int launch_fused16_mode(const GemvParams &p, hipStream_t stream)
 {
     const bool norm = p.src.gamma != nullptr, one = (p.k >> 2) <= 1024;
     const size_t lds = (size_t)p.kt_count * 16 * sizeof(uint4);
-    const dim3 grid((unsigned)p.proj[p.nproj - 1].rb_end);
-#define BITNET_HOT_ARGS p.src.x, p.src.x2, p.src.gamma, p.src.k, p.src.head_dim, p.src.gqa_group
+    const dim3 grid(8u * (unsigned)p.m, ((unsigned)p.proj[p.nproj - 1].rb_end + 7u) / 8u);
+#define BITNET_HOT_ARGS p.src.x, p.src.x2, p.src.gamma, p.src.k, p.src.head_dim, p.src.gqa_group, (int)p.src.ldx
     if (norm && one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 1, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
     else if (norm) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 2, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
     else if (one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, 1, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
@@ -1212,10 +1218,14 @@ int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const f
 }
 
 bool gemv_fused_supported(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
-                          size_t head_dim, const float *gamma)
+                          size_t head_dim, const float *gamma, int sum_order)
 {
     auto al16 = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
-    if (m != 1) return false;  // several tokens: stand-alone quantiser (rows in parallel) + MFMA GEMV
+    // More than GEMV_FUSED_MAX_ROWS tokens: stand-alone quantiser (rows in parallel) + MFMA GEMV.  Two to
+    // GEMV_FUSED_MAX_ROWS tokens: the 16-wavefront kernel with a set of workgroups per token (half the launches; the
+    // weight tiles are fetched once per token, from the caches after the first), where that kernel applies.
+    if (m == 0 || m > (size_t)GEMV_FUSED_MAX_ROWS) return false;
+    if (m > 1 && !((gamma == nullptr || sum_order == BITNET_HIP_SUM_BLOCK256) && k <= 8192 && ldx < ((size_t)1 << 31))) return false;
     if (k % 4 != 0 || ldx % 4 != 0 || k > (size_t)FUSED_NCH * 1024) return false;
     if (!al16(x) || (x2 && !al16(x2)) || (gamma && !al16(gamma))) return false;
     if (input_mode == BITNET_HIP_INPUT_GQA_BROADCAST && head_dim % 4 != 0) return false;

@@ -630,7 +630,29 @@ def test_forward_multi_prefill_gate_up_one_launch():
         assert np.array_equal(got, host(layer.forward(dev(x), gamma=dev(g))))
 
 
-@pytest.mark.parametrize("m", [1, 2, 5, 8])
+@pytest.mark.parametrize("m", [1, 2, 3])
+@pytest.mark.parametrize("n,k", [(1, 4), (17, 260), (1000, 2560), (2560, 6912), (6912 + 5, 2560), (40, 8192)])
+def test_forward_fused_rows_bit_exact(m, n, k):
+    """One to three tokens take the 16-wavefront kernel with the quantiser in its prologue and a set of workgroups per
+    token: row-block groups that do not fill the last 8 of the grid, one / two chunks per thread, four row blocks per
+    workgroup, RMSNorm, bias and residual."""
+    rng = np.random.default_rng(31 * m + n + k)
+    w = synth_weights(rng, n, k)
+    x = synth_activations(rng, m, k, outliers=True)
+    g = (1 + 0.1 * rng.standard_normal(k, dtype=f32)).astype(f32)
+    bias = rng.standard_normal(n, dtype=f32)
+    res = rng.standard_normal((m, n), dtype=f32)
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n, use_bias=True), "rows")
+    layer.update_weights(dev(w))
+    layer.update_bias(dev(bias))
+    qw, ws_ = orc.quantize_weights_absmean(w)
+    for norm in (False, True):
+        ref = orc.bitlinear_forward(x, orc.pack_2bit(qw), n, ws_, g=g if norm else None, eps=1e-5, bias=bias, residual=res)[0]
+        got = host(layer.forward(dev(x), gamma=dev(g) if norm else None, residual=dev(res)))
+        assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8])
 def test_bitlinear_forward_decode_debug_outputs(m):
     """At decode token counts the quantiser runs inside the GEMV launch; its int8 row, scale and the int32
     accumulators are still observable and bit-exact, with and without RMSNorm, at both FFN widths."""
@@ -773,7 +795,7 @@ def oracle_stack(ref, x, hidden, ffn, qh, kvh, hd, eps=1e-5):
     return x, q, k
 
 
-@pytest.mark.parametrize("m", [1, 8])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8])
 def test_decoder_layer_config2_bit_exact(m):
     """BASELINE config 2: one decoder layer's seven projections at BitNet-2B shapes."""
     rng = np.random.default_rng(0)
