@@ -94,6 +94,18 @@ struct bitnet_hip_bitlinear {
 
 namespace {
 
+// Row blocks of the largest launch group (up to GEMV_MAX_PROJ projections share a decode launch).
+size_t launch_group_blocks(bitnet_hip_bitlinear *const *layers, size_t count)
+{
+    size_t most = 0;
+    for (size_t j0 = 0; j0 < count; j0 += GEMV_MAX_PROJ) {
+        size_t sum = 0;
+        for (size_t j = j0; j < count && j < j0 + GEMV_MAX_PROJ; ++j) sum += row_blocks(layers[j]->out_features);
+        most = sum > most ? sum : most;
+    }
+    return most;
+}
+
 // Runs `count` projections that share one input row block [m, k].  At decode token counts the quantiser runs
 // inside the GEMV launch (up to GEMV_MAX_PROJ projections per launch); otherwise the stand-alone quantiser
 // fills q / a_scale / a_sum (scratch the caller provides) and the GEMV or GEMM kernels consume them.
@@ -110,7 +122,7 @@ int run_projections(bitnet_hip_bitlinear *const *layers, int count, const float 
                        out[j], acc ? acc[j] : nullptr, bl->out_features};
         return pj;
     };
-    if (gemv_fused_supported(x, x2, ldx, m, k, input_mode, head_dim, gamma, sum_order)) {
+    if (gemv_fused_supported(x, x2, ldx, m, k, input_mode, head_dim, gamma, sum_order, launch_group_blocks(layers, count))) {
         for (int j0 = 0; j0 < count; j0 += GEMV_MAX_PROJ) {
             GemvProj pjs[GEMV_MAX_PROJ];
             const int nj = count - j0 < GEMV_MAX_PROJ ? count - j0 : GEMV_MAX_PROJ;
@@ -614,7 +626,7 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
 
     hipStream_t s = as_stream(stream);
     const bool debug = dbg_q || dbg_a_scale || dbg_acc;
-    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma, sum_order);
+    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma, sum_order, row_blocks(layer->out_features));
     void *ws = workspace;
     bool own_ws = false;
     QuantScratch sc = {dbg_q, dbg_a_scale, nullptr};
@@ -665,7 +677,7 @@ int bitnet_hip_bitlinear_forward_multi(bitnet_hip_bitlinear *const *layers, size
     }
     const size_t in = layers[0]->in_features;
     hipStream_t s = as_stream(stream);
-    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma, sum_order);
+    const bool fused = gemv_fused_supported(x, nullptr, in, m, in, BITNET_HIP_INPUT_PLAIN, 1, gamma, sum_order, launch_group_blocks(layers, count));
     void *ws = workspace;
     bool own_ws = false;
     QuantScratch sc = {nullptr, nullptr, nullptr};

@@ -42,7 +42,8 @@ namespace bitnet {
 namespace {
 
 constexpr int MODE_PREQUANT = -1;
-constexpr int GEMV_FUSED_MAX_ROWS = 3;  // tokens per fused quantiser + GEMV launch
+constexpr int GEMV_FUSED_MAX_ROWS = 6;   // tokens per fused quantiser + GEMV launch (measured: 2..6 gain, 8 loses)
+constexpr int GEMV_FUSED_MAX_WGS = 512;  // and its workgroups over all tokens: one round on 256 compute units
 constexpr int FUSED_NCH = 7;  // 16-byte f32 chunks per thread kept in registers: K <= 7168
 
 struct GemvProjDev {
@@ -430,7 +431,7 @@ template <int MODE, bool NORM, int NCHB, int RBW>
 __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, const float *hot_x2, const float *hot_gamma, int hot_k, int hot_head_dim,
                                                            int hot_gqa_group, int hot_ldx, GemvParams p)
 {
-    // A launch has one to three tokens (input rows), each with its own workgroups.  Workgroup (x, y) of the grid works on
+    // A launch has one to six tokens (input rows), each with its own workgroups.  Workgroup (x, y) of the grid works on
     // token x / 8 and on group 8y + x % 8 of row blocks: the workgroups of one group are neighbours in dispatch order and,
     // workgroups going to the XCDs in turn, run on the same XCD, so its L2 fetches their weight tiles once.
     // The leading scalar arguments repeat what the first loads need (input rows, RMSNorm weights, k): the file is
@@ -1218,14 +1219,18 @@ int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const f
 }
 
 bool gemv_fused_supported(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
-                          size_t head_dim, const float *gamma, int sum_order)
+                          size_t head_dim, const float *gamma, int sum_order, size_t blocks)
 {
     auto al16 = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
-    // More than GEMV_FUSED_MAX_ROWS tokens: stand-alone quantiser (rows in parallel) + MFMA GEMV.  Two to
-    // GEMV_FUSED_MAX_ROWS tokens: the 16-wavefront kernel with a set of workgroups per token (half the launches; the
-    // weight tiles are fetched once per token, from the caches after the first), where that kernel applies.
+    // Two to GEMV_FUSED_MAX_ROWS tokens: the 16-wavefront kernel with a set of workgroups per token (half the launches;
+    // the weight tiles are fetched once per token, from the caches after the first), where that kernel applies and the
+    // workgroups of all tokens stay within GEMV_FUSED_MAX_WGS.  Otherwise: stand-alone quantiser (rows in parallel) + MFMA GEMV.
     if (m == 0 || m > (size_t)GEMV_FUSED_MAX_ROWS) return false;
-    if (m > 1 && !((gamma == nullptr || sum_order == BITNET_HIP_SUM_BLOCK256) && k <= 8192 && ldx < ((size_t)1 << 31))) return false;
+    if (m > 1) {
+        if (!((gamma == nullptr || sum_order == BITNET_HIP_SUM_BLOCK256) && k <= 8192 && ldx < ((size_t)1 << 31))) return false;
+        const size_t rbw = blocks * m > 512 ? 4 : 1;
+        if ((blocks + rbw - 1) / rbw * m > (size_t)GEMV_FUSED_MAX_WGS) return false;
+    }
     if (k % 4 != 0 || ldx % 4 != 0 || k > (size_t)FUSED_NCH * 1024) return false;
     if (!al16(x) || (x2 && !al16(x2)) || (gamma && !al16(gamma))) return false;
     if (input_mode == BITNET_HIP_INPUT_GQA_BROADCAST && head_dim % 4 != 0) return false;
@@ -1243,7 +1248,7 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
     for (int j = 0; j < nproj; ++j) blocks += row_blocks(projs[j].n);
     // 16 wavefronts per workgroup (the declared summation order only; k <= 8192: two chunks per thread, 32 k-tiles)
     if ((gamma == nullptr || sum_order == BITNET_HIP_SUM_BLOCK256) && k <= 8192) {
-        const int rbw16 = (blocks > 512 && k <= 4096) ? 4 : 1;
+        const int rbw16 = ((m == 1 ? (blocks > 512 && k <= 4096) : blocks * m > 512)) ? 4 : 1;  // workgroups of all tokens: one round
         GemvParams p = {};
         if (fill_projs(p, projs, nproj, 0, k, rbw16) == 0) return BITNET_HIP_OK;
         p.m = (int)m;

@@ -57,7 +57,8 @@ int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const f
 // f32 input quantised inside the GEMV launch; only where gemv_fused_supported() says so.  q_out / a_scale_out /
 // a_sum_out (each optional) receive the quantiser's results.
 bool gemv_fused_supported(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
-                          size_t head_dim, const float *gamma, int sum_order);
+                          size_t head_dim, const float *gamma, int sum_order, size_t blocks);
+// blocks: 16-row blocks of all projections of the launch (of its largest launch group)
 int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const float *x2, size_t ldx, size_t m,
                       size_t k, int input_mode, size_t gqa_group, size_t head_dim, const float *gamma, float eps,
                       int sum_order, int8_t *q_out, float *a_scale_out, int32_t *a_sum_out, hipStream_t stream);

@@ -630,12 +630,13 @@ def test_forward_multi_prefill_gate_up_one_launch():
         assert np.array_equal(got, host(layer.forward(dev(x), gamma=dev(g))))
 
 
-@pytest.mark.parametrize("m", [1, 2, 3])
-@pytest.mark.parametrize("n,k", [(1, 4), (17, 260), (1000, 2560), (2560, 6912), (6912 + 5, 2560), (40, 8192)])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 7])
+@pytest.mark.parametrize("n,k", [(1, 4), (17, 260), (1000, 2560), (2560, 6912), (6912 + 5, 2560), (40, 8192), (13824, 2560)])
 def test_forward_fused_rows_bit_exact(m, n, k):
-    """One to three tokens take the 16-wavefront kernel with the quantiser in its prologue and a set of workgroups per
-    token: row-block groups that do not fill the last 8 of the grid, one / two chunks per thread, four row blocks per
-    workgroup, RMSNorm, bias and residual."""
+    """One to six tokens take the 16-wavefront kernel with the quantiser in its prologue and a set of workgroups per
+    token, as long as those stay within 512 (otherwise, and from seven tokens on, the stand-alone quantiser and the MFMA
+    GEMV run): row-block groups that do not fill the last 8 of the grid, one / two chunks per thread, one / four row
+    blocks per workgroup, RMSNorm, bias and residual."""
     rng = np.random.default_rng(31 * m + n + k)
     w = synth_weights(rng, n, k)
     x = synth_activations(rng, m, k, outliers=True)
@@ -795,7 +796,7 @@ def oracle_stack(ref, x, hidden, ffn, qh, kvh, hd, eps=1e-5):
     return x, q, k
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 8])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8])
 def test_decoder_layer_config2_bit_exact(m):
     """BASELINE config 2: one decoder layer's seven projections at BitNet-2B shapes."""
     rng = np.random.default_rng(0)
