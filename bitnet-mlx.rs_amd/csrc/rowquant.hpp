@@ -236,9 +236,16 @@ __device__ __forceinline__ float scale_from_absmax(float amax)
 
 __device__ __forceinline__ int quant1(float y, float scale)
 {
-    // round half away from zero, then a saturating conversion (NaN converts to 0, as Rust's `as i8` does),
-    // then the clamp to [-128, 127] on the integer
-    const int q = __float2int_rz(roundf(f32_mul(y, scale)));
+    // Round half away from zero, then a saturating conversion (NaN converts to 0, as Rust's `as i8` does), then the clamp
+    // to [-128, 127] on the integer.  The rounding is one addition of +-(1/2 - 2^-25), the largest float below 1/2, and the
+    // truncating conversion: with 1/2 itself the sum for |t| = 1/2 - 2^-25 would round up to 1; with its predecessor
+    // that sum is exact, |t| = 1/2 still rounds up to 1, and every other sum is exact or rounds within the gap between
+    // two integers (past 2^23, where it may not, the clamp decides).  Checked against roundf, cast and clamp over all
+    // 2^32 bit patterns of t.  v_cvt_i32_f32 truncates, saturates and turns NaN into 0.
+    const float t = f32_mul(y, scale);
+    const float s = f32_add(t, __builtin_copysignf(0x1.fffffep-2f, t));
+    int q;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(s));
     return min(max(q, -128), 127);
 }
 

@@ -517,3 +517,16 @@ def test_lookup_kernel_edges():
     assert np.isnan(out[0]) and out[1] == np.inf and np.isnan(out[2])
     assert orc.lookup_compute(0, [-2], [3.0]).tolist() == [0.0] and orc.lookup_compute(1, [-2], [3.0]).tolist() == [-6.0]
     assert np.signbit(orc.lookup_compute(0, [0], [-3.0])[0])  # -3 * 0 = -0
+
+
+def test_quantiser_rounding_identity_over_all_floats(tmp_path):
+    """The HIP quantiser rounds with one addition of +-(1/2 - 2^-25) and a truncating conversion instead of roundf;
+    tests/rounding_identity_check.c compares the two, followed by the saturating cast and the int8 clamp, over all 2^32
+    float bit patterns (about half a minute of CPU time over the available cores)."""
+    import subprocess
+    from pathlib import Path
+    src = Path(__file__).with_name("rounding_identity_check.c")
+    exe = tmp_path / "rounding_identity_check"
+    subprocess.run(["gcc", "-O2", "-fopenmp", "-fno-fast-math", str(src), "-o", str(exe), "-lm"], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=900)
+    assert out.returncode == 0 and "mismatches: 0" in out.stdout, out.stdout[-500:]
