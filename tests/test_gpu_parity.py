@@ -823,6 +823,59 @@ def test_decoder_stack_small_bit_exact(layers):
     assert ei.value.kind == "ShapeMismatch"
 
 
+def random_packed_ternary(rng, n, k):
+    """[n, k] ternary weights as flat 2-bit bytes drawn directly (code 3 folded onto code 1: weight 0), so a
+    30-block stack of 521 MB is generated in a second: P(-1) = P(+1) = 1/4, P(0) = 1/2."""
+    b = rng.integers(0, 256, size=n * k // 4, dtype=np.uint8)
+    return b & ~((b & (b >> 1) & 0x55) << 1)
+
+
+def build_decoder_packed(rng, layers, hidden, ffn, qh, kvh, hd, max_tokens, eps=1e-5):
+    dec = bh.DecoderProjections(layers, hidden, ffn, qh, kvh, hd, eps=eps, max_tokens=max_tokens)
+    ref = []
+    for l in range(layers):
+        packed, scales = [], []
+        for p in range(7):
+            n, k = dec.proj_shape(p)
+            pk = random_packed_ternary(rng, n, k)
+            s = f32(0.016 * (1 + 0.25 * rng.random()))
+            dec.projection(l, p).set_quantized_weights(torch.from_numpy(pk), float(s))
+            packed.append(pk)
+            scales.append(s)
+        ga = (1 + 0.1 * rng.standard_normal(hidden, dtype=f32)).astype(f32)
+        gf = (1 + 0.1 * rng.standard_normal(hidden, dtype=f32)).astype(f32)
+        dec.set_norm(l, 0, torch.from_numpy(ga))
+        dec.set_norm(l, 1, torch.from_numpy(gf))
+        ref.append((packed, scales, ga, gf))
+    return dec, ref
+
+
+def test_decoder_stack_config5_full_depth_bit_exact():
+    """BASELINE config 5 at its real depth: 30 blocks at 2560 / 6912 / 20 / 5 / 128 (521,011,200 packed bytes) on a
+    decoder sized for 8 tokens, one token and eight tokens per step, every block checked against the oracle's chain;
+    then runs of blocks that start and end inside the stack, in place."""
+    dims = (2560, 6912, 20, 5, 128)
+    rng = np.random.default_rng(5)
+    dec, ref = build_decoder_packed(rng, 30, *dims, max_tokens=8)
+    assert dec.weight_bytes() == 521_011_200
+    for m in (1, 8):
+        x = synth_activations(rng, m, dims[0])
+        # the oracle's hidden state after every block
+        states, cur = [x], x
+        for l in range(30):
+            cur, q_ref, k_ref = oracle_stack(ref[l:l + 1], cur, *dims)
+            states.append(cur)
+        assert np.all(np.isfinite(states[-1]))
+        out, q, k = dec.decode(dev(x), want_qk=True)
+        assert np.array_equal(host(out), states[30]), f"m={m}: 30-block output differs from the oracle"
+        assert np.array_equal(host(q), q_ref) and np.array_equal(host(k), k_ref)
+        assert rel_err(host(out), states[30]) <= REL_TOL
+        for lo, hi in ((2, 7), (4, 5), (3, 30), (29, 30)):
+            buf = dev(states[lo].copy())
+            dec.decode(buf, out=buf, layers=(lo, hi))
+            assert np.array_equal(host(buf), states[hi]), f"m={m}: blocks {lo}..{hi - 1}"
+
+
 @pytest.mark.parametrize("dims,layers", [((2560, 6912, 20, 5, 128), 4), ((256, 512, 4, 2, 64), 3),
                                          ((1024, 2816, 8, 8, 128), 2)])
 def test_decoder_single_launch_matches_oracle_and_per_launch_path(dims, layers):
