@@ -69,6 +69,46 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 using namespace bitnet;
 
 // ---------------------------------------------------------------------------------------------------
+// Static scratch of bitnet_hip_bitlinear_forward_noalloc: the quantised activations of one call
+// (int8 [m, in], a_scale [m], a_sum [m]) live in this file-scope device array instead of a workspace the
+// caller passes or the call allocates.  Every GPU the library runs on holds its own copy until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the address each device
+// gave it is looked up once per device and kept in noalloc_scratch_ptr; kernels only ever get that pointer.
+// ---------------------------------------------------------------------------------------------------
+namespace {
+constexpr size_t NOALLOC_MAX_ELEMS = (size_t)1 << 20;  // m * in_features of one call
+constexpr size_t NOALLOC_MAX_ROWS = 4096;              // m of one call
+constexpr size_t NOALLOC_SCRATCH_BYTES = NOALLOC_MAX_ELEMS + 2 * NOALLOC_MAX_ROWS * sizeof(float) + 512;
+constexpr int NOALLOC_MAX_DEVICES = 64;
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+namespace {
+std::mutex noalloc_lock;
+void *noalloc_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+
+// Device address of `scratch` on the current device (looked up on first use, per device).
+int noalloc_scratch(void **out)
+{
+    int device = 0;
+    BITNET_HIP_TRY(hipGetDevice(&device));
+    if (device < 0 || device >= NOALLOC_MAX_DEVICES)
+        return fail(BITNET_HIP_UNSUPPORTED, "device ordinal %d is beyond the %d this library keeps scratch for", device,
+                    NOALLOC_MAX_DEVICES);
+    std::lock_guard<std::mutex> guard(noalloc_lock);
+    if (!noalloc_scratch_ptr[device]) {
+        void *ptr = nullptr;
+        BITNET_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(BITNET_HIP_DEVICE_ERROR, "hipGetSymbolAddress returned no address for the static scratch");
+        noalloc_scratch_ptr[device] = ptr;
+    }
+    *out = noalloc_scratch_ptr[device];
+    return BITNET_HIP_OK;
+}
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------
 // BitLinear object
 // ---------------------------------------------------------------------------------------------------
 struct bitnet_hip_bitlinear {
@@ -211,7 +251,8 @@ int bitnet_hip_init(int device)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(BITNET_HIP_UNSUPPORTED, "device %d is %s; this library carries gfx950 code only", device,
                     prop.gcnArchName);
-    return BITNET_HIP_OK;
+    void *ptr = nullptr;
+    return noalloc_scratch(&ptr);  // this device's address of the static scratch, kept for forward_noalloc
 }
 
 int bitnet_hip_device_info(char *arch_name, size_t arch_name_len, int *compute_units, int *clock_mhz,
@@ -655,6 +696,52 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
             rc = fail(BITNET_HIP_MEMORY_ERROR, "forward: hipFreeAsync failed: %s", hipGetErrorString(e));
     }
     return rc;
+}
+
+int bitnet_hip_bitlinear_forward_noalloc(bitnet_hip_bitlinear *layer, const float *x, const size_t *dims, int rank,
+                                         const float *gamma, float eps, int sum_order, const float *residual,
+                                         float *out, void *stream)
+{
+    if (!layer) return fail(BITNET_HIP_NULL_POINTER, "forward_noalloc: layer is NULL");
+    const size_t in = layer->in_features;
+    if (rank <= 0 || !dims) {
+        size_t e[2] = {1, in};
+        return fail_shape(e, 2, dims, 0, "input");
+    }
+    if (dims[rank - 1] != in) {
+        size_t e[2] = {dims[0], in};
+        return fail_shape(e, 2, dims, rank, "last input dimension");
+    }
+    if (rank != 2 && rank != 3) {
+        size_t e[2] = {1, in};
+        return fail_shape(e, 2, dims, rank, "input rank");
+    }
+    const size_t m = rank == 2 ? dims[0] : dims[0] * dims[1];
+    if (m == 0) return BITNET_HIP_OK;
+    if (!x || !out) return fail(BITNET_HIP_NULL_POINTER, "forward_noalloc: x and out are required");
+    if (m > NOALLOC_MAX_ROWS || m * in > NOALLOC_MAX_ELEMS)
+        return fail(BITNET_HIP_MEMORY_ERROR,
+                    "forward_noalloc: %zu rows x %zu features exceed the static scratch (at most %zu rows and %zu "
+                    "rows*features per call); use bitnet_hip_bitlinear_forward with a workspace",
+                    m, in, NOALLOC_MAX_ROWS, NOALLOC_MAX_ELEMS);
+    static_assert(NOALLOC_MAX_ELEMS % 256 == 0 && (NOALLOC_MAX_ROWS * sizeof(float)) % 256 == 0 &&
+                      NOALLOC_SCRATCH_BYTES >= NOALLOC_MAX_ELEMS + 2 * NOALLOC_MAX_ROWS * sizeof(float) + 256,
+                  "the scratch holds q, a_scale and a_sum of the largest call");
+    void *ws = nullptr;
+    int rc = noalloc_scratch(&ws);
+    if (rc != BITNET_HIP_OK) return rc;
+    if (quant_scratch_bytes(m, in) > NOALLOC_SCRATCH_BYTES)
+        return fail(BITNET_HIP_MEMORY_ERROR, "forward_noalloc: %zu bytes of scratch needed, %zu held", quant_scratch_bytes(m, in),
+                    NOALLOC_SCRATCH_BYTES);
+
+    std::shared_lock<std::shared_mutex> guard(layer->lock);
+    if (!layer->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "forward_noalloc: the layer has no weights yet");
+    const QuantScratch sc = carve_scratch(ws, m, in);
+    bitnet_hip_bitlinear *layers[1] = {layer};
+    const float *res[1] = {residual};
+    float *outs[1] = {out};
+    return run_projections(layers, 1, x, nullptr, in, m, BITNET_HIP_INPUT_PLAIN, 1, 1, gamma, eps, sum_order, res, outs,
+                           nullptr, sc.q, sc.a_scale, sc.a_sum, false, as_stream(stream));
 }
 
 int bitnet_hip_bitlinear_forward_multi(bitnet_hip_bitlinear *const *layers, size_t count, const float *x, size_t m,

@@ -109,6 +109,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_bitlinear_get_quantized": (i32, [vp, C.POINTER(f32), vp, sz]),
         "bitnet_hip_bitlinear_workspace_size": (sz, [vp, sz]),
         "bitnet_hip_bitlinear_forward": (i32, [vp, vp, C.POINTER(sz), i32, vp, f32, i32, vp, vp, vp, sz, vp, vp, vp, vp]),
+        "bitnet_hip_bitlinear_forward_noalloc": (i32, [vp, vp, C.POINTER(sz), i32, vp, f32, i32, vp, vp, vp]),
         "bitnet_hip_bitlinear_forward_multi": (i32, [C.POINTER(vp), sz, vp, sz, vp, f32, i32, C.POINTER(vp), vp, sz, vp]),
         "bitnet_hip_bitlinear_matmul": (i32, [vp, vp, vp, sz, vp, vp, vp, vp, vp]),
         "bitnet_hip_decoder_decode_layers": (i32, [vp, sz, sz, vp, sz, vp, vp, vp, vp]),
@@ -167,6 +168,34 @@ def _dev(t: torch.Tensor, dtype, name: str):
     if not t.is_contiguous():
         raise BitLinearError(INVALID_CONFIG, f"{name} must be contiguous")
     return t
+
+
+def _opt_dev(t: Optional[torch.Tensor], dtype, name: str, numel: int, like: torch.Tensor):
+    """An optional device operand: right device, dtype, contiguity and element count, or a BitLinearError."""
+    if t is None:
+        return None
+    _dev(t, dtype, name)
+    if t.device != like.device:
+        raise BitLinearError(DEVICE_ERROR, f"{name} lives on {t.device}, the input on {like.device}")
+    if t.numel() != numel:
+        raise BitLinearError(SHAPE_MISMATCH, name, [numel], [t.numel()])
+    return t
+
+
+def _check_optional_operands(layer: "BitLinear", x: torch.Tensor, gamma, residual, out=None):
+    """gamma [in], residual [m, out], out [.., out]: checked on the host so that a wrong tensor is a BitLinearError and
+    never a wild pointer inside a kernel.  Shape errors of x itself are left to the library (it reports them as the
+    reference does)."""
+    nin, nout = layer.config.in_features, layer.config.out_features
+    if x.dim() not in (2, 3) or x.shape[-1] != nin:
+        return
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    _opt_dev(gamma, torch.float32, "gamma", nin, x)
+    _opt_dev(residual, torch.float32, "residual", m * nout, x)
+    if out is not None:
+        _opt_dev(out, torch.float32, "out", m * nout, x)
 
 
 def init(device: int = 0):
@@ -488,6 +517,20 @@ class BitLinear:
                                                 _ptr(q), _ptr(a_scale), _ptr(acc), _stream(stream)))
         if debug:
             return out, q, a_scale, acc
+        return out
+
+    def forward_noalloc(self, x: torch.Tensor, out: torch.Tensor, gamma: Optional[torch.Tensor] = None,
+                        residual: Optional[torch.Tensor] = None, stream=None):
+        """forward() into a caller-supplied `out` with the quantised activations in the library's static per-GPU
+        scratch: no device allocation by the library or by this method.  At most 4096 rows and
+        rows * in_features <= 1,048,576 per call; calls that overlap on one GPU race."""
+        _dev(x, torch.float32, "input")
+        _dev(out, torch.float32, "out")
+        _check_optional_operands(self, x, gamma, residual, out)
+        dims = (C.c_size_t * max(x.dim(), 1))(*x.shape)
+        _check(load_library().bitnet_hip_bitlinear_forward_noalloc(
+            self._h, _ptr(x), dims, x.dim(), _ptr(gamma), self.config.rms_norm_eps, self.config.sum_order,
+            _ptr(residual), _ptr(out), _stream(stream)))
         return out
 
     def workspace_size(self, m: int) -> int:

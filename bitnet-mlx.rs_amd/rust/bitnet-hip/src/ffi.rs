@@ -93,6 +93,9 @@ extern "C" {
                                         residual: *const f32, out: *mut f32, workspace: *mut c_void,
                                         workspace_bytes: usize, dbg_q: *mut i8, dbg_a_scale: *mut f32,
                                         dbg_acc: *mut i32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_bitlinear_forward_noalloc(layer: *mut bitnet_hip_bitlinear, x: *const f32, dims: *const usize,
+                                                rank: c_int, gamma: *const f32, eps: f32, sum_order: c_int,
+                                                residual: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_bitlinear_forward_multi(layers: *const *mut bitnet_hip_bitlinear, count: usize, x: *const f32,
                                               m: usize, gamma: *const f32, eps: f32, sum_order: c_int,
                                               outs: *const *mut f32, workspace: *mut c_void, workspace_bytes: usize,

@@ -241,6 +241,20 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
                                  float *out, void *workspace, size_t workspace_bytes, int8_t *dbg_q,
                                  float *dbg_a_scale, int32_t *dbg_acc, void *stream);
 
+/* bitnet_hip_bitlinear_forward for callers that cannot allocate device memory and have no workspace to pass:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference (BitLinearForward::forward returns a fresh tensor, forward.rs:55-92).  The quantised
+ * activations (int8 [m, in], a_scale [m], a_sum [m]) live in a file-scope device array of the library,
+ * 1,081,856 bytes per GPU, held until the process ends; the call performs no hipMalloc / hipFree of any kind.
+ * Limits: m <= 4096 rows and m * in_features <= 1,048,576 per call, otherwise BITNET_HIP_MEMORY_ERROR and
+ * nothing is launched (use bitnet_hip_bitlinear_forward with a workspace).  Same arguments, shape rules and
+ * results (bit for bit) as bitnet_hip_bitlinear_forward without the debug outputs.  All calls on one GPU share
+ * the array: calls that overlap in time on the same GPU (two streams, two threads) race; issue them on one
+ * stream, or order them with events. */
+int bitnet_hip_bitlinear_forward_noalloc(bitnet_hip_bitlinear *layer, const float *x, const size_t *dims, int rank,
+                                         const float *gamma, float eps, int sum_order, const float *residual,
+                                         float *out, void *stream);
+
 /* Several layers applied to the same input x [m, in] (q, k, v of an attention block; gate, up of an FFN):
  * MultiHeadAttention::forward runs q_proj/k_proj/v_proj on one input
  * (bitnet-inference/src/engine/transformer_layers.rs:470-475), FeedForwardNetwork::forward up_proj/gate_proj
