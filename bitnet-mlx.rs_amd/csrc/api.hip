@@ -360,6 +360,10 @@ int bitnet_hip_quantize_weights(const float *w, size_t n, size_t k, int method, 
 {
     if (!w_scale) return fail(BITNET_HIP_NULL_POINTER, "quantize_weights: w_scale is required");
     if (n * k != 0 && (!w || !packed)) return fail(BITNET_HIP_NULL_POINTER, "quantize_weights: null buffer");
+    if (method >= BITNET_HIP_TERNARY_REF_MEAN_THRESHOLD && method <= BITNET_HIP_TERNARY_REF_DETSTE)
+        // the reference's own pipeline with WeightQuantizationConfig's defaults (weights.rs:81-95): normalise, clip at 3.0
+        return bitnet_hip_quantize_weights_reference(w, n, k, method - BITNET_HIP_TERNARY_REF_MEAN_THRESHOLD, 1, 3.0f,
+                                                     threshold_factor, packed, w_scale, q_i8, nullptr, stream);
     if (method != BITNET_HIP_TERNARY_ABSMEAN_ROUNDCLIP && method != BITNET_HIP_TERNARY_MEAN_THRESHOLD)
         return fail(BITNET_HIP_INVALID_CONFIG, "quantize_weights: unknown method %d", method);
     DeviceTemp row_sums;
@@ -369,6 +373,27 @@ int bitnet_hip_quantize_weights(const float *w, size_t n, size_t k, int method, 
                                  w_scale, q_i8, as_stream(stream));
     if (rc != BITNET_HIP_OK) return rc;
     BITNET_HIP_TRY(hipStreamSynchronize(as_stream(stream)));  // row_sums is released on return
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_quantize_weights_reference(const float *w, size_t n, size_t k, int ternary_method, int normalize_weights,
+                                          float outlier_threshold, float custom_threshold_factor, uint8_t *packed,
+                                          float *w_scale, int8_t *q_i8, float *stats, void *stream)
+{
+    if (!w_scale) return fail(BITNET_HIP_NULL_POINTER, "quantize_weights_reference: w_scale is required");
+    if (n * k != 0 && (!w || !packed)) return fail(BITNET_HIP_NULL_POINTER, "quantize_weights_reference: null buffer");
+    if (ternary_method < 0 || ternary_method > 4)
+        return fail(BITNET_HIP_INVALID_CONFIG, "quantize_weights_reference: unknown TernaryMethod %d", ternary_method);
+    // WeightQuantizationConfig::validate (weights.rs:120-150)
+    if (outlier_threshold < 0.0f) return fail(BITNET_HIP_INVALID_CONFIG, "Outlier threshold cannot be negative");
+    if (custom_threshold_factor > 2.0f) return fail(BITNET_HIP_INVALID_CONFIG, "Custom threshold factor must be in range (0, 2]");
+    DeviceTemp scratch;
+    int rc = scratch.alloc(quantize_weights_reference_scratch_bytes(n));
+    if (rc != BITNET_HIP_OK) return rc;
+    rc = launch_quantize_weights_reference(w, n, k, ternary_method, normalize_weights != 0, outlier_threshold,
+                                           custom_threshold_factor, scratch.ptr, packed, w_scale, q_i8, stats, as_stream(stream));
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipStreamSynchronize(as_stream(stream)));  // the scratch is released on return
     return BITNET_HIP_OK;
 }
 
@@ -497,6 +522,7 @@ int bitnet_hip_bitlinear_set_weights_f32(bitnet_hip_bitlinear *layer, const floa
     int rc = flat.alloc((n * k + 3) / 4);
     if (rc != BITNET_HIP_OK) return rc;
     std::unique_lock<std::shared_mutex> guard(layer->lock);
+    BITNET_HIP_TRY(hipDeviceSynchronize());  // forwards already queued on any stream still read the old weights
     rc = bitnet_hip_quantize_weights(src, rows, cols, method, threshold_factor, static_cast<uint8_t *>(flat.ptr),
                                      layer->w_scale, nullptr, stream);
     if (rc != BITNET_HIP_OK) return rc;
@@ -521,6 +547,7 @@ int bitnet_hip_bitlinear_set_weights_packed(bitnet_hip_bitlinear *layer, const u
     }
     hipStream_t s = as_stream(stream);
     std::unique_lock<std::shared_mutex> guard(layer->lock);
+    BITNET_HIP_TRY(hipDeviceSynchronize());  // forwards already queued on any stream still read the old weights
     BITNET_HIP_TRY(hipMemcpyAsync(layer->packed, packed, need, on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, s));
     BITNET_HIP_TRY(hipMemcpyAsync(layer->w_scale, &w_scale, sizeof(float), hipMemcpyHostToDevice, s));
     int rc = launch_retile(layer->packed, n, k, BITNET_HIP_LAYOUT_OUT_IN, layer->tiled, s);
@@ -549,6 +576,7 @@ int bitnet_hip_bitlinear_set_weights_base3(bitnet_hip_bitlinear *layer, const ui
         src = static_cast<const uint8_t *>(staged.ptr);
     }
     std::unique_lock<std::shared_mutex> guard(layer->lock);
+    BITNET_HIP_TRY(hipDeviceSynchronize());  // forwards already queued on any stream still read the old weights
     int rc = launch_base3_to_2bit(src, n * k, layer->packed, s);
     if (rc != BITNET_HIP_OK) return rc;
     BITNET_HIP_TRY(hipMemcpyAsync(layer->w_scale, &w_scale, sizeof(float), hipMemcpyHostToDevice, s));
@@ -588,6 +616,7 @@ int bitnet_hip_bitlinear_set_weights_gguf(bitnet_hip_bitlinear *layer, const uin
     int rc = flat.alloc(codes);
     if (rc != BITNET_HIP_OK) return rc;
     std::unique_lock<std::shared_mutex> guard(layer->lock);
+    BITNET_HIP_TRY(hipDeviceSynchronize());  // forwards already queued on any stream still read the old weights
     BITNET_HIP_TRY(hipMemcpyAsync(flat.ptr, data + 8, codes, on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, s));
     BITNET_HIP_TRY(hipMemcpyAsync(layer->w_scale, &header[0], sizeof(float), hipMemcpyHostToDevice, s));
     rc = launch_retile(static_cast<const uint8_t *>(flat.ptr), n, k, layout, layer->tiled, s);
@@ -608,6 +637,7 @@ int bitnet_hip_bitlinear_set_bias(bitnet_hip_bitlinear *layer, const float *bias
         return fail_shape(e, 1, a, 1, "bias");
     }
     std::unique_lock<std::shared_mutex> guard(layer->lock);
+    BITNET_HIP_TRY(hipDeviceSynchronize());  // forwards already queued on any stream still read the old bias
     BITNET_HIP_TRY(hipMemcpyAsync(layer->bias, bias, sizeof(float) * len,
                                   on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, as_stream(stream)));
     BITNET_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
@@ -816,24 +846,20 @@ struct bitnet_hip_decoder {
     int32_t *a_sum = nullptr;
     float *qb = nullptr, *kb = nullptr, *vb = nullptr, *x1 = nullptr, *gate = nullptr, *up = nullptr;
     float *ping = nullptr;
-    // single-launch decode (decode_stack.hip): pointer table, barrier flags (+ abort word), host-visible status
-    StackLayer *table = nullptr;
-    float *ring = nullptr;     // activations of the single-launch path, one slice per block
-    unsigned *flags = nullptr;
-    unsigned *host_status = nullptr;
-    unsigned epoch = 0;
-    int grid = 0;              // one workgroup per compute unit
-    bool single_launch = false;  // shapes fit and the device takes cooperative launches
-    bool single_launch_enabled = false;  // opt-in: measured on MI355X it only matches the launch-per-group path
-    std::mutex stack_lock;     // launches share the flags: one at a time
+    // One decode at a time: the activation buffers above are shared by every call on this decoder.  The mutex
+    // serialises the enqueue; `done` (recorded behind every decode) makes a decode on another stream wait for it.
+    std::mutex decode_lock;
+    hipEvent_t done = nullptr;
+    hipStream_t done_stream = nullptr;
+    bool done_recorded = false;
 
     ~bitnet_hip_decoder()
     {
         for (auto *p : proj) delete p;
-        void *bufs[] = {gamma, a8, a_scale, a_sum, qb, kb, vb, x1, gate, up, ping, table, flags, ring};
+        void *bufs[] = {gamma, a8, a_scale, a_sum, qb, kb, vb, x1, gate, up, ping};
         for (void *b : bufs)
             if (b) (void)hipFree(b);
-        if (host_status) (void)hipHostFree(host_status);
+        if (done) (void)hipEventDestroy(done);
     }
 };
 
@@ -888,30 +914,8 @@ int bitnet_hip_decoder_create(size_t layers, size_t hidden, size_t ffn, size_t q
         if (e != hipSuccess) rc = fail(BITNET_HIP_DEVICE_ERROR, "decoder_create: hipMemcpy failed: %s", hipGetErrorString(e));
     }
     if (rc == BITNET_HIP_OK) {
-        // single-launch path: one workgroup per compute unit, if the shapes fit its register and LDS plan
-        int dev = 0, cus = 0, coop = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
-            hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) == hipSuccess && coop &&
-            decode_stack_supported(hidden, ffn, kv_dim, head_dim, sum_order, cus)) {
-            d->grid = cus;
-            std::vector<StackLayer> host_table(layers);
-            for (size_t l = 0; l < layers; ++l)
-                for (int p = 0; p < 7; ++p) {
-                    host_table[l].w[p] = d->proj[l * 7 + p]->tiled;
-                    host_table[l].w_scale[p] = d->proj[l * 7 + p]->w_scale;
-                }
-            dev_alloc(&d->table, sizeof(StackLayer) * layers);
-            dev_alloc(&d->flags, sizeof(unsigned) * ((size_t)cus + 1));
-            dev_alloc(&d->ring, sizeof(float) * layers * decode_stack_ring_stride(hidden, ffn, kv_dim));
-            if (rc == BITNET_HIP_OK) {
-                hipError_t e = hipMemcpy(d->table, host_table.data(), sizeof(StackLayer) * layers, hipMemcpyHostToDevice);
-                if (e == hipSuccess) e = hipMemset(d->flags, 0, sizeof(unsigned) * ((size_t)cus + 1));
-                if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void **>(&d->host_status), sizeof(unsigned), hipHostMallocMapped);
-                if (e == hipSuccess) { *d->host_status = 0; d->single_launch = true; }
-                else rc = fail(BITNET_HIP_DEVICE_ERROR, "decoder_create: single-launch set-up failed: %s", hipGetErrorString(e));
-            }
-        }
+        hipError_t e = hipEventCreateWithFlags(&d->done, hipEventDisableTiming);
+        if (e != hipSuccess) rc = fail(BITNET_HIP_DEVICE_ERROR, "decoder_create: hipEventCreate failed: %s", hipGetErrorString(e));
     }
     if (rc != BITNET_HIP_OK) {
         delete d;
@@ -966,37 +970,24 @@ int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin
         size_t e[2] = {dec->max_tokens, dec->hidden}, a[2] = {m, dec->hidden};
         return fail_shape(e, 2, a, 2, "tokens per decode step exceed max_tokens");
     }
-    for (size_t i = layer_begin * 7; i < layer_end * 7; ++i)
-        if (!dec->proj[i]->has_weights)
-            return fail(BITNET_HIP_NOT_INITIALIZED, "decoder_decode: a projection has no weights yet");
     hipStream_t s = as_stream(stream);
     const size_t H = dec->hidden, F = dec->ffn, KV = dec->kv_heads * dec->head_dim;
     const size_t group = dec->q_heads / dec->kv_heads;
     int rc = BITNET_HIP_OK;
-    if (dec->host_status && *dec->host_status != 0)
-        return fail(BITNET_HIP_KERNEL_ERROR, "decoder_decode: an earlier single-launch decode gave up at a grid barrier");
-    auto aligned16 = [](const void *p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    // readers of every projection involved (weight updates take the write lock and wait for the GPU), and one
+    // decode at a time on this decoder's buffers
+    std::vector<std::shared_lock<std::shared_mutex>> guards;
+    guards.reserve((layer_end - layer_begin) * 7);
+    for (size_t i = layer_begin * 7; i < layer_end * 7; ++i) {
+        guards.emplace_back(dec->proj[i]->lock);
+        if (!dec->proj[i]->has_weights)
+            return fail(BITNET_HIP_NOT_INITIALIZED, "decoder_decode: a projection has no weights yet");
+    }
+    std::lock_guard<std::mutex> one_decode(dec->decode_lock);
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     (void)hipStreamIsCapturing(s, &capturing);
-    if (m == 1 && dec->single_launch && dec->single_launch_enabled && capturing == hipStreamCaptureStatusNone &&
-        layer_end - layer_begin <= decode_stack_max_layers() &&
-        aligned16(x_in) && aligned16(x_out) && aligned16(q_last) && aligned16(k_last)) {
-        StackParams sp;
-        sp.table = dec->table; sp.layer_begin = (int)layer_begin; sp.layer_end = (int)layer_end;
-        sp.step_begin = 0; sp.step_end = 4 * (int)(layer_end - layer_begin);
-        sp.x_in = x_in; sp.x_out = x_out; sp.ring = dec->ring;
-        sp.ring_stride = (int)decode_stack_ring_stride(H, F, KV);
-        sp.q_last = q_last; sp.k_last = k_last; sp.gamma = dec->gamma;
-        sp.hidden = (int)H; sp.ffn = (int)F; sp.kv_dim = (int)KV; sp.head_dim = (int)dec->head_dim; sp.gqa_group = (int)group;
-        sp.eps = dec->eps;
-        sp.flags = dec->flags; sp.abort_word = dec->flags + dec->grid; sp.host_status = dec->host_status;
-        sp.spin_limit = 0;
-        std::lock_guard<std::mutex> guard(dec->stack_lock);
-        sp.epoch0 = dec->epoch;
-        rc = launch_decode_stack(sp, dec->grid, s);
-        if (rc == BITNET_HIP_OK) dec->epoch += (unsigned)(4 * (layer_end - layer_begin) - 1);
-        return rc;
-    }
+    if (dec->done_recorded && dec->done_stream != s && capturing == hipStreamCaptureStatusNone)
+        BITNET_HIP_TRY(hipStreamWaitEvent(s, dec->done, 0));  // the previous decode used these buffers on another stream
     // one launch group: `count` projections reading the same (transformed) input
     auto run = [&](bitnet_hip_bitlinear *const *layers, int count, const float *x, const float *x2, size_t ldx, int mode,
                    const float *gamma, const float *res0, float *const *outs) {
@@ -1022,14 +1013,12 @@ int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin
         run(&P[BITNET_HIP_PROJ_DOWN], 1, dec->gate, dec->up, F, BITNET_HIP_INPUT_RELU2_MUL, nullptr, dec->x1, d_out);
         x = x2;
     }
+    if (rc == BITNET_HIP_OK && capturing == hipStreamCaptureStatusNone) {
+        BITNET_HIP_TRY(hipEventRecord(dec->done, s));
+        dec->done_stream = s;
+        dec->done_recorded = true;
+    }
     return rc;
-}
-
-int bitnet_hip_decoder_set_single_launch(bitnet_hip_decoder *dec, int enabled)
-{
-    if (!dec) return fail(BITNET_HIP_NULL_POINTER, "decoder_set_single_launch: null argument");
-    dec->single_launch_enabled = enabled != 0;
-    return dec->single_launch ? 1 : 0;
 }
 
 int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t m, float *x_out, float *q_last,

@@ -31,6 +31,12 @@ int launch_base3_to_2bit(const uint8_t *base3, size_t count, uint8_t *packed, hi
 int launch_quantize_weights(const float *w, size_t n, size_t k, int method, float threshold_factor,
                             double *row_sums, uint8_t *packed, float *w_scale, int8_t *q_i8,
                             hipStream_t stream);
+// BitNetWeightQuantizer::quantize (weights.rs:568-611): method = TernaryMethod 0..4, custom_factor <= 0 = none;
+// scratch: quantize_weights_reference_scratch_bytes(n) bytes of device memory; stats: 12 floats or null
+size_t quantize_weights_reference_scratch_bytes(size_t n);
+int launch_quantize_weights_reference(const float *w, size_t n, size_t k, int method, int normalize, float outlier_threshold,
+                                      float custom_factor, void *scratch, uint8_t *packed, float *w_scale, int8_t *q_i8,
+                                      float *stats, hipStream_t stream);
 int launch_retile(const uint8_t *packed, size_t n, size_t k, int layout, uint8_t *tiled, hipStream_t stream);
 int launch_untile(const uint8_t *tiled, size_t n, size_t k, uint8_t *packed, hipStream_t stream);
 
@@ -72,34 +78,5 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
 int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_sum, size_t m, size_t n, size_t k,
                       int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,
                       const float *residual, float *out, hipStream_t stream);
-
-// decode_stack.hip: the projections of a run of decoder blocks at one token in a single cooperative launch
-struct StackLayer {  // one block: re-tiled weights and scales of q, k, v, o, gate, up, down (BITNET_HIP_PROJ_*)
-    const uint8_t *w[7];
-    const float *w_scale[7];
-};
-struct StackParams {
-    const StackLayer *table;  // [layers], device memory
-    int layer_begin, layer_end;
-    int step_begin, step_end;  // steps of the launch, 4 per block, counted from block layer_begin's first
-    const float *x_in;
-    float *x_out;
-    float *ring;              // [layers][ring_stride]: per block q | k | v | x1 | gate | up | x_next
-    int ring_stride;          // floats
-    float *q_last, *k_last;   // optional destinations of the last block's q and k
-    const float *gamma;       // [layers][2][hidden]
-    int hidden, ffn, kv_dim, head_dim, gqa_group;
-    float eps;
-    unsigned *flags;          // [grid] barrier flags, monotonic epochs
-    unsigned *abort_word;     // device; set when a workgroup gave up waiting
-    unsigned *host_status;    // host-mapped copy of the same fact
-    unsigned epoch0;          // epoch of the last barrier of the previous launch
-    long long spin_limit;
-    int lds_row_bytes;        // set by the launcher
-};
-bool decode_stack_supported(size_t hidden, size_t ffn, size_t kv_dim, size_t head_dim, int sum_order, int grid);
-size_t decode_stack_max_layers();  // blocks one launch can take
-size_t decode_stack_ring_stride(size_t hidden, size_t ffn, size_t kv_dim);
-int launch_decode_stack(const StackParams &params, int grid, hipStream_t stream);
 
 }  // namespace bitnet

@@ -161,6 +161,211 @@ __global__ __launch_bounds__(256) void ternarize_pack_kernel(const float *w, siz
     packed[b] = (uint8_t)byte;
 }
 
+// ---- BitNetWeightQuantizer::quantize, the reference's weight pipeline (bitnet-quant/src/quantization/weights.rs:568-611)
+//
+//   w' = (w - mean) / sqrt(var + 1e-8)                   normalize_before_quantize, :671-686
+//   w'' = clamp(w', mean' - t*mad, mean' + t*mad)        handle_outliers, :688-699 (mad = mean|w'|)
+//   thr by TernaryMethod from mean|w''| (and max|w''|)   :370-480
+//   q = sign(w'') * [|w''| > thr]                        apply_ternary_quantization, :482-496
+//   scale = sum(w''*q) / sum(q*q)                        compute_ternary_scale, :546-559
+//
+// Nothing but the packed codes and the scale is written: w'' is recomputed from w wherever it is needed (two
+// f32 operations and a clamp).  Every tensor-wide sum is carried in f64 in the order of the absmean kernels above
+// (per row: lane l adds columns l, l+64, ..., then the butterfly; the row sums the same way), so the f32 scalars
+// have the bits the CPU restatement of the same order has.  The scalars stay on the device in WqState; one
+// wavefront finishes each reduction and derives the next stage's scalars.
+struct WqState {
+    float mean, sd;            // normalisation (0, 1 when switched off)
+    float clip_mean, clip_mad; // centre and mean |.| of the normalised tensor
+    float lo, hi;              // clip bounds (-inf, +inf when switched off)
+    float mean_abs, max_abs;   // of the processed tensor
+    float thr;
+    float num, den, scale;
+};
+static_assert(sizeof(WqState) == 12 * sizeof(float), "stats are returned as 12 floats");
+
+enum WqPass { WQ_SUM = 0, WQ_SQDIFF, WQ_CLIP_STATS, WQ_ABS_STATS, WQ_OPTIMAL, WQ_SCALE };
+constexpr int WQ_MAX_ACC = 10;
+
+__device__ __forceinline__ float wq_normalised(float w, const WqState &st, bool normalize)
+{
+    return normalize ? f32_div(w - st.mean, st.sd) : w;
+}
+__device__ __forceinline__ float wq_processed(float w, const WqState &st, bool normalize, bool clip)
+{
+    float x = wq_normalised(w, st, normalize);
+    if (clip) {
+        x = x > st.hi ? st.hi : x;
+        x = x < st.lo ? st.lo : x;
+    }
+    return x;
+}
+__device__ __forceinline__ float wq_code(float x, float thr) { return x > thr ? 1.0f : (x < -thr ? -1.0f : 0.0f); }
+
+__constant__ float wq_factors[10] = {0.3f, 0.4f, 0.5f, 0.6f, 0.7f, 0.8f, 0.9f, 1.0f, 1.1f, 1.2f};
+
+// One wavefront per row; accumulator a of row r goes to row_sums[a * n + r] (and the row's max |.| to row_max[r]).
+template <int PASS>
+__global__ __launch_bounds__(256) void wq_rows_kernel(const float *w, size_t n, size_t k, const WqState *state, int normalize,
+                                                      int clip, double *row_sums, float *row_max)
+{
+    constexpr int NACC = PASS == WQ_OPTIMAL ? 10 : ((PASS == WQ_CLIP_STATS || PASS == WQ_SCALE) ? 2 : 1);
+    const int lane = threadIdx.x;
+    const size_t row = (size_t)blockIdx.x * blockDim.y + threadIdx.y;
+    if (row >= n) return;
+    const WqState st = *state;
+    const float *wr = w + row * k;
+    double acc[NACC];
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) acc[a] = 0.0;
+    float mx = 0.0f;
+    float cand[PASS == WQ_OPTIMAL ? 10 : 1];
+    if constexpr (PASS == WQ_OPTIMAL) {
+#pragma unroll
+        for (int f = 0; f < 10; ++f) cand[f] = f32_mul(st.mean_abs, wq_factors[f]);
+    }
+    for (size_t c = lane; c < k; c += 64) {
+        const float v = wr[c];
+        if constexpr (PASS == WQ_SUM) {
+            acc[0] = acc[0] + (double)v;
+        } else if constexpr (PASS == WQ_SQDIFF) {
+            const float d = v - st.mean;
+            acc[0] = acc[0] + (double)f32_mul(d, d);
+        } else if constexpr (PASS == WQ_CLIP_STATS) {
+            const float x = wq_normalised(v, st, normalize != 0);
+            acc[0] = acc[0] + (double)x;
+            acc[1] = acc[1] + (double)fabsf(x);
+        } else if constexpr (PASS == WQ_ABS_STATS) {
+            const float ax = fabsf(wq_processed(v, st, normalize != 0, clip != 0));
+            acc[0] = acc[0] + (double)ax;
+            mx = fmaxf(mx, ax);
+        } else if constexpr (PASS == WQ_OPTIMAL) {
+            const float x = wq_processed(v, st, normalize != 0, clip != 0);
+#pragma unroll
+            for (int f = 0; f < 10; ++f) {
+                const float d = x - wq_code(x, cand[f]);
+                acc[f] = acc[f] + (double)f32_mul(d, d);
+            }
+        } else {
+            const float x = wq_processed(v, st, normalize != 0, clip != 0);
+            const float q = wq_code(x, st.thr);
+            acc[0] = acc[0] + (double)f32_mul(x, q);
+            acc[1] = acc[1] + (double)f32_mul(q, q);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) {
+        const double s = wave_sum_f64(acc[a]);
+        if (lane == 0) row_sums[(size_t)a * n + row] = s;
+    }
+    if constexpr (PASS == WQ_ABS_STATS) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        if (lane == 0) row_max[row] = mx;
+    }
+}
+
+// One wavefront: combines the row sums of every accumulator (lane l takes rows l, l+64, ...; butterfly) and derives
+// the scalars of the next stage.  method: TernaryMethod 0..4; custom <= 0: the method's own factor.
+template <int PASS>
+__global__ __launch_bounds__(64) void wq_final_kernel(const double *row_sums, const float *row_max, size_t n, size_t k,
+                                                      WqState *state, int method, float outlier_threshold, float custom)
+{
+    constexpr int NACC = PASS == WQ_OPTIMAL ? 10 : ((PASS == WQ_CLIP_STATS || PASS == WQ_SCALE) ? 2 : 1);
+    const int lane = threadIdx.x;
+    double tot[NACC];
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) {
+        double s = 0.0;
+        for (size_t r = lane; r < n; r += 64) s = s + row_sums[(size_t)a * n + r];
+        tot[a] = wave_sum_f64(s);
+    }
+    float mx = 0.0f;
+    if constexpr (PASS == WQ_ABS_STATS) {
+        for (size_t r = lane; r < n; r += 64) mx = fmaxf(mx, row_max[r]);
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    }
+    if (lane != 0) return;
+    const double count = (double)n * (double)k;
+    WqState st = *state;
+    if constexpr (PASS == WQ_SUM) {
+        st.mean = (float)(tot[0] / count);
+    } else if constexpr (PASS == WQ_SQDIFF) {
+        const float var = (float)(tot[0] / count);
+        st.sd = f32_sqrt(var + 1e-8f);
+    } else if constexpr (PASS == WQ_CLIP_STATS) {
+        st.clip_mean = (float)(tot[0] / count);
+        st.clip_mad = (float)(tot[1] / count);
+        const float spread = f32_mul(outlier_threshold, st.clip_mad);
+        st.lo = st.clip_mean - spread;
+        st.hi = st.clip_mean + spread;
+    } else if constexpr (PASS == WQ_ABS_STATS) {
+        st.mean_abs = (float)(tot[0] / count);
+        st.max_abs = mx;
+        const bool has_custom = custom > 0.0f;
+        float thr;
+        if (method == 1) thr = f32_mul(st.mean_abs, has_custom ? custom : 0.8f);
+        else if (method == 2)
+            thr = has_custom ? f32_mul(st.mean_abs, custom)
+                             : (st.max_abs > f32_mul(3.0f, st.mean_abs) ? f32_mul(st.mean_abs, 0.5f) : f32_mul(st.mean_abs, 0.7f));
+        else thr = f32_mul(st.mean_abs, has_custom ? custom : 0.7f);  // mean, DetSTE; optimal without its search
+        st.thr = thr;
+    } else if constexpr (PASS == WQ_OPTIMAL) {
+        float best = __builtin_inff(), thr = f32_mul(st.mean_abs, 0.7f);
+#pragma unroll
+        for (int f = 0; f < 10; ++f) {
+            const float mse = (float)(tot[f] / count);
+            if (mse < best) { best = mse; thr = f32_mul(st.mean_abs, wq_factors[f]); }
+        }
+        st.thr = thr;
+    } else {
+        st.num = (float)tot[0];
+        st.den = (float)tot[1];
+        st.scale = fabsf(st.den) < 1.1920929e-07f ? 1.0f : f32_div(st.num, st.den);
+    }
+    *state = st;
+}
+
+__global__ void wq_init_kernel(WqState *state)
+{
+    WqState st;
+    st.mean = 0.0f; st.sd = 1.0f; st.clip_mean = 0.0f; st.clip_mad = 0.0f; st.lo = -__builtin_inff(); st.hi = __builtin_inff();
+    st.mean_abs = 0.0f; st.max_abs = 0.0f; st.thr = 0.0f; st.num = 0.0f; st.den = 0.0f; st.scale = 1.0f;
+    *state = st;
+}
+
+// Ternarise the processed tensor with the threshold found, pack; thread b builds byte b.  Also publishes the scale and
+// (optionally) the twelve scalars.
+__global__ __launch_bounds__(256) void wq_ternarize_pack_kernel(const float *w, size_t count, const WqState *state, int normalize,
+                                                                int clip, uint8_t *packed, int8_t *q_i8, size_t nbytes)
+{
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nbytes) return;
+    const WqState st = *state;
+    unsigned byte = 0;
+    for (int j = 0; j < 4; ++j) {
+        size_t i = 4 * b + j;
+        if (i < count) {
+            const int t = (int)wq_code(wq_processed(w[i], st, normalize != 0, clip != 0), st.thr);
+            if (q_i8) q_i8[i] = (int8_t)t;
+            byte |= ((unsigned)(t + 1) & 3u) << (2 * j);
+        }
+    }
+    packed[b] = (uint8_t)byte;
+}
+
+__global__ void wq_publish_kernel(const WqState *state, int clip, float *w_scale, float *stats)
+{
+    const WqState st = *state;
+    *w_scale = st.scale;
+    if (stats) {
+        const float v[12] = {st.mean, st.sd, st.clip_mean, st.clip_mad, clip ? st.lo : 0.0f, clip ? st.hi : 0.0f,
+                             st.mean_abs, st.max_abs, st.thr, st.num, st.den, st.scale};
+        for (int i = 0; i < 12; ++i) stats[i] = v[i];
+    }
+}
+
 __device__ __forceinline__ unsigned code_at(const uint8_t *packed, size_t e)
 {
     return (packed[e >> 2] >> (2 * (e & 3))) & 3u;
@@ -283,6 +488,52 @@ int launch_quantize_weights(const float *w, size_t n, size_t k, int method, floa
     hipLaunchKernelGGL(ternarize_pack_kernel, dim3(blocks_for(nbytes, 256)), dim3(256), 0, stream, w, count,
                        method, threshold_factor, w_scale, packed, q_i8, nbytes);
     BITNET_HIP_CHECK_LAUNCH("ternarize_pack_kernel");
+    return BITNET_HIP_OK;
+}
+
+size_t quantize_weights_reference_scratch_bytes(size_t n)
+{
+    return sizeof(double) * WQ_MAX_ACC * (n ? n : 1) + sizeof(float) * (n ? n : 1) + 256;
+}
+
+int launch_quantize_weights_reference(const float *w, size_t n, size_t k, int method, int normalize, float outlier_threshold,
+                                      float custom_factor, void *scratch, uint8_t *packed, float *w_scale, int8_t *q_i8,
+                                      float *stats, hipStream_t stream)
+{
+    // scratch: WqState (256 bytes reserved), then WQ_MAX_ACC * n doubles, then n floats
+    WqState *state = static_cast<WqState *>(scratch);
+    double *row_sums = reinterpret_cast<double *>(static_cast<uint8_t *>(scratch) + 256);
+    float *row_max = reinterpret_cast<float *>(row_sums + WQ_MAX_ACC * (n ? n : 1));
+    const int clip = outlier_threshold > 0.0f ? 1 : 0;
+    hipLaunchKernelGGL(wq_init_kernel, dim3(1), dim3(1), 0, stream, state);
+    BITNET_HIP_CHECK_LAUNCH("wq_init_kernel");
+    const size_t count = n * k, nbytes = (count + 3) / 4;
+    if (count != 0) {
+        const dim3 rgrid(blocks_for(n, 4)), rblock(64, 4);
+#define BITNET_WQ_PASS(PASS)                                                                                              \
+    do {                                                                                                                  \
+        hipLaunchKernelGGL((wq_rows_kernel<PASS>), rgrid, rblock, 0, stream, w, n, k, state, normalize, clip, row_sums,  \
+                           row_max);                                                                                      \
+        BITNET_HIP_CHECK_LAUNCH("wq_rows_kernel");                                                                        \
+        hipLaunchKernelGGL((wq_final_kernel<PASS>), dim3(1), dim3(64), 0, stream, row_sums, row_max, n, k, state, method, \
+                           outlier_threshold, custom_factor);                                                             \
+        BITNET_HIP_CHECK_LAUNCH("wq_final_kernel");                                                                       \
+    } while (0)
+        if (normalize) {
+            BITNET_WQ_PASS(WQ_SUM);
+            BITNET_WQ_PASS(WQ_SQDIFF);
+        }
+        if (clip) BITNET_WQ_PASS(WQ_CLIP_STATS);
+        BITNET_WQ_PASS(WQ_ABS_STATS);
+        if (method == 3 && !(custom_factor > 0.0f)) BITNET_WQ_PASS(WQ_OPTIMAL);
+        BITNET_WQ_PASS(WQ_SCALE);
+#undef BITNET_WQ_PASS
+        hipLaunchKernelGGL(wq_ternarize_pack_kernel, dim3(blocks_for(nbytes, 256)), dim3(256), 0, stream, w, count, state,
+                           normalize, clip, packed, q_i8, nbytes);
+        BITNET_HIP_CHECK_LAUNCH("wq_ternarize_pack_kernel");
+    }
+    hipLaunchKernelGGL(wq_publish_kernel, dim3(1), dim3(1), 0, stream, state, clip, w_scale, stats);
+    BITNET_HIP_CHECK_LAUNCH("wq_publish_kernel");
     return BITNET_HIP_OK;
 }
 

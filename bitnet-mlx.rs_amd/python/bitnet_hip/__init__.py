@@ -41,6 +41,11 @@ LAYOUT_OUT_IN = 0
 LAYOUT_IN_OUT = 1
 TERNARY_ABSMEAN_ROUNDCLIP = 0
 TERNARY_MEAN_THRESHOLD = 1
+TERNARY_REF_MEAN_THRESHOLD = 2
+TERNARY_REF_MEDIAN_THRESHOLD = 3
+TERNARY_REF_ADAPTIVE_THRESHOLD = 4
+TERNARY_REF_OPTIMAL_THRESHOLD = 5
+TERNARY_REF_DETSTE = 6
 INPUT_PLAIN = 0
 INPUT_RELU2_MUL = 1
 INPUT_GQA_BROADCAST = 2
@@ -92,6 +97,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_pack_ternary_base3": (i32, [vp, sz, vp, vp]),
         "bitnet_hip_unpack_ternary_base3": (i32, [vp, sz, vp, vp]),
         "bitnet_hip_quantize_weights": (i32, [vp, sz, sz, i32, f32, vp, vp, vp, vp]),
+        "bitnet_hip_quantize_weights_reference": (i32, [vp, sz, sz, i32, i32, f32, f32, vp, vp, vp, vp, vp]),
         "bitnet_hip_tiled_size": (sz, [sz, sz]),
         "bitnet_hip_retile_weights": (i32, [vp, sz, sz, i32, vp, vp]),
         "bitnet_hip_untile_weights": (i32, [vp, sz, sz, vp, vp]),
@@ -113,7 +119,6 @@ def load_library() -> C.CDLL:
         "bitnet_hip_bitlinear_forward_multi": (i32, [C.POINTER(vp), sz, vp, sz, vp, f32, i32, C.POINTER(vp), vp, sz, vp]),
         "bitnet_hip_bitlinear_matmul": (i32, [vp, vp, vp, sz, vp, vp, vp, vp, vp]),
         "bitnet_hip_decoder_decode_layers": (i32, [vp, sz, sz, vp, sz, vp, vp, vp, vp]),
-        "bitnet_hip_decoder_set_single_launch": (i32, [vp, i32]),
         "bitnet_hip_decoder_create": (i32, [sz, sz, sz, sz, sz, sz, f32, i32, sz, C.POINTER(vp)]),
         "bitnet_hip_decoder_destroy": (None, [vp]),
         "bitnet_hip_decoder_projection": (i32, [vp, sz, i32, C.POINTER(vp)]),
@@ -286,6 +291,75 @@ def quantize_weights(w: torch.Tensor, method: int = TERNARY_ABSMEAN_ROUNDCLIP, t
     _check(load_library().bitnet_hip_quantize_weights(_ptr(w), n, k, method, threshold_factor, _ptr(packed),
                                                       _ptr(w_scale), _ptr(q), _stream(stream)))
     return packed, w_scale, q
+
+
+class TernaryMethod:
+    """TernaryMethod (bitnet-quant/src/quantization/weights.rs:17-30)."""
+    MeanThreshold, MedianThreshold, AdaptiveThreshold, OptimalThreshold, DetSTE = range(5)
+
+
+@dataclass
+class WeightQuantizationConfig:
+    """The fields of WeightQuantizationConfig (weights.rs:58-95) that affect arithmetic, with its defaults."""
+    normalize_weights: bool = True
+    outlier_threshold: float = 3.0
+    ternary_method: int = TernaryMethod.MeanThreshold
+    custom_threshold_factor: Optional[float] = None
+
+    def validate(self):
+        """WeightQuantizationConfig::validate (weights.rs:120-150)."""
+        if self.outlier_threshold < 0.0:
+            raise BitLinearError(INVALID_CONFIG, "Outlier threshold cannot be negative")
+        f = self.custom_threshold_factor
+        if f is not None and (f <= 0.0 or f > 2.0):
+            raise BitLinearError(INVALID_CONFIG, "Custom threshold factor must be in range (0, 2]")
+
+
+WQ_STATS = ("mean", "sd", "clip_mean", "clip_mad", "lo", "hi", "mean_abs", "max_abs", "threshold", "num", "den", "scale")
+
+
+@dataclass
+class QuantizedWeight:
+    """QuantizedWeight (weights.rs:158-175): ternary values (int8, the reference stores them as f32 in a tensor),
+    the scalar scale, the original shape; plus the packed bytes the BitLinear layer takes."""
+    values: torch.Tensor
+    scales: torch.Tensor
+    original_shape: tuple
+    packed: torch.Tensor
+    stats: dict
+
+
+class BitNetWeightQuantizer:
+    """BitNetWeightQuantizer (weights.rs:341-611): quantize / dequantize on the GPU."""
+
+    def __init__(self, config: Optional[WeightQuantizationConfig] = None):
+        self.config = config or WeightQuantizationConfig()
+        self.config.validate()
+
+    def validate_input(self, weights: torch.Tensor):
+        """weights.rs:625-639."""
+        if weights.dim() < 2:
+            raise BitLinearError(QUANTIZATION_ERROR, "Weight tensor must have at least 2 dimensions")
+        if weights.dtype != torch.float32:
+            raise BitLinearError(QUANTIZATION_ERROR, "Weight tensor must be float type")
+
+    def quantize(self, weights: torch.Tensor, stream=None) -> QuantizedWeight:
+        self.validate_input(weights)
+        _dev(weights, torch.float32, "weights")
+        n, k = weights.shape[0], weights.numel() // weights.shape[0]
+        packed = torch.empty((packed_size(n * k),), dtype=torch.uint8, device=weights.device)
+        w_scale = torch.empty((1,), dtype=torch.float32, device=weights.device)
+        q = torch.empty(weights.shape, dtype=torch.int8, device=weights.device)
+        stats = torch.empty((12,), dtype=torch.float32, device=weights.device)
+        c = self.config
+        _check(load_library().bitnet_hip_quantize_weights_reference(
+            _ptr(weights), n, k, c.ternary_method, int(c.normalize_weights), c.outlier_threshold,
+            c.custom_threshold_factor or 0.0, _ptr(packed), _ptr(w_scale), _ptr(q), _ptr(stats), _stream(stream)))
+        return QuantizedWeight(q, w_scale, tuple(weights.shape), packed, dict(zip(WQ_STATS, stats.cpu().tolist())))
+
+    def dequantize(self, quantized: QuantizedWeight) -> torch.Tensor:
+        """weights.rs:616-619: values * scales (a host-side convenience through torch; not on the forward path)."""
+        return quantized.values.to(torch.float32) * quantized.scales
 
 
 def retile_weights(packed: torch.Tensor, n: int, k: int, layout: int = LAYOUT_OUT_IN, stream=None) -> torch.Tensor:
@@ -620,14 +694,6 @@ class DecoderProjections:
 
     def weight_bytes(self) -> int:
         return load_library().bitnet_hip_decoder_weight_bytes(self._h)
-
-    def set_single_launch(self, enabled: bool) -> bool:
-        """Turn the one-cooperative-launch path for one-token decode on or off (default off); returns whether this
-        decoder has it."""
-        rc = load_library().bitnet_hip_decoder_set_single_launch(self._h, int(enabled))
-        if rc < 0:
-            _check(-rc)
-        return rc == 1
 
     def decode(self, x: torch.Tensor, out: Optional[torch.Tensor] = None, want_qk: bool = False, stream=None,
                layers: Optional[Sequence[int]] = None):

@@ -29,6 +29,11 @@ pub const BITNET_HIP_LAYOUT_OUT_IN: c_int = 0;
 pub const BITNET_HIP_LAYOUT_IN_OUT: c_int = 1;
 pub const BITNET_HIP_TERNARY_ABSMEAN_ROUNDCLIP: c_int = 0;
 pub const BITNET_HIP_TERNARY_MEAN_THRESHOLD: c_int = 1;
+pub const BITNET_HIP_TERNARY_REF_MEAN_THRESHOLD: c_int = 2;
+pub const BITNET_HIP_TERNARY_REF_MEDIAN_THRESHOLD: c_int = 3;
+pub const BITNET_HIP_TERNARY_REF_ADAPTIVE_THRESHOLD: c_int = 4;
+pub const BITNET_HIP_TERNARY_REF_OPTIMAL_THRESHOLD: c_int = 5;
+pub const BITNET_HIP_TERNARY_REF_DETSTE: c_int = 6;
 pub const BITNET_HIP_INPUT_PLAIN: c_int = 0;
 pub const BITNET_HIP_INPUT_RELU2_MUL: c_int = 1;
 pub const BITNET_HIP_INPUT_GQA_BROADCAST: c_int = 2;
@@ -55,6 +60,10 @@ extern "C" {
     pub fn bitnet_hip_unpack_ternary_base3(packed: *const u8, count: usize, q: *mut i8, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_quantize_weights(w: *const f32, n: usize, k: usize, method: c_int, threshold_factor: f32,
                                        packed: *mut u8, w_scale: *mut f32, q_i8: *mut i8, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_quantize_weights_reference(w: *const f32, n: usize, k: usize, ternary_method: c_int,
+                                                 normalize_weights: c_int, outlier_threshold: f32,
+                                                 custom_threshold_factor: f32, packed: *mut u8, w_scale: *mut f32,
+                                                 q_i8: *mut i8, stats: *mut f32, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_tiled_size(n: usize, k: usize) -> usize;
     pub fn bitnet_hip_retile_weights(packed: *const u8, n: usize, k: usize, layout: c_int, tiled: *mut u8,
                                      stream: *mut c_void) -> c_int;
@@ -117,5 +126,4 @@ extern "C" {
     pub fn bitnet_hip_decoder_decode_layers(dec: *mut bitnet_hip_decoder, layer_begin: usize, layer_end: usize,
                                             x_in: *const f32, m: usize, x_out: *mut f32, q_last: *mut f32,
                                             k_last: *mut f32, stream: *mut c_void) -> c_int;
-    pub fn bitnet_hip_decoder_set_single_launch(dec: *mut bitnet_hip_decoder, enabled: c_int) -> c_int;
 }

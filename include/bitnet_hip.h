@@ -54,6 +54,16 @@ typedef enum bitnet_hip_status {
 #define BITNET_HIP_TERNARY_MEAN_THRESHOLD 1    /* q = sign(w) * [|w| > factor * mean|w|], scale = mean|W|
                                                   (bitnet-quant/src/simd/ternary.rs:27-41,87-101) */
 
+/* BitNetWeightQuantizer::quantize (weights.rs:568-611) with WeightQuantizationConfig's defaults (normalise, clip
+ * at 3.0 mean|w|, :81-95) and one of the five TernaryMethods (:17-30); threshold_factor is then
+ * custom_threshold_factor (<= 0: none, the method's own factor).  bitnet_hip_quantize_weights_reference takes the
+ * whole configuration. */
+#define BITNET_HIP_TERNARY_REF_MEAN_THRESHOLD 2     /* TernaryMethod::MeanThreshold: BitLinear's default (layer.rs:53-63) */
+#define BITNET_HIP_TERNARY_REF_MEDIAN_THRESHOLD 3   /* TernaryMethod::MedianThreshold */
+#define BITNET_HIP_TERNARY_REF_ADAPTIVE_THRESHOLD 4 /* TernaryMethod::AdaptiveThreshold */
+#define BITNET_HIP_TERNARY_REF_OPTIMAL_THRESHOLD 5  /* TernaryMethod::OptimalThreshold */
+#define BITNET_HIP_TERNARY_REF_DETSTE 6             /* TernaryMethod::DetSTE */
+
 /* Input transform fused in front of the activation quantiser. */
 #define BITNET_HIP_INPUT_PLAIN 0     /* row = x[m, :] */
 #define BITNET_HIP_INPUT_RELU2_MUL 1 /* row = x2[m, :] * relu(x[m, :])^2   (x = gate, x2 = up):
@@ -135,10 +145,25 @@ int bitnet_hip_unpack_ternary_base3(const uint8_t *packed, size_t count, int8_t 
 /* Ternarise an f32 weight matrix [n, k] (row-major) and pack it in the reference's byte format.
  *   replaces SimdTernaryOps::{compute_absmean, quantize_batch} (bitnet-quant/src/simd/ternary.rs:27-66)
  *   / BitNetWeightQuantizer::quantize (bitnet-quant/src/quantization/weights.rs:568-611) + the packer.
- *   method   BITNET_HIP_TERNARY_*;  threshold_factor only for MEAN_THRESHOLD (reference: 0.5 / 0.7)
+ *   method   BITNET_HIP_TERNARY_*;  threshold_factor: MEAN_THRESHOLD's factor (reference: 0.5 / 0.7), the custom
+ *            factor of the REF_* methods (<= 0: none), unused for ABSMEAN_ROUNDCLIP
  *   packed   [(n*k+3)/4] u8 out;  w_scale  1 f32 out (device);  q_i8 [n*k] int8 out or NULL. */
 int bitnet_hip_quantize_weights(const float *w, size_t n, size_t k, int method, float threshold_factor,
                                 uint8_t *packed, float *w_scale, int8_t *q_i8, void *stream);
+
+/* The reference's weight pipeline with its whole configuration, on the GPU:
+ *   replaces BitNetWeightQuantizer::quantize (bitnet-quant/src/quantization/weights.rs:568-611):
+ *   normalize_before_quantize (:671-686, if normalize_weights), handle_outliers (:688-699, if outlier_threshold > 0),
+ *   quantize_ternary_with_method (:370-480; ternary_method 0 MeanThreshold, 1 MedianThreshold, 2 AdaptiveThreshold,
+ *   3 OptimalThreshold, 4 DetSTE; custom_threshold_factor <= 0 means None), apply_ternary_quantization (:482-496),
+ *   compute_ternary_scale (:546-559).  INVALID_CONFIG where WeightQuantizationConfig::validate errs (:120-150).
+ *   w [n, k] f32;  packed [(n*k+3)/4] u8 out (codes q + 1);  w_scale 1 f32 out: sum(w''q)/sum(q q);  q_i8 [n*k] or NULL;
+ *   stats 12 f32 out or NULL: mean, sd, clip centre, clip mean|.|, lo, hi, mean|w''|, max|w''|, threshold, numerator,
+ *   denominator, scale.  Tensor-wide sums are carried in f64 in a fixed order (per row 64 strided partials and a
+ *   butterfly, then the rows likewise); the reference sums in f32 in candle-core's order. */
+int bitnet_hip_quantize_weights_reference(const float *w, size_t n, size_t k, int ternary_method, int normalize_weights,
+                                          float outlier_threshold, float custom_threshold_factor, uint8_t *packed,
+                                          float *w_scale, int8_t *q_i8, float *stats, void *stream);
 
 /* Device layout both contraction kernels stream: tiles of 16 rows x 256 columns, 1 KiB each, stored
  * [row_block][k_tile]; inside a tile the 16 bytes at offset 16*(16*kq + r) hold row r's columns
@@ -303,7 +328,9 @@ int bitnet_hip_decoder_set_norm(bitnet_hip_decoder *dec, size_t layer, int which
                                 int on_device, void *stream);
 /* Packed-weight bytes one decode step streams (sum of n*k/4 over all projections). */
 size_t bitnet_hip_decoder_weight_bytes(const bitnet_hip_decoder *dec);
-/* One decode step: x_in [m, hidden] -> x_out [m, hidden] through all blocks.  q_last / k_last (may be
+/* One decode step: x_in [m, hidden] -> x_out [m, hidden] through all blocks.  A decoder owns one set of activation
+ * buffers: its decode calls are serialised (a call on another stream waits, on the GPU, for the one before it); use one
+ * decoder per concurrent sequence group.  q_last / k_last (may be
  * NULL) receive the last block's q [m, hidden] and k [m, kv_heads*head_dim] projections. */
 int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t m, float *x_out,
                               float *q_last, float *k_last, void *stream);
@@ -311,18 +338,6 @@ int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t
 int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin, size_t layer_end,
                                      const float *x_in, size_t m, float *x_out, float *q_last, float *k_last,
                                      void *stream);
-/* Optional at one token: the blocks' projections as ONE cooperative launch with barriers across the grid in
- * place of launch boundaries (same results, bit for bit), for shapes that fit and up to 32 blocks per call.  Off
- * by default: on MI355X a barrier across the eight XCDs costs about what a kernel boundary costs, so the path
- * only matches the launch-per-group one (about 5 % faster over a 30-block stack, slower for single blocks
- * because a cooperative launch is dearer to start).  It is ignored with more than one token and while the
- * stream is being captured into a graph.  enabled = 1 turns it on, 0 off.  Returns 1 if the path is available
- * for this decoder, 0 if not, a negative status on error.  A wait at a grid barrier that exceeds 50 ms is
- * abandoned by every workgroup; the next decode call on the decoder then fails with BITNET_HIP_KERNEL_ERROR.
- * (The reference runs its blocks layer by layer, bitnet-inference/src/engine/transformer_layers.rs:626-710; this
- * switch only selects how the same work is issued.) */
-int bitnet_hip_decoder_set_single_launch(bitnet_hip_decoder *dec, int enabled);
-
 #ifdef __cplusplus
 }
 #endif

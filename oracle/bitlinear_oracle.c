@@ -25,10 +25,15 @@
  *                                        rows, one-hot rows), scale equivariance and an f64 bound; the
  *                                        bits of the ORC_SUM_BLOCK256 order are a declaration of this build
  *   orc_epilogue                         two IEEE f32 operations; closed form
- *   orc_quantize_weights_reference       PARITY UNPINNED for the f32 statistics: the reference computes
- *                                        mean/sum with candle-core 0.8 (third party, not vendored), whose
- *                                        summation order is not visible; this restatement accumulates in
- *                                        f64.  Ternary values are pinned by the threshold tests.
+ *   orc_quantize_weights_reference       the reference's tests for it are property tests (ternary values, positive
+ *                                        scale, determinism): pinned by those, by what each stage must satisfy
+ *                                        (mean 0 / variance 1 after normalising, the clip bounds attained exactly
+ *                                        by the clipped elements, the strict threshold, the least-squares scale,
+ *                                        each method's factor and the argmin of the ten candidates) and by an
+ *                                        independent f64 numpy model with one case per branch that a swapped
+ *                                        stage order or a wrong bound fails.  The last bit of its f32 scalars
+ *                                        (candle-core 0.8 sums, third party, not vendored, order not visible)
+ *                                        is a declaration of this build: sums are carried in f64 in a stated order.
  */
 #include <math.h>
 #include <stddef.h>
@@ -244,56 +249,130 @@ void orc_dequantize_ternary(const int8_t *q, size_t n, float scale, float *out)
     for (size_t i = 0; i < n; ++i) out[i] = q[i] == 1 ? scale : (q[i] == -1 ? -scale : 0.0f);
 }
 
-/* The reference's default BitLinear weight recipe.
- *   reference: bitnet-quant/src/quantization/weights.rs:568-611 with
- *     normalize_before_quantize :671-686   (w - mean) / sqrt(var + 1e-8)
- *     handle_outliers           :688-699   clamp to mean' +- t * mean|w'|   (t = outlier_threshold)
- *     mean-threshold ternarise  :384-394   thr = factor * mean|w''|, strict '>' (:482-496)
- *     compute_ternary_scale     :546-559   sum(w''*q) / sum(q*q), 1.0 if the denominator < f32::EPSILON
- * Statistics are accumulated sequentially in f64 and rounded to f32 where the reference holds an f32
- * scalar (candle's own order is not visible: parity unpinned for those scalars). */
-float orc_quantize_weights_reference(const float *w, size_t n, int normalize, float outlier_threshold,
-                                     float threshold_factor, int8_t *q, float *processed /* n, scratch */)
+/* Sum of an f32 tensor viewed as [rows, cols], carried in f64 in the order orc_absmean declares: per row,
+ * lane l (of 64) adds columns l, l+64, ... in ascending order, the 64 partials meet in the butterfly
+ * off = 32..1; the row sums are combined the same way (lane l takes rows l, l+64, ...). */
+static double orc_tensor_sum_f64(const float *v, size_t rows, size_t cols)
 {
-    if (n == 0) return 1.0f;
+    double *row_sum = (double *)malloc(sizeof(double) * (rows ? rows : 1));
+    double *tmp = (double *)malloc(sizeof(double) * (cols ? cols : 1));
+    for (size_t r = 0; r < rows; ++r) {
+        for (size_t c = 0; c < cols; ++c) tmp[c] = (double)v[r * cols + c];
+        row_sum[r] = orc_wave64_sum_f64(tmp, cols);
+    }
+    double total = orc_wave64_sum_f64(row_sum, rows);
+    free(tmp);
+    free(row_sum);
+    return total;
+}
+
+/* BitNetWeightQuantizer::quantize: the reference's weight pipeline with its five TernaryMethods.
+ *   reference: bitnet-quant/src/quantization/weights.rs:568-611 with
+ *     normalize_before_quantize :671-686   (w - mean) / sqrt(var + 1e-8), var = mean((w - mean)^2)
+ *     handle_outliers           :688-699   clamp to mean' +- t * mean|w'|   (t = outlier_threshold, skipped if 0)
+ *     quantize_ternary_with_method :370-480:
+ *       0 MeanThreshold      thr = mean|w''| * (custom or 0.7)                                  (:384-394)
+ *       1 MedianThreshold    thr = mean|w''| * (custom or 0.8)   (the "median" is a mean, :397-408)
+ *       2 AdaptiveThreshold  thr = mean|w''| * custom, or mean|w''| * (max|w''| > 3 mean|w''| ? 0.5 : 0.7)  (:411-436)
+ *       3 OptimalThreshold   thr = mean|w''| * custom, or the first of mean|w''| * {0.3 .. 1.2} with the smallest
+ *                            mean((w'' - q)^2), compared with '<' (:439-468)
+ *       4 DetSTE             thr = mean|w''| * (custom or 0.7)                                  (:471-479)
+ *     apply_ternary_quantization :482-496  q = sign(w'') * [|w''| > thr]  (strict)
+ *     compute_ternary_scale     :546-559   sum(w''*q) / sum(q*q), 1.0 if |denominator| < f32::EPSILON
+ *   custom_factor <= 0 means None.  Defaults of WeightQuantizationConfig (:81-95): normalize, t = 3.0, no custom factor.
+ * Every element-wise step is one f32 operation; every tensor-wide sum is carried in f64 in the order of
+ * orc_tensor_sum_f64 and rounded to f32 where the reference holds an f32 scalar (the reference's own sums are
+ * candle-core's, whose order is not visible: the f32 bits of these scalars are this build's declaration).
+ * processed (rows*cols floats) receives w''; stats (12 floats, may be NULL) receives mean, sd, clip centre,
+ * clip mad, lo, hi, mean|w''|, max|w''|, thr, numerator, denominator, scale. */
+float orc_quantize_weights_reference(const float *w, size_t rows, size_t cols, int method, int normalize,
+                                     float outlier_threshold, float custom_factor, int8_t *q, float *processed,
+                                     float *stats)
+{
+    const size_t n = rows * cols;
+    float st[12] = {0.0f, 1.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 1.0f};
+    if (n == 0) {
+        if (stats) memcpy(stats, st, sizeof st);
+        return 1.0f;
+    }
+    float *tmp = (float *)malloc(sizeof(float) * n);
     for (size_t i = 0; i < n; ++i) processed[i] = w[i];
     if (normalize) {
-        double s = 0.0;
-        for (size_t i = 0; i < n; ++i) s += processed[i];
-        float mean = (float)(s / (double)n);
-        double v = 0.0;
+        float mean = (float)(orc_tensor_sum_f64(processed, rows, cols) / (double)n);
         for (size_t i = 0; i < n; ++i) {
             float d = processed[i] - mean;
-            v += (double)(d * d);
+            tmp[i] = d * d;
         }
-        float var = (float)(v / (double)n);
+        float var = (float)(orc_tensor_sum_f64(tmp, rows, cols) / (double)n);
         float sd = sqrtf(var + 1e-8f);
-        for (size_t i = 0; i < n; ++i) processed[i] = (processed[i] - mean) / sd;
+        for (size_t i = 0; i < n; ++i) {
+            float d = processed[i] - mean;
+            processed[i] = d / sd;
+        }
+        st[0] = mean; st[1] = sd;
     }
     if (outlier_threshold > 0.0f) {
-        double s = 0.0, a = 0.0;
-        for (size_t i = 0; i < n; ++i) { s += processed[i]; a += fabsf(processed[i]); }
-        float mean = (float)(s / (double)n);
-        float mad = (float)(a / (double)n);
-        float lo = mean - outlier_threshold * mad, hi = mean + outlier_threshold * mad;
+        float mean = (float)(orc_tensor_sum_f64(processed, rows, cols) / (double)n);
+        for (size_t i = 0; i < n; ++i) tmp[i] = fabsf(processed[i]);
+        float mad = (float)(orc_tensor_sum_f64(tmp, rows, cols) / (double)n);
+        float spread = outlier_threshold * mad;
+        float lo = mean - spread, hi = mean + spread;
         for (size_t i = 0; i < n; ++i) {
             float t = processed[i];
-            processed[i] = t < lo ? lo : (t > hi ? hi : t);
+            t = t > hi ? hi : t;  /* candle clamp: min with the upper bound, then max with the lower */
+            t = t < lo ? lo : t;
+            processed[i] = t;
         }
+        st[2] = mean; st[3] = mad; st[4] = lo; st[5] = hi;
     }
-    double a = 0.0;
-    for (size_t i = 0; i < n; ++i) a += fabsf(processed[i]);
-    float mean_abs = (float)(a / (double)n);
-    float thr = mean_abs * threshold_factor;
-    orc_ternarize_threshold(processed, n, thr, q);
-    double num = 0.0, den = 0.0;
+    float max_abs = 0.0f;
     for (size_t i = 0; i < n; ++i) {
-        num += (double)(processed[i] * (float)q[i]);
-        den += (double)((float)q[i] * (float)q[i]);
+        tmp[i] = fabsf(processed[i]);
+        max_abs = fmaxf(max_abs, tmp[i]);
     }
-    float fnum = (float)num, fden = (float)den;
-    if (fabsf(fden) < 1.1920929e-07f) return 1.0f;
-    return fnum / fden;
+    float mean_abs = (float)(orc_tensor_sum_f64(tmp, rows, cols) / (double)n);
+    st[6] = mean_abs; st[7] = max_abs;
+    float thr;
+    const int custom = custom_factor > 0.0f;
+    switch (method) {
+        case 1: thr = mean_abs * (custom ? custom_factor : 0.8f); break;
+        case 2:
+            if (custom) thr = mean_abs * custom_factor;
+            else thr = max_abs > 3.0f * mean_abs ? mean_abs * 0.5f : mean_abs * 0.7f;
+            break;
+        case 3:
+            if (custom) {
+                thr = mean_abs * custom_factor;
+            } else {
+                static const float factors[10] = {0.3f, 0.4f, 0.5f, 0.6f, 0.7f, 0.8f, 0.9f, 1.0f, 1.1f, 1.2f};
+                float best_err = INFINITY;
+                thr = mean_abs * 0.7f;
+                for (int f = 0; f < 10; ++f) {
+                    float cand = mean_abs * factors[f];
+                    for (size_t i = 0; i < n; ++i) {
+                        float v = processed[i];
+                        float qv = v > cand ? 1.0f : (v < -cand ? -1.0f : 0.0f);
+                        float d = v - qv;
+                        tmp[i] = d * d;
+                    }
+                    float mse = (float)(orc_tensor_sum_f64(tmp, rows, cols) / (double)n);
+                    if (mse < best_err) { best_err = mse; thr = cand; }
+                }
+            }
+            break;
+        default: thr = mean_abs * (custom ? custom_factor : 0.7f); break;  /* MeanThreshold, DetSTE */
+    }
+    st[8] = thr;
+    orc_ternarize_threshold(processed, n, thr, q);
+    for (size_t i = 0; i < n; ++i) tmp[i] = processed[i] * (float)q[i];
+    float fnum = (float)orc_tensor_sum_f64(tmp, rows, cols);
+    for (size_t i = 0; i < n; ++i) tmp[i] = (float)q[i] * (float)q[i];
+    float fden = (float)orc_tensor_sum_f64(tmp, rows, cols);
+    free(tmp);
+    float scale = fabsf(fden) < 1.1920929e-07f ? 1.0f : fnum / fden;
+    st[9] = fnum; st[10] = fden; st[11] = scale;
+    if (stats) memcpy(stats, st, sizeof st);
+    return scale;
 }
 
 /* ------------------------------------------------------------------------------------------------

@@ -138,12 +138,25 @@ def quantize_weights_absmean(w):
     return ternarize_roundclip(w, s), s
 
 
-def quantize_weights_reference(w, normalize=True, outlier_threshold=3.0, threshold_factor=0.7):
+METHOD_MEAN, METHOD_MEDIAN, METHOD_ADAPTIVE, METHOD_OPTIMAL, METHOD_DETSTE = range(5)
+WQ_STATS = ("mean", "sd", "clip_mean", "clip_mad", "lo", "hi", "mean_abs", "max_abs", "threshold", "num", "den", "scale")
+
+
+def quantize_weights_reference(w, method=METHOD_MEAN, normalize=True, outlier_threshold=3.0, custom_factor=None,
+                               want_details=False):
+    """BitNetWeightQuantizer::quantize (weights.rs:568-611) on a 2-D f32 tensor; custom_factor None = method default.
+    Returns (q, scale), or (q, scale, processed, stats dict) with want_details."""
     w = _f32(w)
+    assert w.ndim == 2
     q = np.empty(w.shape, dtype=np.int8)
-    scratch = np.empty(w.size, dtype=np.float32)
-    s = lib().orc_quantize_weights_reference(_p(w), _sz(w.size), C.c_int(int(normalize)), C.c_float(outlier_threshold),
-                                             C.c_float(threshold_factor), _p(q), _p(scratch))
+    processed = np.empty(w.shape, dtype=np.float32)
+    stats = np.zeros(12, dtype=np.float32)
+    s = lib().orc_quantize_weights_reference(_p(w), _sz(w.shape[0]), _sz(w.shape[1]), C.c_int(int(method)),
+                                             C.c_int(int(normalize)), C.c_float(outlier_threshold),
+                                             C.c_float(custom_factor if custom_factor else 0.0), _p(q), _p(processed),
+                                             _p(stats))
+    if want_details:
+        return q, np.float32(s), processed, dict(zip(WQ_STATS, stats))
     return q, np.float32(s)
 
 

@@ -110,6 +110,56 @@ def test_quantize_weights_reference_vectors():
     assert host(s)[0] == 0.0 and not host(q).any()
 
 
+@pytest.mark.parametrize("method", range(5))
+@pytest.mark.parametrize("normalize,t,custom", [(True, 3.0, None), (False, 0.0, None), (True, 0.0, 0.45), (False, 2.0, None)])
+def test_reference_weight_pipeline_bit_exact(method, normalize, t, custom):
+    """BitNetWeightQuantizer::quantize with each TernaryMethod: ternary values, packed bytes, the scale and all twelve
+    f32 scalars of the pipeline equal to the oracle's, bit for bit (stated bar: q exact, scale within 1e-6 relative)."""
+    rng = np.random.default_rng(method * 10 + int(normalize) + int(t))
+    for n, k in ((48, 200), (5, 7), (640, 2560)):
+        w = (0.3 + 1.7 * rng.standard_normal((n, k))).astype(f32)
+        w[rng.random(w.shape) < 0.01] *= f32(6.0)
+        cfg = bh.WeightQuantizationConfig(normalize_weights=normalize, outlier_threshold=t, ternary_method=method,
+                                          custom_threshold_factor=custom)
+        got = bh.BitNetWeightQuantizer(cfg).quantize(dev(w))
+        q_ref, s_ref, _, st_ref = orc.quantize_weights_reference(w, method=method, normalize=normalize, outlier_threshold=t,
+                                                                 custom_factor=custom, want_details=True)
+        assert np.array_equal(host(got.values), q_ref)
+        assert np.array_equal(host(got.packed), orc.pack_2bit(q_ref))
+        assert abs(float(host(got.scales)[0]) - float(s_ref)) <= 1e-6 * abs(float(s_ref))
+        assert host(got.scales)[0] == s_ref
+        for name, v in st_ref.items():
+            assert f32(got.stats[name]) == v, (name, got.stats[name], v)
+
+
+def test_reference_weight_pipeline_through_the_layer():
+    """BitLinear with the reference's default quantiser (MeanThreshold, normalise, clip 3.0: layer.rs:53-63): the layer then
+    holds the oracle's codes and scale, and forward follows from them."""
+    rng = np.random.default_rng(21)
+    n, k = 96, 512
+    w = synth_weights(rng, n, k)
+    for method, factor in ((bh.TERNARY_REF_MEAN_THRESHOLD, 0.0), (bh.TERNARY_REF_OPTIMAL_THRESHOLD, 0.0),
+                           (bh.TERNARY_REF_ADAPTIVE_THRESHOLD, 0.0), (bh.TERNARY_REF_DETSTE, 0.9)):
+        layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n, ternary_method=method, threshold_factor=factor), "ref")
+        layer.update_weights(dev(w))
+        q_ref, s_ref = orc.quantize_weights_reference(w, method=method - bh.TERNARY_REF_MEAN_THRESHOLD,
+                                                      custom_factor=factor or None)
+        packed, ws = layer.get_quantized_weights()
+        assert ws == s_ref and np.array_equal(packed.numpy(), orc.pack_2bit(q_ref))
+        x = synth_activations(rng, 3, k)
+        ref = orc.bitlinear_forward(x, orc.pack_2bit(q_ref), n, float(s_ref))[0]
+        assert np.array_equal(host(layer.forward(dev(x))), ref)
+    with pytest.raises(bh.BitLinearError) as ei:
+        bh.BitNetWeightQuantizer(bh.WeightQuantizationConfig(custom_threshold_factor=2.5))
+    assert ei.value.kind == "InvalidConfig"
+    with pytest.raises(bh.BitLinearError):
+        bh.BitNetWeightQuantizer().quantize(torch.ones(4, device="cuda"))
+    # an all-zero tensor: no non-zero code, scale 1.0 (compute_ternary_scale, weights.rs:554-556)
+    z = bh.BitNetWeightQuantizer(bh.WeightQuantizationConfig(normalize_weights=False, outlier_threshold=0.0)).quantize(
+        torch.zeros(4, 8, device="cuda"))
+    assert not host(z.values).any() and host(z.scales)[0] == 1.0
+
+
 # ---- R1 + A1 -------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("m,k", [(1, 2560), (4, 2560), (3, 6912), (2, 1024), (5, 4096), (2, 8192), (2, 12000),
@@ -878,33 +928,38 @@ def test_decoder_stack_config5_full_depth_bit_exact():
 
 @pytest.mark.parametrize("dims,layers", [((2560, 6912, 20, 5, 128), 4), ((256, 512, 4, 2, 64), 3),
                                          ((1024, 2816, 8, 8, 128), 2)])
-def test_decoder_single_launch_matches_oracle_and_per_launch_path(dims, layers):
-    """One token: the whole run of blocks as one cooperative launch (grid barriers between the steps) gives the
-    oracle's bits, the same as the (default) launch-per-step path; repeated calls, sub-ranges of blocks and
-    in-place hidden states included."""
+def test_decoder_repeated_calls_subranges_and_streams(dims, layers):
+    """One token: repeated calls, sub-ranges of blocks, in-place hidden states, one block at a time (as the benchmark
+    does), and calls issued from two streams in turn (the decoder's buffers are shared: the second call waits for the
+    first on the GPU)."""
     rng = np.random.default_rng(layers + dims[0])
     dec, ref = build_decoder(rng, layers, *dims, max_tokens=2)
-    assert dec.set_single_launch(True), "the single-launch path should be available at these shapes"
     x = synth_activations(rng, 1, dims[0])
     x_ref, q_ref, k_ref = oracle_stack(ref, x, *dims)
-    for _ in range(3):  # the barrier epochs keep growing from call to call
+    for _ in range(3):
         out, q, k = dec.decode(dev(x), want_qk=True)
         assert np.array_equal(host(out), x_ref)
         assert np.array_equal(host(q), q_ref) and np.array_equal(host(k), k_ref)
-    dec.set_single_launch(False)
-    out2, q2, k2 = dec.decode(dev(x), want_qk=True)
-    assert np.array_equal(host(out2), x_ref) and np.array_equal(host(q2), q_ref) and np.array_equal(host(k2), k_ref)
-    dec.set_single_launch(True)
-    # blocks 1 .. layers-1 only, hidden state updated in place
     x1_ref = oracle_stack(ref[:1], x, *dims)[0]
     buf = dev(x1_ref.copy())
     dec.decode(buf, out=buf, layers=(1, layers))
     assert np.array_equal(host(buf), x_ref)
-    # one block at a time, as the benchmark does
     cur = dev(x)
     for l in range(layers):
         cur = dec.decode(cur, layers=(l, l + 1))
     assert np.array_equal(host(cur), x_ref)
+    # two streams in alternation, no host synchronisation in between
+    xs = [dev(synth_activations(rng, 2, dims[0])) for _ in range(4)]
+    refs = [oracle_stack(ref, host(t), *dims)[0] for t in xs]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    outs = []
+    for i, t in enumerate(xs):
+        with torch.cuda.stream(streams[i % 2]):
+            outs.append(dec.decode(t, stream=streams[i % 2]))
+    torch.cuda.synchronize()
+    for o, r in zip(outs, refs):
+        assert np.array_equal(host(o), r)
 
 
 @pytest.mark.parametrize("layout", [bh.LAYOUT_OUT_IN, bh.LAYOUT_IN_OUT])

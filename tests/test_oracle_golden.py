@@ -143,24 +143,183 @@ def test_roundclip_is_half_absmean_threshold():
     assert orc.ternarize_roundclip(np.array([1.0, -1.0], dtype=f32), 0.0).tolist() == [0, 0]
 
 
-def test_reference_default_recipe_properties():
-    # the reference's own tests for this recipe are property tests (values, scale > 0, sign, determinism)
-    rng = np.random.default_rng(2)
-    w = synth_weights(rng, 64, 128, std=1.0)
-    q, s = orc.quantize_weights_reference(w)
-    q2, s2 = orc.quantize_weights_reference(w)
-    assert np.array_equal(q, q2) and s == s2
-    assert set(np.unique(q).tolist()) <= {-1, 0, 1} and s > 0
-    nz = q != 0
-    assert np.all(np.sign(w - w.mean())[nz] == q[nz])
-    # without normalisation / clipping it is the plain 0.7 * mean|w| threshold with a least-squares scale
-    q3, s3 = orc.quantize_weights_reference(w, normalize=False, outlier_threshold=0.0, threshold_factor=0.7)
-    thr = f32(np.abs(w.astype(np.float64)).mean()) * f32(0.7)
-    assert np.array_equal(q3, orc.ternarize_threshold(w, thr))
-    ls = float((w.astype(np.float64) * q3).sum() / (q3.astype(np.float64) ** 2).sum())
-    assert abs(float(s3) - ls) < 1e-5 * abs(ls)
+# The reference's own tests for BitNetWeightQuantizer are property tests (ternary values, positive scale,
+# determinism).  The restatement is pinned further by an independent f64 model of weights.rs:568-611,671-699 written
+# with whole-array numpy operations (the oracle loops in f32 with f64 sums), by what each stage must satisfy on its
+# own, and by inputs on which a plausible mistake changes the answer.
+
+def _model_weight_pipeline(w, method=0, normalize=True, t=3.0, custom=None):
+    """f64 model: returns processed tensor, threshold, q, scale, stats."""
+    x = w.astype(np.float64)
+    st = {}
+    if normalize:
+        mu = x.mean()
+        var = ((x - mu) ** 2).mean()
+        x = (x - mu) / np.sqrt(var + 1e-8)
+        st.update(mean=mu, sd=np.sqrt(var + 1e-8))
+    if t > 0:
+        mu2, mad = x.mean(), np.abs(x).mean()
+        st.update(lo=mu2 - t * mad, hi=mu2 + t * mad)
+        x = np.clip(x, st["lo"], st["hi"])
+    ma, mx = np.abs(x).mean(), np.abs(x).max()
+    st.update(mean_abs=ma, max_abs=mx)
+    if method == orc.METHOD_MEDIAN:
+        thr = ma * (custom or 0.8)
+    elif method == orc.METHOD_ADAPTIVE:
+        thr = ma * custom if custom else (ma * 0.5 if mx > 3.0 * ma else ma * 0.7)
+    elif method == orc.METHOD_OPTIMAL and not custom:
+        errs = []
+        for f in (0.3, 0.4, 0.5, 0.6, 0.7, 0.8, 0.9, 1.0, 1.1, 1.2):
+            qq = np.sign(x) * (np.abs(x) > ma * f)
+            errs.append(((x - qq) ** 2).mean())
+        st["errs"] = errs
+        thr = ma * (0.3 + 0.1 * int(np.argmin(errs)))
+    else:
+        thr = ma * (custom or 0.7)
+    q = (np.sign(x) * (np.abs(x) > thr)).astype(np.int8)
+    den = float((q.astype(np.float64) ** 2).sum())
+    scale = 1.0 if den < 1.1920929e-07 else float((x * q).sum() / den)
+    return x, thr, q, scale, st
+
+
+def _check_against_model(w, **kw):
+    q, s, processed, st = orc.quantize_weights_reference(w, want_details=True, **{
+        "method": kw.get("method", 0), "normalize": kw.get("normalize", True),
+        "outlier_threshold": kw.get("t", 3.0), "custom_factor": kw.get("custom")})
+    x, thr, q_m, s_m, st_m = _model_weight_pipeline(w, **kw)
+    scale_of_values = max(1.0, float(np.abs(x).max()))
+    assert np.max(np.abs(processed.astype(np.float64) - x)) <= 4e-6 * scale_of_values
+    assert abs(float(st["threshold"]) - thr) <= 2e-6 * max(thr, 1e-30)
+    differ = q != q_m
+    # ternary values equal to the model's except inside a sliver around the threshold
+    assert np.all(np.abs(np.abs(x[differ]) - thr) <= 1e-6 * scale_of_values), int(differ.sum())
+    assert differ.mean() < 1e-4
+    assert abs(float(s) - s_m) <= 1e-5 * abs(s_m) + 1e-7
+    assert set(np.unique(q).tolist()) <= {-1, 0, 1}
+    return q, s, processed, st, st_m
+
+
+@pytest.mark.parametrize("method", [orc.METHOD_MEAN, orc.METHOD_MEDIAN, orc.METHOD_ADAPTIVE, orc.METHOD_OPTIMAL, orc.METHOD_DETSTE])
+@pytest.mark.parametrize("normalize,t", [(True, 3.0), (True, 0.0), (False, 3.0), (False, 0.0), (True, 1.5)])
+def test_reference_weight_pipeline_against_f64_model(method, normalize, t):
+    rng = np.random.default_rng(10 * method + int(normalize) + int(t * 2))
+    # mean 3 and spread 5: normalising matters, and var != sd
+    w = (3.0 + 5.0 * rng.standard_normal((48, 200))).astype(f32)
+    w[rng.random(w.shape) < 0.01] *= f32(6.0)  # outliers for the clip stage
+    _check_against_model(w, method=method, normalize=normalize, t=t)
+    _check_against_model(w, method=method, normalize=normalize, t=t, custom=0.45)
+
+
+def test_reference_weight_pipeline_stage_properties():
+    rng = np.random.default_rng(77)
+    w = (-2.0 + 0.3 * rng.standard_normal((64, 128))).astype(f32)
+    w[::7, ::5] *= f32(4.0)
+    # normalise only: mean 0, variance 1 (to f32 accuracy), an affine increasing map of w
+    q, s, x, st = orc.quantize_weights_reference(w, normalize=True, outlier_threshold=0.0, want_details=True)
+    x64 = x.astype(np.float64)
+    assert abs(x64.mean()) < 1e-5 and abs(x64.var() - 1.0) < 1e-4
+    assert np.array_equal(np.argsort(w, axis=None, kind="stable"), np.argsort(x, axis=None, kind="stable"))
+    assert st["sd"] == f32(np.sqrt(f32(((w.astype(np.float64) - float(st["mean"])) ** 2).mean()) + f32(1e-8))) or \
+        abs(float(st["sd"]) - np.sqrt(w.astype(np.float64).var() + 1e-8)) < 1e-6 * float(st["sd"])
+    # clip on top: the bounds are mean' -+ t * mean|w'| of the NORMALISED tensor, attained exactly by what was clipped
+    q2, s2, y, st2 = orc.quantize_weights_reference(w, normalize=True, outlier_threshold=2.0, want_details=True)
+    lo, hi = st2["lo"], st2["hi"]
+    assert abs(float(hi) - (x64.mean() + 2.0 * np.abs(x64).mean())) < 1e-5
+    assert abs(float(lo) - (x64.mean() - 2.0 * np.abs(x64).mean())) < 1e-5
+    clipped_hi, clipped_lo = x > hi, x < lo
+    assert clipped_hi.any() and clipped_lo.any()
+    assert np.all(y[clipped_hi] == hi) and np.all(y[clipped_lo] == lo)
+    inside = ~(clipped_hi | clipped_lo)
+    assert np.array_equal(y[inside], x[inside]) and y.max() == hi and y.min() == lo
+    # threshold: strict '>' on the processed tensor, sign of the processed (not the raw) value
+    thr = st2["threshold"]
+    assert thr == st2["mean_abs"] * f32(0.7)
+    assert np.array_equal(q2, np.where(y > thr, 1, np.where(y < -thr, -1, 0)).astype(np.int8))
+    assert np.all(w < 0) and (q2 == 1).any()  # raw weights are all negative: the sign comes from the normalised tensor
+    # least-squares scale: the minimiser of |y - s q|^2, so the residual is orthogonal to q
+    resid = y.astype(np.float64) - float(s2) * q2
+    assert abs((resid * q2).sum()) < 1e-3 and s2 > 0
+    assert abs(float(s2) - float(st2["num"]) / float(st2["den"])) < 1e-7 and st2["den"] == f32((q2 != 0).sum())
+    # determinism, zero matrix, an exact tie stays zero
+    q3, s3 = orc.quantize_weights_reference(w, outlier_threshold=2.0)
+    assert np.array_equal(q2, q3) and s2 == s3
     q0, s0 = orc.quantize_weights_reference(np.zeros((4, 4), dtype=f32), normalize=False, outlier_threshold=0.0)
     assert not q0.any() and s0 == 1.0
+    tie = np.array([[1.0, -1.0, 2.0, -2.0]], dtype=f32)  # mean|w| = 1.5, custom factor 2/3 is not exact in f32 -> use 1.0 / 1.5
+    qt, _, _, stt = orc.quantize_weights_reference(tie, normalize=False, outlier_threshold=0.0, custom_factor=1.0,
+                                                   want_details=True)
+    assert stt["threshold"] == 1.5 and qt.tolist() == [[0, 0, 1, -1]]
+
+
+def test_reference_weight_pipeline_plausible_mistakes_change_the_answer():
+    """Inputs on which dividing by the variance instead of the standard deviation, clipping before normalising, a clip
+    bound built from the standard deviation, or the raw tensor in the scale would each give different ternary values
+    or a different scale: the restatement agrees with the f64 model, the mutated models do not."""
+    rng = np.random.default_rng(5)
+    w = (1.0 + 4.0 * rng.standard_normal((32, 96))).astype(f32)
+    w.flat[rng.choice(w.size, 40, replace=False)] *= f32(8.0)
+    q, s, x, st, _ = _check_against_model(w, method=0, normalize=True, t=3.0)
+    w64 = w.astype(np.float64)
+    mu, var = w64.mean(), w64.var()
+
+    def finish(xx, lo, hi):
+        xx = np.clip(xx, lo, hi)
+        thr = 0.7 * np.abs(xx).mean()
+        qq = (np.sign(xx) * (np.abs(xx) > thr)).astype(np.int8)
+        return qq, float((xx * qq).sum() / max((qq != 0).sum(), 1))
+
+    # (a) variance in place of the standard deviation
+    xa = (w64 - mu) / (var + 1e-8)
+    qa, sa = finish(xa, xa.mean() - 3 * np.abs(xa).mean(), xa.mean() + 3 * np.abs(xa).mean())
+    assert abs(sa - float(s)) > 1e-2 * float(s)
+    # (b) clip first, then normalise
+    xb = np.clip(w64, mu - 3 * np.abs(w64).mean(), mu + 3 * np.abs(w64).mean())
+    xb = (xb - xb.mean()) / np.sqrt(xb.var() + 1e-8)
+    qb, sb = finish(xb, -np.inf, np.inf)
+    assert (qb != q).mean() > 1e-3 or abs(sb - float(s)) > 1e-3 * float(s)
+    # (c) clip bound from the standard deviation (1.0 after normalising) instead of the mean absolute value
+    xc = (w64 - mu) / np.sqrt(var + 1e-8)
+    qc, sc = finish(xc, xc.mean() - 3.0, xc.mean() + 3.0)
+    assert abs(sc - float(s)) > 1e-3 * float(s)
+    # (d) scale against the raw tensor
+    sd_ = float((w64 * q).sum() / (q != 0).sum())
+    assert abs(sd_ - float(s)) > 1e-2 * float(s)
+
+
+def test_reference_weight_methods_pick_their_factors():
+    rng = np.random.default_rng(9)
+    w = rng.standard_normal((40, 64)).astype(f32)
+    kw = dict(normalize=False, outlier_threshold=0.0, want_details=True)
+    ma = orc.quantize_weights_reference(w, **kw)[3]["mean_abs"]
+    assert orc.quantize_weights_reference(w, method=orc.METHOD_MEAN, **kw)[3]["threshold"] == ma * f32(0.7)
+    assert orc.quantize_weights_reference(w, method=orc.METHOD_MEDIAN, **kw)[3]["threshold"] == ma * f32(0.8)
+    assert orc.quantize_weights_reference(w, method=orc.METHOD_DETSTE, **kw)[3]["threshold"] == ma * f32(0.7)
+    # adaptive: a gaussian has max|w| > 3 mean|w| (factor 0.5); a two-level tensor does not (factor 0.7)
+    st = orc.quantize_weights_reference(w, method=orc.METHOD_ADAPTIVE, **kw)[3]
+    assert st["max_abs"] > f32(3.0) * ma and st["threshold"] == ma * f32(0.5)
+    flat = np.where(rng.random((40, 64)) < 0.5, 1.0, -2.0).astype(f32)
+    st = orc.quantize_weights_reference(flat, method=orc.METHOD_ADAPTIVE, **kw)[3]
+    assert st["max_abs"] <= f32(3.0) * st["mean_abs"] and st["threshold"] == st["mean_abs"] * f32(0.7)
+    # a custom factor overrides every method's choice
+    for method in range(5):
+        st = orc.quantize_weights_reference(w, method=method, custom_factor=1.1, **kw)[3]
+        assert st["threshold"] == ma * f32(1.1)
+    # optimal: the first smallest of the ten candidates; for a gaussian the error of an unscaled {-1,0,1} code is
+    # smallest at the low end, for a two-level tensor {+-1 mostly, few +-0.2} at the top of the zeros' plateau
+    x, thr, q_m, s_m, st_m = _model_weight_pipeline(w, method=orc.METHOD_OPTIMAL, normalize=False, t=0.0)
+    st = orc.quantize_weights_reference(w, method=orc.METHOD_OPTIMAL, **kw)[3]
+    errs = np.array(st_m["errs"])
+    assert np.sort(errs)[1] - np.sort(errs)[0] > 1e-5  # the argmin is not a near-tie
+    assert st["threshold"] == ma * f32(0.3 + 0.1 * int(np.argmin(errs)))
+    two = np.where(rng.random((40, 64)) < 0.8, 1.0, 0.2).astype(f32) * np.sign(rng.standard_normal((40, 64))).astype(f32)
+    x, thr, q_m, s_m, st_m = _model_weight_pipeline(two, method=orc.METHOD_OPTIMAL, normalize=False, t=0.0)
+    q, s, _, st = orc.quantize_weights_reference(two, method=orc.METHOD_OPTIMAL, **kw)
+    # every candidate between 0.2/0.84 and 1/0.84 of mean|w| gives the same code: ties keep the FIRST ('<' comparison)
+    errs = np.array(st_m["errs"])
+    first = int(np.argmin(errs))
+    assert np.sum(np.isclose(errs, errs[first], rtol=0, atol=1e-12)) >= 3
+    assert st["threshold"] == st["mean_abs"] * np.array([0.3, 0.4, 0.5, 0.6, 0.7, 0.8, 0.9, 1.0, 1.1, 1.2], dtype=f32)[first]
+    assert np.array_equal(q, q_m)
 
 
 # ---- G1 / G2: contraction ---------------------------------------------------------------------------
