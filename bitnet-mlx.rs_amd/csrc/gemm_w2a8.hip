@@ -30,8 +30,8 @@
 // (f32 output only, n % 4 == 0, scales within the short division's range) is straight-line code
 // (store_fragments_fast), everything else goes through store_fragments_general: same bits.
 //
-// gemm_dma8_kernel: the same data path with eight wavefronts per workgroup, for launches with about one tile
-// per compute unit (see its own comment).
+// gemm_ld8_kernel: the same data path with eight multiplying and two loading wavefronts per workgroup, for launches
+// with at most one tile per compute unit (see its own comment).
 //
 // gemm_tiled_kernel (any shape, computes the row sums itself): activations pass through registers.
 // Activations are staged through LDS one weight tile (256 columns) at a time, double buffered: the global
@@ -649,36 +649,42 @@ int launch_dma(GemmParams p, hipStream_t stream)
     return BITNET_HIP_OK;
 }
 
-// ---- eight wavefronts per workgroup, the k range of every stage split between two groups of four ---------
+// ---- eight MFMA wavefronts per workgroup fed by two loader wavefronts -------------------------------------------
 //
-// One wavefront per SIMD cannot keep the MFMA pipe busy (its own LDS waits and unpack instructions sit between
-// its MFMAs); two can.  When a launch has too few tiles for two workgroups per compute unit, the second
-// wavefront per SIMD comes from inside the workgroup instead: 512 threads, wavefronts 0..3 take columns
-// 0..127 of every 256-column stage and wavefronts 4..7 columns 128..255, each group accumulating the whole
-// BM x BN tile.  The two partial tiles are exchanged through LDS at the end (int32 sums: exact), each group
-// finishing half of the fragments.  A stage is one 256-column weight tile plus BM x 256 activation bytes.
-constexpr int D8_NST = 3;
+// For launches with at most one 128 x 160 tile per compute unit.  One wavefront per SIMD cannot keep the MFMA pipe
+// busy (its own LDS waits and unpack instructions sit between its MFMAs); two can.  With too few tiles for two
+// workgroups per compute unit the second wavefront per SIMD comes from inside the workgroup: wavefronts 0..3 take
+// columns 0..127 of every 256-column stage and wavefronts 4..7 columns 128..255, each group accumulating the whole
+// BM x BN tile; the two partial tiles are exchanged through LDS at the end (int32 sums: exact), each group
+// finishing half of the fragments.  A stage is one 256-column weight tile plus BM x 256 activation bytes, three
+// stages in LDS, loads two stages ahead.
+// The LDS-direct loads are issued by two further wavefronts (8 and 9) that never multiply.  A wavefront that issues
+// a load while the queue of the load path is full waits at that instruction, and while it waits it issues no MFMA;
+// with the loads spread over the multiplying wavefronts every one of them paid that wait every stage (measured at
+// 2048 x 2560 x 6912: 40.8 us with the loads on the eight wavefronts, 33.6 us with no loads in the loop at all,
+// 35.8 us with the two loaders).  The multiplying wavefronts meet the loaders at the stage barrier and otherwise
+// only read LDS and run MFMAs.
+constexpr int LD8_NST = 3;
 template <int BM, int BN>
-constexpr size_t dma8_lds_bytes() { return (size_t)D8_NST * (BM * 256 + (BN / 16) * 1024) + rowp_bytes<BM>(); }
+constexpr size_t ld8_lds_bytes() { return (size_t)LD8_NST * (BM * 256 + (BN / 16) * 1024) + rowp_bytes<BM>(); }
 
 template <int BM, int BN>
-__global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
+__global__ __launch_bounds__(640, 1) void gemm_ld8_kernel(GemmParams p)
 {
     constexpr int WTM = BM / 2, WTN = BN / 2, FM = WTM / 16, FN = WTN / 16;
     constexpr int A_STAGE = BM * 256;
-    constexpr int A_DMA = A_STAGE / 1024 / 8;   // LDS-direct loads per wavefront per stage
+    constexpr int A_CHUNKS = A_STAGE / 1024;    // 1 KiB LDS-direct loads per stage
     constexpr int B_TILES = BN / 16;
-    constexpr int B_DMA = (B_TILES + 7) / 8;    // per wavefront (the last ones may repeat a tile)
     constexpr int B_STAGE = B_TILES * 1024;
     constexpr int STAGE = A_STAGE + B_STAGE;
-    constexpr int GROUP = A_DMA + B_DMA;
-    static_assert(A_STAGE % 8192 == 0 && WTM % 32 == 0 && WTN % 16 == 0, "tile shape");
-    static_assert((FM / 2) * FN * 4 * 256 * 8 <= D8_NST * STAGE, "exchange area");
+    constexpr int A_PER = A_CHUNKS / 2, B_PER = (B_TILES + 1) / 2;  // per loader wavefront
+    constexpr int GROUP = A_PER + B_PER;
+    static_assert(A_CHUNKS % 2 == 0 && WTM % 32 == 0 && WTN % 16 == 0 && 2 * GROUP < 64, "tile shape, vmcnt range");
+    static_assert((FM / 2) * FN * 4 * 256 * 8 <= LD8_NST * STAGE, "exchange area");
 
-    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [NST][A half 0 | A half 1 | B]
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [NST][A half 0 | A half 1 | B], then the row operands
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kg = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1, lr = lane & 15, lg = lane >> 4;
 
     int tile_id;
     {
@@ -688,7 +694,6 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
         tile_id = xcd * per_xcd + idx;
         if (tile_id >= total) return;
     }
-    // tiles_n counts the column tiles of all projections of the launch, one after the other
     const int tm = tile_id / p.tiles_n, tn_all = tile_id % p.tiles_n;
     int pj = 0;
     if (p.nproj > 1 && tn_all >= p.proj[0].tn_end) pj = 1;
@@ -696,58 +701,71 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
     const GemmProjDev PJ = p.proj[pj];  // uniform over the workgroup
     const int tn = tn_all - (pj ? p.proj[pj - 1].tn_end : 0);
     const int m0 = tm * BM, n0 = tn * BN;
+    constexpr uint32_t ROWP = LD8_NST * STAGE;
 
-    // Activation loads: chunk c = wave*A_DMA + q of a stage is 8 rows x 128 columns: half c / (BM/8), rows
-    // 8*(c % (BM/8)) .. +7.  Lane l lands in row l/8 at physical 16-byte chunk l%8 and fetches logical chunk
-    // (l%8) ^ (row & 7).  Rows past m re-read row m-1 (their results are never stored).
-    uint32_t a_off[A_DMA];  // byte offsets into the activation matrix (below 4 GiB: checked by the launcher)
+    if (wave >= 8) {
+        // ---- loader wavefront L: activation chunks A_PER*L .. and weight tiles B_PER*L .. of every stage ----
+        const int L = wave - 8;
+        uint32_t a_off[A_PER], b_off[B_PER], b_dst[B_PER];
 #pragma unroll
-    for (int q = 0; q < A_DMA; ++q) {
-        const int c = wave * A_DMA + q;
-        const int half = c / (BM / 8), row = 8 * (c % (BM / 8)) + (lane >> 3);
-        const int lc = (lane & 7) ^ (row & 7);
-        int grow = m0 + row;
-        if (grow >= p.m) grow = p.m - 1;
-        a_off[q] = (uint32_t)grow * (uint32_t)p.k + half * 128 + lc * 16;
+        for (int q = 0; q < A_PER; ++q) {
+            const int c = L * A_PER + q;
+            const int half = c / (BM / 8), row = 8 * (c % (BM / 8)) + (lane >> 3);
+            const int lc = (lane & 7) ^ (row & 7);
+            int grow = m0 + row;
+            if (grow >= p.m) grow = p.m - 1;
+            a_off[q] = (uint32_t)grow * (uint32_t)p.k + half * 128 + lc * 16;
+        }
+        const int rb0 = n0 / 16, rb_last = (PJ.n + 15) / 16 - 1;
+#pragma unroll
+        for (int q = 0; q < B_PER; ++q) {
+            int tix = L * B_PER + q;
+            if (tix >= B_TILES) tix = B_TILES - 1;
+            int rb = rb0 + tix;
+            if (rb > rb_last) rb = rb_last;
+            b_off[q] = ((uint32_t)rb * (uint32_t)p.kt_count * 64 + lane) * 16;
+            b_dst[q] = A_STAGE + tix * 1024;
+        }
+        auto issue = [&](int kt) {
+            const uint32_t stage = lds_base + (kt % LD8_NST) * STAGE;
+#pragma unroll
+            for (int q = 0; q < B_PER; ++q) dma16(PJ.w + (size_t)kt * 1024, b_off[q], stage + b_dst[q]);
+#pragma unroll
+            for (int q = 0; q < A_PER; ++q) dma16(p.a + (size_t)kt * 256, a_off[q], stage + (L * A_PER + q) * 1024);
+        };
+        // the per-row epilogue operands: a_sum by loader 0, a_scale by loader 1 (BM / 64 loads of 64 rows each)
+#pragma unroll
+        for (int ch = 0; ch < BM / 64; ++ch) {
+            int grow = m0 + ch * 64 + lane;
+            if (grow >= p.m) grow = p.m - 1;
+            if (L == 0) dma4(p.a_sum, (uint32_t)grow * 4u, lds_base + ROWP + ch * 256);
+            else if (p.a_scale) dma4(p.a_scale, (uint32_t)grow * 4u, lds_base + ROWP + BM * 4 + ch * 256);
+        }
+        issue(0);
+        if (p.kt_count > 1) issue(1);
+        for (int kt = 0; kt < p.kt_count; ++kt) {
+            if (kt + 1 < p.kt_count) wait_vm<GROUP>(); else wait_vm<0>();
+            __syncthreads();
+            if (kt + 2 < p.kt_count) issue(kt + 2);
+        }
+        __syncthreads();  // the two barriers of the exchange
+        __syncthreads();
+        return;
     }
-    const int rb0 = n0 / 16;
-    const int rb_last = (PJ.n + 15) / 16 - 1;
-    uint32_t b_off[B_DMA], b_dst[B_DMA];
-#pragma unroll
-    for (int q = 0; q < B_DMA; ++q) {
-        int tix = wave + 8 * q;
-        if (tix >= B_TILES) tix = B_TILES - 1;
-        int rb = rb0 + tix;
-        if (rb > rb_last) rb = rb_last;
-        b_off[q] = ((uint32_t)rb * (uint32_t)p.kt_count * 64 + lane) * 16;
-        b_dst[q] = A_STAGE + tix * 1024;
-    }
-    auto issue = [&](int kt) {
-        const uint32_t stage = lds_base + (kt % D8_NST) * STAGE;
-#pragma unroll
-        for (int q = 0; q < B_DMA; ++q) dma16(PJ.w + (size_t)kt * 1024, b_off[q], stage + b_dst[q]);
-#pragma unroll
-        for (int q = 0; q < A_DMA; ++q) dma16(p.a + (size_t)kt * 256, a_off[q], stage + (wave * A_DMA + q) * 1024);
-    };
 
+    const int kg = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1, lr = lane & 15, lg = lane >> 4;
     v4i acc[FM][FN];
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j] = (v4i){0, 0, 0, 0};
-
-    constexpr uint32_t ROWP = D8_NST * STAGE;
-    fetch_row_operands<BM>(p, m0, wave, lane, lds_base + ROWP);
-    issue(0);
-    if (p.kt_count > 1) issue(1);
-
     uint32_t a_rd[FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i) a_rd[i] = kg * (BM * 128) + (wm * WTM + i * 16 + lr) * 128;
     const int sw = lr & 7;
 
     auto compute = [&](int kt) {
-        const uint8_t *abuf = lds + (kt % D8_NST) * STAGE;
+        const uint8_t *abuf = lds + (kt % LD8_NST) * STAGE;
         const uint8_t *bbuf = abuf + A_STAGE + (wn * FN) * 1024 + lane * 16 + kg * 8;
         uint2 bp[FN];  // dwords 2*kg, 2*kg+1 of the slot: this group's two k-steps
 #pragma unroll
@@ -773,19 +791,16 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
         }
     };
     for (int kt = 0; kt < p.kt_count; ++kt) {
-        if (kt + 1 < p.kt_count) wait_vm<GROUP>(); else wait_vm<0>();
-        __syncthreads();
-        if (kt + 2 < p.kt_count) issue(kt + 2);
+        __syncthreads();  // the loaders arrive here once stage kt has landed
         compute(kt);
     }
 
     // ---- exchange: group 0 finishes fragments i < FM/2, group 1 the others ----
     __syncthreads();  // every wavefront is done with the stage buffers
+    constexpr int HALF = FM / 2;
     {
-        constexpr int HALF = FM / 2;
         v4i *xch = reinterpret_cast<v4i *>(lds);
         const int mine = wave, partner = wave ^ 4;
-        // what this wavefront gives away: the half of the fragments the partner finishes
 #pragma unroll
         for (int i = 0; i < HALF; ++i)
 #pragma unroll
@@ -800,9 +815,6 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
                 if (kg == 0) acc[i][j] += o; else acc[i + HALF][j] += o;
             }
     }
-
-    // this group's finished fragments (kg is uniform over the wavefront)
-    constexpr int HALF = FM / 2;
     v4i fin[HALF][FN];
     int lrows[HALF];
 #pragma unroll
@@ -815,19 +827,19 @@ __global__ __launch_bounds__(512, 1) void gemm_dma8_kernel(GemmParams p)
 }
 
 template <int BM, int BN>
-int launch_dma8(GemmParams p, hipStream_t stream)
+int launch_ld8(GemmParams p, hipStream_t stream)
 {
     p.tiles_m = (p.m + BM - 1) / BM;
     p.tiles_n = 0;
     for (int j = 0; j < p.nproj; ++j) p.proj[j].tn_end = p.tiles_n += (p.proj[j].n + BN - 1) / BN;
     const int total = p.tiles_m * p.tiles_n;
     const int grid = ((total + 7) / 8) * 8;
-    constexpr size_t lds = dma8_lds_bytes<BM, BN>();
+    constexpr size_t lds = ld8_lds_bytes<BM, BN>();
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static const hipError_t attr = raise_lds_limit(&gemm_dma8_kernel<BM, BN>, lds);
+    static const hipError_t attr = raise_lds_limit(&gemm_ld8_kernel<BM, BN>, lds);
     BITNET_HIP_TRY(attr);
-    hipLaunchKernelGGL((gemm_dma8_kernel<BM, BN>), dim3(grid), dim3(512), lds, stream, p);
-    BITNET_HIP_CHECK_LAUNCH("gemm_dma8_kernel");
+    hipLaunchKernelGGL((gemm_ld8_kernel<BM, BN>), dim3(grid), dim3(640), lds, stream, p);
+    BITNET_HIP_CHECK_LAUNCH("gemm_ld8_kernel");
     return BITNET_HIP_OK;
 }
 
@@ -877,10 +889,11 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
     //                                           activation stages each (more resident wavefronts beat deeper
     //                                           pipelines: 2.45 POP/s at 8192 x 2560 x 6912, against 2.23 with two
     //                                           workgroups of three stages);
-    //   0.75 to one tile per compute unit    -> 128 x 160, one workgroup of 8 wavefronts (k split inside it);
+    //   0.4 to one tile per compute unit     -> 128 x 160, one workgroup of 8 multiplying wavefronts (k split inside it)
+    //                                           and two loader wavefronts;
     //   otherwise                            -> 64 x 160, four workgroups of 4 wavefronts per compute unit.
     if (tiles >= 640) return launch_dma<128, 160, 2, 3>(p, stream);
-    if (tiles >= 192 && tiles <= 256) return launch_dma8<128, 160>(p, stream);
+    if (tiles >= 100 && tiles <= 256) return launch_ld8<128, 160>(p, stream);
     return launch_dma<64, 160, 2, 4>(p, stream);
 }
 
