@@ -39,6 +39,7 @@
 // one barrier per stage.  Rows are padded to 272 bytes so that the 16-byte fragment reads of 8 consecutive
 // lanes fall in distinct banks.
 #include "kernels.hpp"
+#include "ldsdma.hpp"
 
 namespace bitnet {
 
@@ -262,35 +263,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p)
 }
 
 // ---- LDS-direct pipeline -------------------------------------------------------------------------------
-
-// LDS-direct load of 16 bytes per lane: m0 carries the LDS base of the wavefront's 1 KiB destination, lane l
-// lands at base + 16*l.  The global address is a scalar base plus a 32-bit per-lane byte offset: the offsets are
-// loop invariant, so advancing a stage costs two scalar additions and no vector instruction.
-__device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_off)
-{
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1\n\t"
-                 : : "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory", "m0");
-}
-// s_setprio takes an immediate.
-__device__ __forceinline__ void set_wave_priority(int pr)
-{
-    if (pr == 0) __builtin_amdgcn_s_setprio(0);
-    else if (pr == 1) __builtin_amdgcn_s_setprio(1);
-    else if (pr == 2) __builtin_amdgcn_s_setprio(2);
-    else __builtin_amdgcn_s_setprio(3);
-}
-template <int N>
-__device__ __forceinline__ void wait_vm()
-{
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
-
-// The same for 4 bytes per lane: lane l lands at base + 4*l.
-__device__ __forceinline__ void dma4(const void *sbase, uint32_t voff, uint32_t lds_off)
-{
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1\n\t"
-                 : : "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds_off)) : "memory", "m0");
-}
 
 // Per-row epilogue operands of a BM-row tile, fetched into LDS by LDS-direct loads (no registers are held across
 // the k loop): a_sum[BM] as int32, then a_scale[BM].  Wavefront w < BM/64 fetches rows 64*w .. of a_sum, the

@@ -36,6 +36,7 @@
 #include "kernels.hpp"
 #include "rowquant.hpp"
 #include "tiledot.hpp"
+#include "ldsdma.hpp"
 
 namespace bitnet {
 
@@ -1010,6 +1011,161 @@ __global__ __launch_bounds__(256) void gemv_mfma_lds_kernel(const int8_t *hot_a,
     }
 }
 
+// 17 and more tokens: gemv_mfma_lds_kernel's scheme with the tokens cut into groups of 16, one workgroup per
+// (group of RB row blocks, token group).  gemv_mfma_kernel gives every workgroup ALL token rows (16 * MT of them) for
+// its 16 * RB output rows, gathered per wavefront straight from memory: at 64 tokens that is 164 KB (k = 2560) to
+// 442 KB (k = 6912) through the one L1 of a compute unit for 32 output rows, 70 MB of L2 traffic per launch for a
+// 4.4 MB weight matrix, and the kernel takes 11 to 15 us.  Here a workgroup copies only its 16 token rows into LDS
+// (dense 16-byte loads, rows k + 16 bytes apart) and the weight tiles are read once per token group: with the token
+// groups of a row-block group placed on the same XCD, from HBM once and from that XCD's L2 afterwards.
+// The copy is made by LDS-direct loads, all in flight at once, and the wavefront's k-tiles (kt = wave + 4u, at most NT of
+// them) are requested as one batch right behind it, so the two latencies overlap.  k % 256 == 0, activations 16-byte
+// aligned, m * k < 4 GiB, 16 * (k + 16) bytes of dynamic LDS.
+template <int RB, int NT>
+__global__ __launch_bounds__(256) void gemv_mfma_tg_kernel(const int8_t *hot_a, int hot_k, int hot_m, int hot_kt_count, int hot_groups,
+                                                           int hot_tgroups, GemvMfmaParams p)
+{
+    extern __shared__ uint4 lds_act[];        // [16][k / 16 + 1] chunks of 16 int8
+    __shared__ int red[4][RB][64][4];         // partial accumulators of the four wavefronts
+    __shared__ int red_sum[4][16];            // per wavefront: sum_k a[t, k] over its k-tiles
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lr = lane & 15, lg = lane >> 4;
+    const int cpr = hot_k >> 4, stride = cpr + 1;  // chunks per row in memory and in LDS
+
+    // Workgroups go to the eight XCDs in turn: the ids that share an XCD walk the (row-block group, token group) pairs
+    // with the token group fastest, so the token groups of one row-block group meet in one L2.
+    const int total = hot_groups * hot_tgroups;
+    const int per_xcd = (total + 7) >> 3;
+    const int idx = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (idx >= total) return;  // uniform over the workgroup
+    const int grp_all = idx / hot_tgroups, tg = idx - grp_all * hot_tgroups;
+    const int t0 = tg * 16, rows_here = min(16, hot_m - t0);
+
+    // The copy, by LDS-direct loads (no registers, every load of the wavefront in flight at once): load q of the
+    // workgroup fills the LDS chunks 64q .. 64q + 63, lane l the chunk L = 64q + l = (row L / stride, column chunk
+    // L % stride); it fetches that chunk of its token row (rows past the end repeat the last one, the pad chunk of a
+    // row repeats the chunk before it: neither is ever read).
+    {
+        const uint32_t lds_base = (uint32_t)(uintptr_t)lds_act;
+        const int nl = 16 * stride;
+        const uint32_t row_bytes = (uint32_t)hot_k;
+        const uint32_t base_off = (uint32_t)t0 * row_bytes;  // the launcher keeps m * k below 4 GiB
+        for (int q = wave; q * 64 < nl; q += 4) {
+            const int L = min(q * 64 + lane, nl - 1);
+            const int r = L / stride, cc = L - r * stride;
+            dma16(hot_a, base_off + (uint32_t)min(r, rows_here - 1) * row_bytes + (uint32_t)min(cc, cpr - 1) * 16u,
+                  lds_base + (uint32_t)q * 1024u);
+        }
+    }
+
+    int pj = 0;
+#pragma unroll
+    for (int j = 0; j < GEMV_MAX_PROJ - 1; ++j)
+        if (j + 1 < p.nproj && grp_all >= p.proj[j].rb_end) pj = j + 1;
+    const GemvProjDev &P = p.proj[pj];
+    const int rb0 = (grp_all - (pj ? p.proj[pj - 1].rb_end : 0)) * RB;
+    const int rb_count = (P.n + TILE_ROWS - 1) / TILE_ROWS;
+    const uint4 *wbase = reinterpret_cast<const uint4 *>(P.w) + lane;
+    // all k-tiles of this wavefront in one batch, requested right behind the copy; tiles and row blocks past the end
+    // repeat the last one.  The weights are read by the other token groups too, so these loads keep their cache lines
+    // (no non-temporal hint).
+    uint4 w[NT][RB];
+#pragma unroll
+    for (int u = 0; u < NT; ++u)
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+            w[u][r] = wbase[((size_t)min(rb0 + r, rb_count - 1) * hot_kt_count + min(wave + 4 * u, hot_kt_count - 1)) * 64];
+    __builtin_amdgcn_sched_barrier(0);
+    wait_vm<NT * RB>();  // loads return in order: the copy has landed, the weight tiles may still be in flight
+    lds_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+
+    constexpr int FPW = (RB + 3) / 4;
+    const float *absent = reinterpret_cast<const float *>(P.w);
+    int lane_zero = 0;
+    asm volatile("" : "+v"(lane_zero));
+    const float ws = (P.out ? P.w_scale : absent)[lane_zero];
+    float e_bias[FPW], e_scale[FPW][4], e_res[FPW][4];
+#pragma unroll
+    for (int f = 0; f < FPW; ++f) {
+        const int fr = min(wave + 4 * f, RB - 1);
+        const int e_n = min((rb0 + fr) * TILE_ROWS + lr, P.n - 1);
+        e_bias[f] = *(P.bias ? P.bias + e_n : absent);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = t0 + min(lg * 4 + i, rows_here - 1);
+            e_scale[f][i] = *(P.out ? p.a_scale + t : absent);
+            e_res[f][i] = *(P.residual ? P.residual + ((size_t)t * P.n + e_n) : absent);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    v4i acc[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) acc[r] = (v4i){0, 0, 0, 0};
+    int rowsum = 0;
+    const bool row_ok = lr < rows_here;
+    const uint4 *arow = lds_act + (row_ok ? lr : 0) * stride + lg;  // A operand: token row lr, columns 64t + 16lg .. +15 of a k-tile
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+        const int kt = wave + 4 * u;
+        if (kt < hot_kt_count) {  // uniform over the wavefront
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                v4i af = (v4i){0, 0, 0, 0};
+                if (row_ok) af = *reinterpret_cast<const v4i *>(arow + kt * 16 + t * 4);
+                rowsum = __builtin_amdgcn_sdot4(af[0], 0x01010101, rowsum, false);
+                rowsum = __builtin_amdgcn_sdot4(af[1], 0x01010101, rowsum, false);
+                rowsum = __builtin_amdgcn_sdot4(af[2], 0x01010101, rowsum, false);
+                rowsum = __builtin_amdgcn_sdot4(af[3], 0x01010101, rowsum, false);
+#pragma unroll
+                for (int r = 0; r < RB; ++r) {
+                    const uint4 w4 = w[u][r];
+                    const uint32_t wd = t == 0 ? w4.x : (t == 1 ? w4.y : (t == 2 ? w4.z : w4.w));
+                    v4i bf;
+                    bf[0] = (int)(wd & 0x03030303u);
+                    bf[1] = (int)((wd >> 2) & 0x03030303u);
+                    bf[2] = (int)((wd >> 4) & 0x03030303u);
+                    bf[3] = (int)((wd >> 6) & 0x03030303u);
+                    acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf, acc[r], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    rowsum = sum_over_lane_groups(rowsum);
+    if (lane < 16) red_sum[wave][lane] = rowsum;
+#pragma unroll
+    for (int r = 0; r < RB; ++r) *reinterpret_cast<v4i *>(&red[wave][r][lane][0]) = acc[r];
+    lds_barrier();
+#pragma unroll
+    for (int f = 0; f < FPW; ++f) {
+        if (wave + 4 * f >= RB) break;  // uniform over the wavefront
+        const int fr = wave + 4 * f;
+        const int n = (rb0 + fr) * TILE_ROWS + lr;  // result register i of lane l is C[4*(l/16) + i][l mod 16]
+        const v4i s0 = *reinterpret_cast<const v4i *>(&red[0][fr][lane][0]), s1 = *reinterpret_cast<const v4i *>(&red[1][fr][lane][0]);
+        const v4i s2 = *reinterpret_cast<const v4i *>(&red[2][fr][lane][0]), s3 = *reinterpret_cast<const v4i *>(&red[3][fr][lane][0]);
+        const v4i sum = s0 + s1 + s2 + s3;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int tl = lg * 4 + i;
+            if (n < P.n && tl < rows_here) {
+                const int asum = red_sum[0][tl] + red_sum[1][tl] + red_sum[2][tl] + red_sum[3][tl];
+                const int total_acc = sum[i] - asum;
+                const size_t o = (size_t)(t0 + tl) * P.n + n;
+                if (P.acc) P.acc[o] = total_acc;
+                if (P.out) {
+                    float v = f32_div(f32_mul((float)total_acc, ws), e_scale[f][i]);
+                    if (P.bias) v = f32_add(v, e_bias[f]);
+                    if (P.residual) v = f32_add(v, e_res[f][i]);
+                    P.out[o] = v;
+                }
+            }
+        }
+    }
+}
+
 // The reference's flat row-major packing, any n and k (rows need not start on a byte boundary).
 // One wavefront per output row; lane l takes columns 4l..4l+3, 4l+256.., gathers their codes one by one.
 __global__ __launch_bounds__(256) void gemv_rowmajor_kernel(const uint8_t *packed, const int8_t *a,
@@ -1164,6 +1320,41 @@ int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const floa
     return BITNET_HIP_OK;
 }
 
+// 17 and more token rows, k a multiple of 256 up to 8192, aligned activations: token groups of 16 (gemv_mfma_tg_kernel)
+template <int RB>
+int launch_mfma_tg(const GemvProj *projs, int nproj, const int8_t *a, const float *a_scale, size_t m, size_t k, hipStream_t stream)
+{
+    GemvMfmaParams p = {};
+    int end = 0;
+    for (int j = 0; j < nproj; ++j) {
+        const GemvProj &s = projs[j];
+        GemvProjDev &d = p.proj[j];
+        d.w = s.tiled; d.w_scale = s.w_scale; d.bias = s.bias; d.residual = s.residual; d.out = s.out; d.acc = s.acc;
+        d.n = (int)s.n;
+        end += (int)((row_blocks(s.n) + RB - 1) / RB);
+        d.rb_end = end;
+    }
+    for (int j = nproj; j < GEMV_MAX_PROJ; ++j) p.proj[j] = p.proj[nproj - 1];
+    p.nproj = nproj; p.a = a; p.a_scale = a_scale; p.m = (int)m; p.k = (int)k; p.kt_count = (int)k_tiles(k);
+    if (end == 0) return BITNET_HIP_OK;
+    const int tgroups = (int)((m + 15) / 16), total = end * tgroups;
+    const unsigned grid = (unsigned)((total + 7) / 8 * 8);
+    const size_t lds = 16 * (k + 16);
+    if (p.kt_count <= 12) {
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mfma_tg_kernel<RB, 3>),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 16 * (3072 + 16));
+        BITNET_HIP_TRY(attr);
+        hipLaunchKernelGGL((gemv_mfma_tg_kernel<RB, 3>), dim3(grid), dim3(256), lds, stream, p.a, p.k, p.m, p.kt_count, end, tgroups, p);
+    } else {
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mfma_tg_kernel<RB, 8>),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 16 * (8192 + 16));
+        BITNET_HIP_TRY(attr);
+        hipLaunchKernelGGL((gemv_mfma_tg_kernel<RB, 8>), dim3(grid), dim3(256), lds, stream, p.a, p.k, p.m, p.kt_count, end, tgroups, p);
+    }
+    BITNET_HIP_CHECK_LAUNCH("gemv_mfma_tg_kernel");
+    return BITNET_HIP_OK;
+}
+
 }  // namespace
 
 int launch_gemv_rowmajor(const uint8_t *packed, const int8_t *a, int32_t *out, size_t n, size_t k,
@@ -1185,6 +1376,15 @@ int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const f
         // take more row blocks when there are plenty of them, so that fewer workgroups re-read the activations.
         size_t blocks = 0;
         for (int j = 0; j < nproj; ++j) blocks += row_blocks(projs[j].n);
+        if (m > 16 && k % TILE_K == 0 && k <= 8192 && (reinterpret_cast<uintptr_t>(a) & 15) == 0 && m * k < ((size_t)1 << 32)) {
+            // token groups of 16 with their rows in LDS.  Row blocks per workgroup: the activation copy is what a workgroup
+            // spends its time on, so a workgroup takes several row blocks once there are enough workgroups for every
+            // compute unit (LDS holds three workgroups up to k = 3072, one above).
+            const size_t tgroups = (m + 15) / 16, slots = k <= 3072 ? 768 : 256;
+            if (blocks * tgroups > 2 * slots) return launch_mfma_tg<4>(projs, nproj, a, a_scale, m, k, stream);
+            if (blocks * tgroups > slots) return launch_mfma_tg<2>(projs, nproj, a, a_scale, m, k, stream);
+            return launch_mfma_tg<1>(projs, nproj, a, a_scale, m, k, stream);
+        }
         for (size_t t0 = 0; t0 < m; t0 += (size_t)GEMV_MFMA_MAX_M) {
             GemvProj sub[GEMV_MAX_PROJ];
             const size_t rows = m - t0 < (size_t)GEMV_MFMA_MAX_M ? m - t0 : (size_t)GEMV_MFMA_MAX_M;

@@ -378,6 +378,26 @@ def test_batched_decode_sweep_bit_exact(m, n, k):
     assert np.array_equal(host(out), orc.epilogue(acc_ref, ws, a_scale))
 
 
+@pytest.mark.parametrize("m", [17, 31, 32, 33, 48, 80, 95])
+@pytest.mark.parametrize("n,k", [(33, 256), (650, 2560), (6912, 2560), (2560, 6912), (100, 8192), (4000, 3072), (1000, 3328),
+                                 (640, 2564)])
+def test_token_group_gemv_bit_exact(m, n, k):
+    """17 to 95 tokens: token groups of 16 with their rows in LDS (k a multiple of 256 up to 8192; one, two or four row
+    blocks per workgroup; a last token group that is not full; output rows that do not fill a row block), with bias and
+    residual; k = 2564 takes the gathering kernel instead."""
+    rng = np.random.default_rng(m * 131 + n + k)
+    packed, ws, a, a_scale = make_problem(rng, m, n, k, outliers=True)
+    tiled = bh.retile_weights(dev(packed), n, k)
+    bias = rng.standard_normal(n, dtype=f32)
+    res = rng.standard_normal((m, n), dtype=f32)
+    acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale), bias=dev(bias), residual=dev(res))
+    acc_ref = orc.gemm_w2a8(packed, a, n)
+    assert np.array_equal(host(acc), acc_ref)
+    assert np.array_equal(host(out), orc.epilogue(acc_ref, ws, a_scale, bias, res))
+    acc2, _ = bh.matmul_w2a8(tiled, dev(a), n, want_out=False)
+    assert np.array_equal(host(acc2), acc_ref)
+
+
 @pytest.mark.parametrize("n,k", [(6912, 2560), (2560, 6912)])
 @pytest.mark.parametrize("with_sum", [True, False], ids=["lds_direct_kernel", "register_staged_kernel"])
 def test_prefill_gemm_full_size(n, k, with_sum):
@@ -629,7 +649,7 @@ def test_bitlinear_forward_shapes_bias_norm_and_layouts():
     assert np.array_equal(host(layer_p.forward(dev(x))), ref0)
 
 
-@pytest.mark.parametrize("m", [1, 3, 8, 20, 200, 1100])
+@pytest.mark.parametrize("m", [1, 3, 8, 20, 40, 64, 200, 1100])
 def test_forward_multi_matches_single_forwards(m):
     """q/k/v-style: several layers on one input give exactly what each layer gives alone, and what the oracle gives.
     (m = 200 and 1100: the projections share launches of the 64 x 160 and of the eight-wavefront prefill GEMM.)"""
