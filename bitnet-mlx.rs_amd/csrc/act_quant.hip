@@ -366,7 +366,137 @@ void launch_mode(const ActQuantParams &p, bool vec, hipStream_t s)
 
 inline bool aligned(const void *ptr, size_t a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }
 
+// ---- absmax_quantize_activations: one scale for the whole tensor (bitnet-quant/src/quantization/activations.rs:530-641) ----
+//
+// Pass 1: abs-max / min / max of the tensor (order-free).  Pass 2: q = ternary code or 8-bit value of x / scale and the
+// squared error of every element, summed in f64 over "rows" of 4096 consecutive elements (lane l of a wavefront adds
+// elements l, l + 64, ... of its row in ascending order, butterfly 32..1; the row sums are combined the same way by
+// one wavefront).  Elements past the end count as +0.
+struct AbsmaxState {
+    float abs_max, lo, hi, scale;
+};
+
+__global__ __launch_bounds__(256) void absmax_partial_kernel(const float *x, size_t n, float *part /* [3][gridDim.x] */)
+{
+    float am = 0.0f, lo = __builtin_inff(), hi = -__builtin_inff();
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        const float v = x[i];
+        am = fmaxf(am, fabsf(v));
+        lo = fminf(lo, v);
+        hi = fmaxf(hi, v);
+    }
+    __shared__ float sh[3][4];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        am = fmaxf(am, __shfl_xor(am, off, 64));
+        lo = fminf(lo, __shfl_xor(lo, off, 64));
+        hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+    }
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { sh[0][wave] = am; sh[1][wave] = lo; sh[2][wave] = hi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        part[blockIdx.x] = fmaxf(fmaxf(sh[0][0], sh[0][1]), fmaxf(sh[0][2], sh[0][3]));
+        part[gridDim.x + blockIdx.x] = fminf(fminf(sh[1][0], sh[1][1]), fminf(sh[1][2], sh[1][3]));
+        part[2 * gridDim.x + blockIdx.x] = fmaxf(fmaxf(sh[2][0], sh[2][1]), fmaxf(sh[2][2], sh[2][3]));
+    }
+}
+
+__global__ __launch_bounds__(64) void absmax_scale_kernel(const float *part, int blocks, int precision, AbsmaxState *state)
+{
+    float am = 0.0f, lo = __builtin_inff(), hi = -__builtin_inff();
+    for (int b = threadIdx.x; b < blocks; b += 64) {
+        am = fmaxf(am, part[b]);
+        lo = fminf(lo, part[blocks + b]);
+        hi = fmaxf(hi, part[2 * blocks + b]);
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        am = fmaxf(am, __shfl_xor(am, off, 64));
+        lo = fminf(lo, __shfl_xor(lo, off, 64));
+        hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+    }
+    if (threadIdx.x == 0) {
+        float scale = 1.0f;  // abs_max below f32::EPSILON: no division by (almost) zero, activations.rs:557-561
+        if (!(am < 1.1920929e-07f)) scale = precision == BITNET_HIP_PRECISION_EIGHT_BIT ? f32_div(am, 127.0f) : am;
+        state->abs_max = am; state->lo = lo; state->hi = hi; state->scale = scale;
+    }
+}
+
+// one wavefront per row of 4096 elements
+__global__ __launch_bounds__(256) void absmax_quantize_kernel(const float *x, size_t n, size_t rows, int precision,
+                                                              const AbsmaxState *state, int8_t *q, double *row_sums)
+{
+    const int lane = threadIdx.x;
+    const size_t row = (size_t)blockIdx.x * blockDim.y + threadIdx.y;
+    if (row >= rows) return;
+    const float scale = state->scale;
+    double s = 0.0;
+    for (size_t i = row * 4096 + lane; i < (row + 1) * 4096 && i < n; i += 64) {
+        const float v = x[i];
+        const float scaled = f32_div(v, scale);
+        float qv;
+        if (precision == BITNET_HIP_PRECISION_EIGHT_BIT) {
+            float c = scaled > 127.0f ? 127.0f : scaled;
+            c = c < -127.0f ? -127.0f : c;
+            qv = roundf(c);  // halves away from zero, as f32::round
+        } else {
+            qv = scaled > 0.5f ? 1.0f : (scaled < -0.5f ? -1.0f : 0.0f);
+        }
+        const int8_t qi = (qv != qv) ? (int8_t)0 : (int8_t)qv;
+        q[i] = qi;
+        const float d = v - f32_mul((float)qi, scale);
+        s = s + (double)f32_mul(d, d);
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) s = s + __shfl_xor(s, off, 64);
+    if (lane == 0) row_sums[row] = s;
+}
+
+__global__ __launch_bounds__(64) void absmax_finish_kernel(const double *row_sums, size_t rows, size_t n, const AbsmaxState *state,
+                                                           float *stats)
+{
+    double s = 0.0;
+    for (size_t r = threadIdx.x; r < rows; r += 64) s = s + row_sums[r];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) s = s + __shfl_xor(s, off, 64);
+    if (threadIdx.x == 0) {
+        stats[0] = state->scale;
+        stats[1] = n ? (float)(s / (double)n) : 0.0f;
+        stats[2] = state->lo;
+        stats[3] = state->hi;
+    }
+}
+
 }  // namespace
+
+size_t absmax_quantize_scratch_bytes(size_t n)
+{
+    const size_t rows = (n + 4095) / 4096;
+    return 256 + sizeof(float) * 3 * 1024 + sizeof(double) * (rows ? rows : 1);
+}
+
+int launch_absmax_quantize(const float *x, size_t n, int precision, void *scratch, int8_t *q, float *stats, hipStream_t stream)
+{
+    AbsmaxState *state = static_cast<AbsmaxState *>(scratch);
+    float *part = reinterpret_cast<float *>(static_cast<uint8_t *>(scratch) + 256);
+    double *row_sums = reinterpret_cast<double *>(static_cast<uint8_t *>(scratch) + 256 + sizeof(float) * 3 * 1024);
+    const size_t rows = (n + 4095) / 4096;
+    int blocks = (int)((n + 255) / 256);
+    blocks = blocks < 1 ? 1 : (blocks > 1024 ? 1024 : blocks);
+    hipLaunchKernelGGL(absmax_partial_kernel, dim3(blocks), dim3(256), 0, stream, x, n, part);
+    BITNET_HIP_CHECK_LAUNCH("absmax_partial_kernel");
+    hipLaunchKernelGGL(absmax_scale_kernel, dim3(1), dim3(64), 0, stream, part, blocks, precision, state);
+    BITNET_HIP_CHECK_LAUNCH("absmax_scale_kernel");
+    if (rows) {
+        hipLaunchKernelGGL(absmax_quantize_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(64, 4), 0, stream, x, n, rows, precision,
+                           state, q, row_sums);
+        BITNET_HIP_CHECK_LAUNCH("absmax_quantize_kernel");
+    }
+    hipLaunchKernelGGL(absmax_finish_kernel, dim3(1), dim3(64), 0, stream, row_sums, rows, n, state, stats);
+    BITNET_HIP_CHECK_LAUNCH("absmax_finish_kernel");
+    return BITNET_HIP_OK;
+}
 
 int launch_act_quant(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
                      size_t gqa_group, size_t head_dim, const float *gamma, float eps, int sum_order,

@@ -307,6 +307,22 @@ int bitnet_hip_quantize_activations_i8(const float *x, const float *x2, size_t l
                             a_sum, y_f32, as_stream(stream));
 }
 
+int bitnet_hip_absmax_quantize_activations(const float *x, size_t count, int precision, int8_t *values, float *stats,
+                                           void *stream)
+{
+    if (precision != BITNET_HIP_PRECISION_ONE_FIVE_FIVE_BIT && precision != BITNET_HIP_PRECISION_EIGHT_BIT)
+        return fail(BITNET_HIP_UNSUPPORTED, "absmax_quantize_activations: unsupported precision %d", precision);
+    if (!stats) return fail(BITNET_HIP_NULL_POINTER, "absmax_quantize_activations: stats is required");
+    if (count != 0 && (!x || !values)) return fail(BITNET_HIP_NULL_POINTER, "absmax_quantize_activations: null buffer");
+    DeviceTemp scratch;
+    int rc = scratch.alloc(absmax_quantize_scratch_bytes(count));
+    if (rc != BITNET_HIP_OK) return rc;
+    rc = launch_absmax_quantize(x, count, precision, scratch.ptr, values, stats, as_stream(stream));
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipStreamSynchronize(as_stream(stream)));  // the scratch is released on return
+    return BITNET_HIP_OK;
+}
+
 // ---- lookup-table kernels ----------------------------------------------------------------------------
 
 int bitnet_hip_lookup_compute(int kind, const int8_t *weights, size_t n_weights, const float *inputs, size_t n_inputs,
@@ -1026,6 +1042,154 @@ int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t
 {
     if (!dec) return fail(BITNET_HIP_NULL_POINTER, "decoder_decode: null argument");
     return bitnet_hip_decoder_decode_layers(dec, 0, dec->layers, x_in, m, x_out, q_last, k_last, stream);
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------------------------
+// Inference backend (InferenceBackend, bitnet-inference/src/engine/mod.rs:126-138)
+// ---------------------------------------------------------------------------------------------------
+struct bitnet_hip_backend {
+    int device = 0;
+    size_t total_mem = 0;
+    bitnet_hip_decoder *model = nullptr;  // not owned
+    float *stage_in = nullptr, *stage_out = nullptr;  // [max_tokens, hidden] each
+    size_t stage_bytes = 0;
+    std::mutex lock;  // execute_batch calls share the staging buffers
+
+    ~bitnet_hip_backend()
+    {
+        if (stage_in) (void)hipFree(stage_in);
+        if (stage_out) (void)hipFree(stage_out);
+    }
+};
+
+namespace {
+size_t decoder_device_bytes(const bitnet_hip_decoder *d)
+{
+    size_t total = 0;
+    for (const bitnet_hip_bitlinear *p : d->proj) {
+        total += (p->in_features * p->out_features + 3) / 4 + tiled_bytes(p->out_features, p->in_features) + sizeof(float);
+        if (p->use_bias) total += sizeof(float) * p->out_features;
+    }
+    const size_t kv = d->kv_heads * d->head_dim, widest = d->hidden > d->ffn ? d->hidden : d->ffn, t = d->max_tokens;
+    total += sizeof(float) * d->layers * 2 * d->hidden;                                        // norms
+    total += t * widest + 2 * sizeof(float) * t;                                               // a8, a_scale, a_sum
+    total += sizeof(float) * t * (d->hidden /*q*/ + 2 * kv + d->hidden /*x1*/ + 2 * d->ffn + d->hidden /*ping*/);
+    return total;
+}
+}  // namespace
+
+extern "C" {
+
+int bitnet_hip_backend_create(int device, bitnet_hip_backend **backend)
+{
+    if (!backend) return fail(BITNET_HIP_NULL_POINTER, "backend_create: backend is NULL");
+    *backend = nullptr;
+    int rc = bitnet_hip_init(device);
+    if (rc != BITNET_HIP_OK) return rc;
+    bitnet_hip_backend *b = new (std::nothrow) bitnet_hip_backend;
+    if (!b) return fail(BITNET_HIP_MEMORY_ERROR, "backend_create: out of host memory");
+    b->device = device;
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) {
+        delete b;
+        return fail(BITNET_HIP_DEVICE_ERROR, "backend_create: hipGetDeviceProperties failed: %s", hipGetErrorString(e));
+    }
+    b->total_mem = prop.totalGlobalMem;
+    *backend = b;
+    return BITNET_HIP_OK;
+}
+
+void bitnet_hip_backend_destroy(bitnet_hip_backend *backend) { delete backend; }
+
+int bitnet_hip_backend_optimize_model(bitnet_hip_backend *backend, bitnet_hip_decoder *model)
+{
+    if (!backend || !model) return fail(BITNET_HIP_NULL_POINTER, "backend_optimize_model: null argument");
+    for (const bitnet_hip_bitlinear *p : model->proj)
+        if (!p->has_weights) return fail(BITNET_HIP_NOT_INITIALIZED, "backend_optimize_model: a projection of the model has no weights yet");
+    std::lock_guard<std::mutex> guard(backend->lock);
+    const size_t bytes = sizeof(float) * model->max_tokens * model->hidden;
+    if (bytes > backend->stage_bytes) {
+        BITNET_HIP_TRY(hipDeviceSynchronize());
+        if (backend->stage_in) (void)hipFree(backend->stage_in);
+        if (backend->stage_out) (void)hipFree(backend->stage_out);
+        backend->stage_in = backend->stage_out = nullptr;
+        backend->stage_bytes = 0;
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&backend->stage_in), bytes);
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&backend->stage_out), bytes);
+        if (e != hipSuccess) return fail(BITNET_HIP_MEMORY_ERROR, "backend_optimize_model: hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+        backend->stage_bytes = bytes;
+    }
+    backend->model = model;
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_backend_execute_batch(bitnet_hip_backend *backend, const float *const *inputs, const size_t *rows,
+                                     size_t count, float *const *outputs, void *stream)
+{
+    if (!backend) return fail(BITNET_HIP_NULL_POINTER, "backend_execute_batch: backend is NULL");
+    std::lock_guard<std::mutex> guard(backend->lock);
+    bitnet_hip_decoder *dec = backend->model;
+    if (!dec) return fail(BITNET_HIP_NOT_INITIALIZED, "backend_execute_batch: no model bound (optimize_model first)");
+    if (count == 0) return BITNET_HIP_OK;
+    if (!inputs || !rows || !outputs) return fail(BITNET_HIP_NULL_POINTER, "backend_execute_batch: null argument");
+    const size_t H = dec->hidden, cap = dec->max_tokens;
+    hipStream_t s = as_stream(stream);
+    for (size_t i = 0; i < count; ++i) {
+        if (rows[i] != 0 && (!inputs[i] || !outputs[i])) return fail(BITNET_HIP_NULL_POINTER, "backend_execute_batch: input or output %zu is NULL", i);
+        if (rows[i] > cap) {
+            size_t e[2] = {cap, H}, a[2] = {rows[i], H};
+            return fail_shape(e, 2, a, 2, "rows of one input exceed the model's max_tokens");
+        }
+    }
+    size_t i = 0;
+    while (i < count) {
+        // the longest run of inputs from i on whose rows fit one pass
+        size_t j = i, total = 0;
+        while (j < count && total + rows[j] <= cap) total += rows[j++];
+        if (total == 0) { i = j > i ? j : i + 1; continue; }
+        if (j == i + 1) {  // one input: no staging
+            int rc = bitnet_hip_decoder_decode(dec, inputs[i], rows[i], outputs[i], nullptr, nullptr, stream);
+            if (rc != BITNET_HIP_OK) return rc;
+        } else {
+            size_t at = 0;
+            for (size_t t = i; t < j; ++t) {
+                if (rows[t] == 0) continue;
+                BITNET_HIP_TRY(hipMemcpyAsync(backend->stage_in + at * H, inputs[t], sizeof(float) * rows[t] * H, hipMemcpyDeviceToDevice, s));
+                at += rows[t];
+            }
+            int rc = bitnet_hip_decoder_decode(dec, backend->stage_in, total, backend->stage_out, nullptr, nullptr, stream);
+            if (rc != BITNET_HIP_OK) return rc;
+            at = 0;
+            for (size_t t = i; t < j; ++t) {
+                if (rows[t] == 0) continue;
+                BITNET_HIP_TRY(hipMemcpyAsync(outputs[t], backend->stage_out + at * H, sizeof(float) * rows[t] * H, hipMemcpyDeviceToDevice, s));
+                at += rows[t];
+            }
+        }
+        i = j;
+    }
+    return BITNET_HIP_OK;
+}
+
+size_t bitnet_hip_backend_get_memory_usage(const bitnet_hip_backend *backend)
+{
+    if (!backend || !backend->model) return 0;
+    return decoder_device_bytes(backend->model) + 2 * backend->stage_bytes;
+}
+
+int bitnet_hip_backend_capabilities(const bitnet_hip_backend *backend, int *supports_batching, int *supports_streaming,
+                                    size_t *max_batch_size, size_t *memory_limit, int *device)
+{
+    if (!backend) return fail(BITNET_HIP_NULL_POINTER, "backend_capabilities: backend is NULL");
+    if (supports_batching) *supports_batching = 1;
+    if (supports_streaming) *supports_streaming = 0;
+    if (max_batch_size) *max_batch_size = backend->model ? backend->model->max_tokens : 0;
+    if (memory_limit) *memory_limit = backend->total_mem;
+    if (device) *device = backend->device;
+    return BITNET_HIP_OK;
 }
 
 }  // extern "C"

@@ -19,6 +19,11 @@ int launch_act_quant(const float *x, const float *x2, size_t ldx, size_t m, size
                      size_t gqa_group, size_t head_dim, const float *gamma, float eps, int sum_order,
                      int8_t *q, float *a_scale, int32_t *a_sum, float *y, hipStream_t stream);
 
+// absmax_quantize_activations (activations.rs:530-641): one scale per tensor; scratch of absmax_quantize_scratch_bytes(n)
+// bytes; stats: 4 floats (scale, mse, min, max)
+size_t absmax_quantize_scratch_bytes(size_t n);
+int launch_absmax_quantize(const float *x, size_t n, int precision, void *scratch, int8_t *q, float *stats, hipStream_t stream);
+
 // weight_prep.hip
 int launch_pack_2bit(const int8_t *q, size_t count, uint8_t *packed, hipStream_t stream);
 int launch_unpack_2bit(const uint8_t *packed, size_t count, int8_t *q, hipStream_t stream);

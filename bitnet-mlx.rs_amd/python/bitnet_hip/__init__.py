@@ -89,6 +89,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_init": (i32, [i32]),
         "bitnet_hip_device_info": (i32, [C.c_char_p, sz, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz)]),
         "bitnet_hip_quantize_activations_i8": (i32, [vp, vp, sz, sz, sz, i32, sz, sz, vp, f32, i32, vp, vp, vp, vp, vp]),
+        "bitnet_hip_absmax_quantize_activations": (i32, [vp, sz, i32, vp, vp, vp]),
         "bitnet_hip_lookup_compute": (i32, [i32, vp, sz, vp, sz, vp, sz, vp]),
         "bitnet_hip_packed_size": (sz, [sz]),
         "bitnet_hip_pack_ternary_2bit": (i32, [vp, sz, vp, vp]),
@@ -125,6 +126,12 @@ def load_library() -> C.CDLL:
         "bitnet_hip_decoder_set_norm": (i32, [vp, sz, i32, vp, i32, vp]),
         "bitnet_hip_decoder_weight_bytes": (sz, [vp]),
         "bitnet_hip_decoder_decode": (i32, [vp, vp, sz, vp, vp, vp, vp]),
+        "bitnet_hip_backend_create": (i32, [i32, C.POINTER(vp)]),
+        "bitnet_hip_backend_destroy": (None, [vp]),
+        "bitnet_hip_backend_optimize_model": (i32, [vp, vp]),
+        "bitnet_hip_backend_execute_batch": (i32, [vp, C.POINTER(vp), C.POINTER(sz), sz, C.POINTER(vp), vp]),
+        "bitnet_hip_backend_get_memory_usage": (sz, [vp]),
+        "bitnet_hip_backend_capabilities": (i32, [vp, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz), C.POINTER(sz), C.POINTER(i32)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -234,6 +241,73 @@ def quantize_activations_i8(x: torch.Tensor, gamma: Optional[torch.Tensor] = Non
                                                   _ptr(gamma), eps, sum_order, _ptr(q), _ptr(a_scale), _ptr(a_sum),
                                                   _ptr(y), _stream(stream)))
     return q, a_scale, a_sum, y
+
+
+class QuantizationPrecision:
+    """The precisions of QuantizationPrecision (bitnet-quant/src/quantization/mod.rs) that absmax_quantize_activations
+    implements."""
+    OneFiveFiveBit, EightBit = 0, 1
+
+
+@dataclass
+class QuantizedActivation:
+    """QuantizedActivation (activations.rs:95-112): values (int8, the tensor's shape), scales (one f32 on the device),
+    zero_points (None: symmetric), original_shape, stats (scale_factor, quantization_error, min_value, max_value,
+    elements_count, compression_ratio), sequence_length (None)."""
+    values: torch.Tensor
+    scales: torch.Tensor
+    zero_points: Optional[torch.Tensor]
+    original_shape: tuple
+    precision: int
+    stats: dict
+    sequence_length: Optional[int] = None
+
+    def effective_bit_width(self) -> float:
+        return 1.58 if self.precision == QuantizationPrecision.OneFiveFiveBit else 8.0
+
+    def memory_footprint(self) -> int:
+        return self.values.numel() * self.values.element_size() + self.scales.numel() * self.scales.element_size()
+
+
+def absmax_quantize_activations(activations: torch.Tensor, precision: Optional[int] = None, stream=None) -> QuantizedActivation:
+    """absmax_quantize_activations (activations.rs:530-641): ONE scale for the whole tensor, ternary codes by default
+    (precision None = OneFiveFiveBit) or 8-bit values.  The values keep their sign (the reference's U8 cast of the 8-bit
+    branch loses it).  The per-token int8 quantiser of the BitLinear path is quantize_activations_i8."""
+    _dev(activations, torch.float32, "activations")
+    precision = QuantizationPrecision.OneFiveFiveBit if precision is None else precision
+    values = torch.empty(activations.shape, dtype=torch.int8, device=activations.device)
+    stats = torch.empty((4,), dtype=torch.float32, device=activations.device)
+    _check(load_library().bitnet_hip_absmax_quantize_activations(_ptr(activations), activations.numel(), precision,
+                                                                 _ptr(values), _ptr(stats), _stream(stream)))
+    scale, mse, lo, hi = stats.cpu().tolist()
+    bits = 1.58 if precision == QuantizationPrecision.OneFiveFiveBit else 8.0
+    info = {"elements_count": activations.numel(), "quantization_error": mse, "compression_ratio": 32.0 / bits,
+            "min_value": lo, "max_value": hi, "scale_factor": scale, "zero_point": None}
+    return QuantizedActivation(values, stats[0:1], None, tuple(activations.shape), precision, info)
+
+
+class ActivationQuantizer:
+    """The quantize / dequantize pair of ActivationQuantizer (activations.rs:169-199) over absmax_quantize_activations."""
+
+    def __init__(self, precision: int = QuantizationPrecision.OneFiveFiveBit):
+        self.precision = precision
+
+    def validate_activations(self, activations: torch.Tensor):
+        if activations.numel() == 0:
+            raise BitLinearError(QUANTIZATION_ERROR, "Activation tensor is empty")
+        if activations.dtype != torch.float32:
+            raise BitLinearError(QUANTIZATION_ERROR, "Activation tensor must be float type")
+
+    def quantize(self, activations: torch.Tensor) -> QuantizedActivation:
+        self.validate_activations(activations)
+        return absmax_quantize_activations(activations, self.precision)
+
+    def quantize_dynamic(self, activations: torch.Tensor) -> QuantizedActivation:
+        return self.quantize(activations)
+
+    def dequantize(self, quantized: QuantizedActivation) -> torch.Tensor:
+        """values * scales (a host-side convenience through torch; not on the forward path)."""
+        return quantized.values.to(torch.float32) * quantized.scales
 
 
 def packed_size(count: int) -> int:
@@ -708,3 +782,68 @@ class DecoderProjections:
         _check(load_library().bitnet_hip_decoder_decode_layers(self._h, lo, hi, _ptr(x), m, _ptr(out), _ptr(q), _ptr(k),
                                                                _stream(stream)))
         return (out, q, k) if want_qk else out
+
+
+@dataclass
+class BackendCapabilities:
+    """BackendCapabilities (bitnet-inference/src/engine/mod.rs:141-148)."""
+    supports_batching: bool
+    supports_streaming: bool
+    max_batch_size: int
+    memory_limit: Optional[int]
+    device_type: str
+
+
+class HipInferenceBackend:
+    """InferenceBackend (bitnet-inference/src/engine/mod.rs:126-138) for this path: execute_batch runs every input
+    through the bound decoder stack; the model is bound with optimize_model."""
+
+    def __init__(self, device: int = 0):
+        h = C.c_void_p()
+        _check(load_library().bitnet_hip_backend_create(device, C.byref(h)))
+        self._h = h
+        self._model = None
+
+    def __del__(self):
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.bitnet_hip_backend_destroy(self._h)
+            self._h = None
+
+    def optimize_model(self, model: "DecoderProjections"):
+        _check(load_library().bitnet_hip_backend_optimize_model(self._h, model._h))
+        self._model = model  # keeps the decoder alive while the backend refers to it
+
+    def execute_batch(self, inputs: Sequence[torch.Tensor], stream=None):
+        if self._model is None:  # the library reports it the way the trait's implementations do
+            _check(load_library().bitnet_hip_backend_execute_batch(self._h, None, None, 0, None, _stream(stream)))
+        hidden = self._model.hidden
+        mats = []
+        for i, t in enumerate(inputs):
+            _dev(t, torch.float32, f"input {i}")
+            t2 = t.reshape(1, -1) if t.dim() == 1 else t
+            if t2.dim() != 2 or t2.shape[1] != hidden:
+                raise BitLinearError(SHAPE_MISMATCH, f"input {i}", [t2.shape[0] if t2.dim() else 1, hidden], list(t.shape))
+            mats.append(t2)
+        outs = [torch.empty_like(t) for t in mats]
+        n = len(mats)
+        ins = (C.c_void_p * n)(*[t.data_ptr() for t in mats])
+        rows = (C.c_size_t * n)(*[t.shape[0] for t in mats])
+        ous = (C.c_void_p * n)(*[t.data_ptr() for t in outs])
+        _check(load_library().bitnet_hip_backend_execute_batch(self._h, ins, rows, n, ous, _stream(stream)))
+        return [o.reshape(t.shape) for o, t in zip(outs, inputs)]
+
+    def get_memory_usage(self) -> int:
+        return int(load_library().bitnet_hip_backend_get_memory_usage(self._h))
+
+    def capabilities(self) -> BackendCapabilities:
+        sb, ss, dv = C.c_int(0), C.c_int(0), C.c_int(0)
+        mb, ml = C.c_size_t(0), C.c_size_t(0)
+        _check(load_library().bitnet_hip_backend_capabilities(self._h, C.byref(sb), C.byref(ss), C.byref(mb), C.byref(ml), C.byref(dv)))
+        return BackendCapabilities(bool(sb.value), bool(ss.value), mb.value, ml.value or None, f"hip:{dv.value}")
+
+
+def create_backend(device: str = "hip:0") -> HipInferenceBackend:
+    """InferenceEngine::create_backend (bitnet-inference/src/api/mod.rs:426-460) for a HIP device string "hip:N"."""
+    if not device.startswith("hip"):
+        raise BitLinearError(UNSUPPORTED, f"this library serves HIP devices only, not {device!r}")
+    return HipInferenceBackend(int(device.split(":")[1]) if ":" in device else 0)

@@ -11,6 +11,10 @@ pub struct bitnet_hip_bitlinear {
 pub struct bitnet_hip_decoder {
     _private: [u8; 0],
 }
+#[repr(C)]
+pub struct bitnet_hip_backend {
+    _private: [u8; 0],
+}
 
 pub const BITNET_HIP_OK: c_int = 0;
 pub const BITNET_HIP_SHAPE_MISMATCH: c_int = 1;
@@ -37,6 +41,8 @@ pub const BITNET_HIP_TERNARY_REF_DETSTE: c_int = 6;
 pub const BITNET_HIP_INPUT_PLAIN: c_int = 0;
 pub const BITNET_HIP_INPUT_RELU2_MUL: c_int = 1;
 pub const BITNET_HIP_INPUT_GQA_BROADCAST: c_int = 2;
+pub const BITNET_HIP_PRECISION_ONE_FIVE_FIVE_BIT: c_int = 0;
+pub const BITNET_HIP_PRECISION_EIGHT_BIT: c_int = 1;
 pub const BITNET_HIP_LOOKUP_TERNARY: c_int = 0;
 pub const BITNET_HIP_LOOKUP_I2S: c_int = 1;
 
@@ -50,6 +56,8 @@ extern "C" {
                                               input_mode: c_int, gqa_group: usize, head_dim: usize, gamma: *const f32,
                                               eps: f32, sum_order: c_int, q: *mut i8, a_scale: *mut f32,
                                               a_sum: *mut i32, y_f32: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_absmax_quantize_activations(x: *const f32, count: usize, precision: c_int, values: *mut i8,
+                                                  stats: *mut f32, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_lookup_compute(kind: c_int, weights: *const i8, n_weights: usize, inputs: *const f32,
                                      n_inputs: usize, output: *mut f32, n_output: usize, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_packed_size(count: usize) -> usize;
@@ -126,4 +134,13 @@ extern "C" {
     pub fn bitnet_hip_decoder_decode_layers(dec: *mut bitnet_hip_decoder, layer_begin: usize, layer_end: usize,
                                             x_in: *const f32, m: usize, x_out: *mut f32, q_last: *mut f32,
                                             k_last: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_backend_create(device: c_int, backend: *mut *mut bitnet_hip_backend) -> c_int;
+    pub fn bitnet_hip_backend_destroy(backend: *mut bitnet_hip_backend);
+    pub fn bitnet_hip_backend_optimize_model(backend: *mut bitnet_hip_backend, model: *mut bitnet_hip_decoder) -> c_int;
+    pub fn bitnet_hip_backend_execute_batch(backend: *mut bitnet_hip_backend, inputs: *const *const f32, rows: *const usize,
+                                            count: usize, outputs: *const *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_backend_get_memory_usage(backend: *const bitnet_hip_backend) -> usize;
+    pub fn bitnet_hip_backend_capabilities(backend: *const bitnet_hip_backend, supports_batching: *mut c_int,
+                                           supports_streaming: *mut c_int, max_batch_size: *mut usize,
+                                           memory_limit: *mut usize, device: *mut c_int) -> c_int;
 }

@@ -106,6 +106,21 @@ int bitnet_hip_quantize_activations_i8(const float *x, const float *x2, size_t l
                                        const float *gamma, float eps, int sum_order, int8_t *q,
                                        float *a_scale, int32_t *a_sum, float *y_f32, void *stream);
 
+/* QuantizationPrecision values absmax_quantize_activations supports (bitnet-quant/src/quantization/mod.rs). */
+#define BITNET_HIP_PRECISION_ONE_FIVE_FIVE_BIT 0 /* ternary: q = [x/scale > 0.5] - [x/scale < -0.5], scale = abs_max */
+#define BITNET_HIP_PRECISION_EIGHT_BIT 1         /* q = round(clamp(x/scale, -127, 127)), scale = abs_max / 127 */
+
+/* One scale for the whole tensor:
+ *   replaces absmax_quantize_activations (bitnet-quant/src/quantization/activations.rs:530-641), the body behind
+ *   QuantizedActivation / DynamicActivationQuantizer (:95-112,203-454).
+ *   x [count] f32 (any shape, flattened);  values [count] int8 out;  stats 4 f32 out (device): scale (abs_max below
+ *   f32::EPSILON gives 1.0), quantization_error = mean((x - q*scale)^2), min_value, max_value (QuantizationStats,
+ *   :609-626).  Anything but the two precisions above is BITNET_HIP_UNSUPPORTED (UnsupportedPrecision, :603-607).
+ *   The reference casts its 8-bit result to U8 (:599), which zeroes every negative value; values stay signed here.
+ *   The per-token int8 quantiser of the BitLinear path is bitnet_hip_quantize_activations_i8, not this function. */
+int bitnet_hip_absmax_quantize_activations(const float *x, size_t count, int precision, int8_t *values, float *stats,
+                                           void *stream);
+
 /* ---- lookup-table kernels --------------------------------------------------------------------- */
 
 #define BITNET_HIP_LOOKUP_TERNARY 0 /* weights {-1,0,+1}, anything else counts as 0 */
@@ -338,6 +353,37 @@ int bitnet_hip_decoder_decode(bitnet_hip_decoder *dec, const float *x_in, size_t
 int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin, size_t layer_end,
                                      const float *x_in, size_t m, float *x_out, float *q_last, float *k_last,
                                      void *stream);
+/* ---- inference backend -------------------------------------------------------------------------------- */
+
+typedef struct bitnet_hip_backend bitnet_hip_backend; /* opaque; the InferenceBackend of this path */
+
+/* The plug-in point InferenceEngine::create_backend selects a backend at (bitnet-inference/src/api/mod.rs:426-460):
+ *   replaces CpuInferenceBackend::new / MetalInferenceBackend::new behind the trait InferenceBackend
+ *   (bitnet-inference/src/engine/mod.rs:126-138; CPU implementation engine/cpu_backend.rs:203-260).
+ * Selects `device` (as bitnet_hip_init) and prepares an empty backend. */
+int bitnet_hip_backend_create(int device, bitnet_hip_backend **backend);
+void bitnet_hip_backend_destroy(bitnet_hip_backend *backend);
+/* InferenceBackend::optimize_model (engine/mod.rs:131): binds the model this backend executes, a decoder stack whose
+ * projections hold their weights (the decoder stays owned by the caller and must outlive the backend's use of it), and
+ * allocates the staging buffers of execute_batch for up to the decoder's max_tokens rows. */
+int bitnet_hip_backend_optimize_model(bitnet_hip_backend *backend, bitnet_hip_decoder *model);
+/* InferenceBackend::execute_batch(&[Tensor]) -> Vec<Tensor> (engine/mod.rs:128): `count` inputs, input i a [rows[i], hidden]
+ * f32 DEVICE matrix, output i a [rows[i], hidden] f32 DEVICE matrix owned by the caller: the hidden states after the
+ * bound decoder stack.  inputs / rows / outputs are HOST arrays.  Inputs whose rows together fit the decoder's
+ * max_tokens share one pass over the weights (the reference fans the inputs out over host threads,
+ * cpu_backend.rs:206-238); every row's result is independent of what it is batched with.  NOT_INITIALIZED before
+ * optimize_model; SHAPE_MISMATCH if one input alone exceeds max_tokens. */
+int bitnet_hip_backend_execute_batch(bitnet_hip_backend *backend, const float *const *inputs, const size_t *rows,
+                                     size_t count, float *const *outputs, void *stream);
+/* InferenceBackend::get_memory_usage (engine/mod.rs:134): device bytes held by the bound model (packed and re-tiled
+ * weights, scales, norms, activation buffers) and by the backend's staging buffers; 0 before optimize_model. */
+size_t bitnet_hip_backend_get_memory_usage(const bitnet_hip_backend *backend);
+/* InferenceBackend::capabilities (engine/mod.rs:137; BackendCapabilities :141-148).  HOST outputs, each may be NULL:
+ * supports_batching (1), supports_streaming (0), max_batch_size (rows per pass: the bound decoder's max_tokens, 0 before
+ * optimize_model), memory_limit (the device's total memory), device (the HIP device ordinal). */
+int bitnet_hip_backend_capabilities(const bitnet_hip_backend *backend, int *supports_batching, int *supports_streaming,
+                                    size_t *max_batch_size, size_t *memory_limit, int *device);
+
 #ifdef __cplusplus
 }
 #endif

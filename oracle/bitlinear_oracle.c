@@ -21,6 +21,10 @@
  *   orc_gemv_w2a8 / orc_gemm_w2a8        pinned: reference 3x4 GEMV / 2x3x2 GEMM vectors + brute force
  *   orc_quantize_activations_i8          pinned by invariants (max|q|=127, oddness, zero rows, exact ties);
  *                                        the reference holds no exact-value vector for it
+ *   orc_absmax_quantize_activations      pinned: the reference's own vectors (scale 100/127 for [100,-50,25,-75], scale 4
+ *                                        for [4,-2,1,-3], signs of [3,-3,0.1,-0.1], zeros, statistics) + an
+ *                                        independent numpy model; the U8 cast of the 8-bit branch is a reference
+ *                                        defect that is not reproduced
  *   orc_rmsnorm                          the reference holds NO fixture: pinned by closed forms (constant
  *                                        rows, one-hot rows), scale equivariance and an f64 bound; the
  *                                        bits of the ORC_SUM_BLOCK256 order are a declaration of this build
@@ -175,6 +179,51 @@ void orc_rmsnorm_quantize_i8(const float *x, const float *g, float eps, size_t m
         orc_quantize_activations_i8(y, 1, k, q + r * k, a_scale + r, row_sum ? row_sum + r : NULL);
     }
     free(y);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * A2  absmax_quantize_activations: one scale for the whole tensor.
+ *   reference: bitnet-quant/src/quantization/activations.rs:530-641
+ *   abs_max = max|x|;  scale = abs_max < f32::EPSILON ? 1.0 : (1.58-bit: abs_max, 8-bit: abs_max / 127)   (:557-570)
+ *   1.58-bit: q = [x / scale > 0.5] - [x / scale < -0.5]                                                   (:573-592)
+ *   8-bit:    q = round(clamp(x / scale, -127, 127))                                                       (:594-601)
+ *   stats: scale, mse = mean((x - q * scale)^2), min, max                                                  (:609-626)
+ * precision: 0 = OneFiveFiveBit (the function's default), 1 = EightBit.
+ * The reference then stores the 8-bit values with `to_dtype(DType::U8)` (:599), which turns every negative
+ * value into 0: a defect that is not reproduced, q stays signed.  The mean is carried in f64 over "rows" of 4096
+ * consecutive elements in the order of orc_tensor_sum_f64 (elements past the end count as +0) and rounded once.
+ * stats receives 4 floats. */
+static double orc_tensor_sum_f64(const float *v, size_t rows, size_t cols);
+void orc_absmax_quantize_activations(const float *x, size_t n, int precision, int8_t *q, float *stats)
+{
+    float abs_max = 0.0f, lo = INFINITY, hi = -INFINITY;
+    for (size_t i = 0; i < n; ++i) {
+        abs_max = fmaxf(abs_max, fabsf(x[i]));
+        lo = fminf(lo, x[i]);
+        hi = fmaxf(hi, x[i]);
+    }
+    float scale = 1.0f;
+    if (!(abs_max < 1.1920929e-07f)) scale = precision == 1 ? abs_max / 127.0f : abs_max;
+    size_t rows = (n + 4095) / 4096;
+    float *sq = (float *)calloc(rows ? rows * 4096 : 1, sizeof(float));
+    for (size_t i = 0; i < n; ++i) {
+        float scaled = x[i] / scale;
+        float qv;
+        if (precision == 1) {
+            float c = scaled > 127.0f ? 127.0f : scaled;
+            c = c < -127.0f ? -127.0f : c;
+            qv = roundf(c);
+        } else {
+            qv = scaled > 0.5f ? 1.0f : (scaled < -0.5f ? -1.0f : 0.0f);
+        }
+        q[i] = (qv != qv) ? 0 : (int8_t)qv;
+        float deq = (float)q[i] * scale;
+        float d = x[i] - deq;
+        sq[i] = d * d;
+    }
+    float mse = n ? (float)(orc_tensor_sum_f64(sq, rows, 4096) / (double)n) : 0.0f;
+    free(sq);
+    stats[0] = scale; stats[1] = mse; stats[2] = lo; stats[3] = hi;
 }
 
 /* ------------------------------------------------------------------------------------------------

@@ -98,6 +98,18 @@ def rmsnorm_quantize_i8(x, g, eps, order=SUM_BLOCK256):
     return q, s, rs
 
 
+PRECISION_ONE_FIVE_FIVE_BIT, PRECISION_EIGHT_BIT = 0, 1
+
+
+def absmax_quantize_activations(x, precision=PRECISION_ONE_FIVE_FIVE_BIT):
+    """absmax_quantize_activations (activations.rs:530-641): returns (q int8 with x's shape, dict scale/mse/min/max)."""
+    x = _f32(x)
+    q = np.empty(x.shape, dtype=np.int8)
+    stats = np.zeros(4, dtype=np.float32)
+    lib().orc_absmax_quantize_activations(_p(x), _sz(x.size), C.c_int(int(precision)), _p(q), _p(stats))
+    return q, dict(zip(("scale", "mse", "min", "max"), stats))
+
+
 def round_clip(x, lo=-1.0, hi=1.0) -> float:
     return float(lib().orc_round_clip(C.c_float(x), C.c_float(lo), C.c_float(hi)))
 

@@ -160,6 +160,33 @@ def test_reference_weight_pipeline_through_the_layer():
     assert not host(z.values).any() and host(z.scales)[0] == 1.0
 
 
+# ---- A2 ------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("precision", [bh.QuantizationPrecision.OneFiveFiveBit, bh.QuantizationPrecision.EightBit])
+@pytest.mark.parametrize("shape", [(4,), (32, 128), (3, 5, 7), (300, 4096 + 17), (1, 1)])
+def test_absmax_quantize_activations_bit_exact(precision, shape):
+    """absmax_quantize_activations (one scale per tensor): values, scale, error, min and max equal to the oracle's."""
+    rng = np.random.default_rng(len(shape) * 10 + precision)
+    x = (rng.standard_normal(shape) * 3).astype(f32)
+    if x.size >= 4:
+        x.flat[:4] = [100.0, -50.0, 25.0, -75.0]  # the reference's vector (activations.rs:815-840)
+    got = bh.absmax_quantize_activations(dev(x), precision)
+    q_ref, st = orc.absmax_quantize_activations(x, precision)
+    assert np.array_equal(host(got.values), q_ref) and got.original_shape == shape
+    assert f32(got.stats["scale_factor"]) == st["scale"] and host(got.scales)[0] == st["scale"]
+    assert f32(got.stats["quantization_error"]) == st["mse"]
+    assert f32(got.stats["min_value"]) == st["min"] and f32(got.stats["max_value"]) == st["max"]
+    assert got.stats["elements_count"] == x.size and got.stats["compression_ratio"] > 1.0 and got.zero_points is None
+    assert got.effective_bit_width() == (1.58 if precision == 0 else 8.0)
+    deq = bh.ActivationQuantizer(precision).dequantize(got)
+    assert tuple(deq.shape) == shape
+    zeros = bh.absmax_quantize_activations(torch.zeros(2, 2, device="cuda"), precision)
+    assert not host(zeros.values).any() and zeros.stats["scale_factor"] == 1.0
+    with pytest.raises(bh.BitLinearError) as ei:
+        bh.absmax_quantize_activations(dev(x), 7)
+    assert ei.value.kind == "Unsupported"
+
+
 # ---- R1 + A1 -------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("m,k", [(1, 2560), (4, 2560), (3, 6912), (2, 1024), (5, 4096), (2, 8192), (2, 12000),
@@ -1013,6 +1040,44 @@ def test_gguf_ternary_tensor_ingestion(n, k, layout):
     with pytest.raises(bh.BitLinearError) as ei:
         layer.load_gguf_ternary(torch.from_numpy(tensor[:-1].copy()), layout)
     assert ei.value.kind == "ShapeMismatch"
+
+
+# ---- inference backend ---------------------------------------------------------------------------------------
+
+def test_inference_backend_execute_batch_matches_per_input_oracle():
+    """HipInferenceBackend (InferenceBackend, engine/mod.rs:126-138): a batch of inputs of different row counts, each
+    result equal to the oracle's decoder chain on that input alone, however the inputs were grouped into passes."""
+    dims = (256, 512, 4, 2, 64)
+    rng = np.random.default_rng(77)
+    dec, ref = build_decoder(rng, 2, *dims, max_tokens=8)
+    backend = bh.create_backend("hip:0")
+    caps = backend.capabilities()
+    assert caps.supports_batching and not caps.supports_streaming and caps.max_batch_size == 0 and caps.device_type == "hip:0"
+    assert backend.get_memory_usage() == 0
+    with pytest.raises(bh.BitLinearError) as ei:
+        backend.execute_batch([dev(synth_activations(rng, 1, dims[0]))])
+    assert ei.value.kind == "NotInitialized"
+    backend.optimize_model(dec)
+    assert backend.capabilities().max_batch_size == 8 and backend.capabilities().memory_limit > 1 << 30
+    assert backend.get_memory_usage() > dec.weight_bytes() * 2
+    xs = [synth_activations(rng, r, dims[0]) for r in (1, 3, 2, 4, 8, 1, 1)]  # 1+3+2 | 4 | 8 | 1+1
+    outs = backend.execute_batch([dev(x) for x in xs])
+    assert len(outs) == len(xs)
+    for x, o in zip(xs, outs):
+        assert np.array_equal(host(o), oracle_stack(ref, x, *dims)[0])
+    one = backend.execute_batch([dev(xs[0][0])])  # a rank-1 input is one row
+    assert tuple(one[0].shape) == (dims[0],) and np.array_equal(host(one[0]), oracle_stack(ref, xs[0], *dims)[0][0])
+    assert backend.execute_batch([]) == []
+    with pytest.raises(bh.BitLinearError) as ei:
+        backend.execute_batch([dev(synth_activations(rng, 9, dims[0]))])
+    assert ei.value.kind == "ShapeMismatch"
+    with pytest.raises(bh.BitLinearError) as ei:
+        backend.execute_batch([dev(synth_activations(rng, 2, dims[0] + 4))])
+    assert ei.value.kind == "ShapeMismatch"
+    empty = bh.DecoderProjections(1, *dims, max_tokens=2)
+    with pytest.raises(bh.BitLinearError) as ei:
+        bh.HipInferenceBackend().optimize_model(empty)
+    assert ei.value.kind == "NotInitialized"
 
 
 # ---- C++ host mirror -----------------------------------------------------------------------------------------

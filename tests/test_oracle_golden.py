@@ -322,6 +322,50 @@ def test_reference_weight_methods_pick_their_factors():
     assert np.array_equal(q, q_m)
 
 
+# ---- A2: absmax_quantize_activations -----------------------------------------------------------------------
+
+def test_absmax_quantize_activations_reference_vectors():
+    for c in G["absmax_quantize_activations"]:
+        x = np.array(c["input"], dtype=f32)
+        prec = orc.PRECISION_EIGHT_BIT if c["precision"] == "EightBit" else orc.PRECISION_ONE_FIVE_FIVE_BIT
+        q, st = orc.absmax_quantize_activations(x, prec)
+        if "scale" in c:
+            want = f32(100.0) / f32(127.0) if c["scale"] == "100/127" else f32(c["scale"])
+            assert st["scale"] == want
+        if "abs_values_at_most" in c:
+            assert np.abs(q.astype(int)).max() <= c["abs_values_at_most"]
+            assert q.tolist() == [127, -64, 32, -95]  # halves away from zero: -63.5 -> -64; signs kept
+        if "sign_of_first_two" in c:
+            assert np.sign(q[:2]).tolist() == c["sign_of_first_two"]
+        if "elements_count" in c:
+            assert q.size == c["elements_count"] and st["scale"] > 0 and st["min"] <= st["max"]
+        if c.get("all_zero"):
+            assert not q.any() and st["scale"] == 1.0 and st["mse"] == 0.0
+
+
+@pytest.mark.parametrize("precision", [orc.PRECISION_ONE_FIVE_FIVE_BIT, orc.PRECISION_EIGHT_BIT])
+def test_absmax_quantize_activations_against_numpy_model(precision):
+    rng = np.random.default_rng(precision)
+    x = synth_activations(rng, 37, 300, outliers=True)
+    q, st = orc.absmax_quantize_activations(x, precision)
+    am = np.abs(x).max()
+    scale = f32(am) / f32(127.0) if precision == orc.PRECISION_EIGHT_BIT else f32(am)
+    assert st["scale"] == scale and st["min"] == x.min() and st["max"] == x.max()
+    scaled = x / scale  # f32 division, elementwise: the same single operation
+    if precision == orc.PRECISION_EIGHT_BIT:
+        c = np.clip(scaled, -127, 127)
+        want = (np.sign(c) * np.floor(np.abs(c) + f32(0.5))).astype(np.int8)  # half away from zero
+        tie_risk = np.abs(np.abs(c) - np.floor(np.abs(c)) - 0.5) < 1e-6  # |x| + 0.5 rounds differently only at a tie's edge
+        assert np.array_equal(q[~tie_risk], want[~tie_risk]) and np.abs(q.astype(int)).max() == 127
+    else:
+        assert np.array_equal(q, (scaled > 0.5).astype(np.int8) - (scaled < -0.5).astype(np.int8))
+    mse = ((x.astype(np.float64) - q.astype(np.float64) * float(scale)) ** 2).mean()
+    assert abs(float(st["mse"]) - mse) <= 1e-5 * mse
+    # a tensor of tiny values: the scale stays 1.0 (abs_max < f32::EPSILON)
+    q, st = orc.absmax_quantize_activations(np.array([1e-8, -1e-8], f32), precision)
+    assert st["scale"] == 1.0 and not q.any()
+
+
 # ---- G1 / G2: contraction ---------------------------------------------------------------------------
 
 @pytest.mark.parametrize("case", G["gemv"], ids=lambda c: f'{c["m"]}x{c["k"]}')
