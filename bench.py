@@ -8,7 +8,10 @@ decoder layer (hidden 2560, FFN 6912, 20 query / 5 KV heads): fused RMSNorm + in
 q/k/v and before gate/up, int8 quantisation before o and down, seven packed-ternary GEMVs with the scale
 epilogue.  Consecutive steps use the weights of consecutive layers of a 30-layer stack (521 MB of packed
 weights in total), so no step finds its weights in cache.  Inputs and weights are resident in HBM before
-the timed region.  value = packed-weight bytes streamed per second over the whole timed region.
+the timed region: an untimed pass over all 30 layers comes first (first touch of every weight page), then the
+warm-up steps, then the region of exactly K steps, which is run REPEATS times back to back; the line reports the
+median region (every region's time is listed under config.region_ms), so that a short run (--steps 20) and a long one
+agree.  value = packed-weight bytes streamed per second over that region, by the host's clock around it.
 
 The timed region contains one kernel family only, the decode GEMV with the activation quantiser fused into
 its prologue (four launches per step: q+k+v, o, gate+up, down), so the roofline of the dominant kernel comes
@@ -58,6 +61,7 @@ def time_events(torch, fn):
     return start.elapsed_time(stop)
 
 
+REPEATS = 7  # timed regions of --steps steps each; the median is reported
 LAUNCHES_PER_STEP = 4  # q+k+v | o | gate+up | down, each one gemv_fused16_kernel<MODE, NORM, NCHB, RBW> launch
 # HBM bytes per launch of that kernel from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (two runs of this
 # script with --no-extras --calibration-copy), each scaled by what the same counter reads for the plain
@@ -190,6 +194,24 @@ def stack_latency(bh, torch, dec, gen, reps=20):
     return out
 
 
+def sequential_order_decode(bh, torch, dec, gen, reps=20):
+    """The headline workload with the reference's literal RMSNorm summation order (one running f32 sum,
+    inference_integration.rs:476) instead of the build's declared block order: same stack, same steps."""
+    seq = bh.DecoderProjections(dec.layers, HIDDEN, FFN, Q_HEADS, KV_HEADS, HEAD_DIM, eps=1e-5, max_tokens=1,
+                                sum_order=bh.SUM_SEQUENTIAL)
+    for l in range(dec.layers):
+        for p in range(7):
+            packed, scale = dec.projection(l, p).get_quantized_weights()
+            seq.projection(l, p).set_quantized_weights(packed.cuda(), scale)
+    x = torch.randn((1, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
+    y = torch.empty_like(x)
+    seq.decode(x, out=y)
+    times = sorted(time_events(torch, lambda: [seq.decode(x, out=y) for _ in range(reps)]) / reps for _ in range(5))
+    ms = times[len(times) // 2]
+    return {"us_per_layer_step": round(ms * 1e3 / dec.layers, 2), "gbs_packed_weights": round(dec.weight_bytes() / (ms * 1e-3) / 1e9, 1),
+            "timed": f"median of 5 loops of {reps} 30-layer token steps"}
+
+
 def time_forward_graph(torch, bls, x, y, ws, replays=10):
     """Device time of one BitLinear.forward (quantiser + GEMV launches): one forward per layer of `bls` captured
     into a HIP graph and replayed, so that the host's per-call cost (about 10 us through ctypes) is not what is
@@ -229,42 +251,63 @@ def time_forward_graph(torch, bls, x, y, ws, replays=10):
         return ms, f"eager loop of {calls} calls (graph capture failed: {type(exc).__name__})"
 
 
-def cpu_baseline(torch, dec, budget_s=15.0):
-    """The reference's BitLinear::forward on the host cores: per call, materialise q*scale as f32 [N,K], then an
-    f32 GEMV (bitnet-quant/src/bitlinear/forward.rs:153-258), for the seven projections of one layer."""
+def cpu_baseline(torch, dec, budget_s=8.0):
+    """The reference's CPU BitLinear on the host cores, one layer's seven projections at batch 1, three restatements:
+    ref_f32  what BitLinear::forward executes per call: materialise q*scale as f32 [N,K], then an f32 GEMV
+             (bitnet-quant/src/bitlinear/forward.rs:153-258); the headline figure of this object, all cores
+    ref_simd the reference's ternary SIMD GEMV semantics: i8 weights widened to f32, FMA with f32 activations
+             (bitnet-quant/src/simd/matrix.rs:287-368,471-490)
+    oracle_i8 the int8 x ternary int32 path the GPU kernels reproduce (the oracle's BitLinear forward)
+    each on all cores and on one thread, a bounded sample each."""
     import numpy as np
 
     from oracle import oracle as orc
 
     cores = orc.cpu_threads()
-    orc.cpu_set_threads(cores)
     mats = []
     for p in range(7):
         n, k = dec.proj_shape(p)
         packed, scale = dec.projection(0, p).get_quantized_weights()
         q = orc.unpack_2bit(packed.numpy(), n * k).reshape(n, k)
-        mats.append((q, np.float32(scale), np.empty(n * k, dtype=np.float32), np.empty((1, n), dtype=np.float32)))
+        mats.append((q, np.float32(scale), np.empty(n * k, dtype=np.float32), np.empty((1, n), dtype=np.float32), packed.numpy()))
     rng = np.random.default_rng(0)
     x = {k: rng.standard_normal((1, k), dtype=np.float32) for k in (HIDDEN, FFN)}
 
-    def one_layer():
-        for q, s, wf, out in mats:
+    def ref_f32():
+        for q, s, wf, out, _ in mats:
             orc.cpu_ref_f32_forward(x[q.shape[1]], q, s, wf, out)
 
-    one_layer()
-    t0 = time.perf_counter()
-    reps = 0
-    while True:
-        one_layer()
-        reps += 1
-        if time.perf_counter() - t0 > budget_s or reps >= 200:
-            break
-    dt = (time.perf_counter() - t0) / reps
+    def ref_simd():
+        for q, s, _, out, _ in mats:
+            orc.cpu_ref_simd_gemv(q, x[q.shape[1]], out, s)
+
+    def oracle_i8():
+        for q, s, _, _, packed in mats:
+            orc.bitlinear_forward(x[q.shape[1]], packed, q.shape[0], s)
+
+    def sample(fn, threads, budget):
+        orc.cpu_set_threads(threads)
+        fn()
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            fn()
+            reps += 1
+            if time.perf_counter() - t0 > budget or reps >= 200:
+                break
+        dt = (time.perf_counter() - t0) / reps
+        return {"gbs": round(LAYER_BYTES / dt / 1e9, 3), "ms_per_layer": round(dt * 1e3, 3), "threads": threads, "passes": reps}
+
+    main_leg = sample(ref_f32, cores, budget_s)
+    variants = {"ref_f32_1_thread": sample(ref_f32, 1, 3.0),
+                "ref_simd_all_cores": sample(ref_simd, cores, 3.0), "ref_simd_1_thread": sample(ref_simd, 1, 3.0),
+                "oracle_i8_all_cores": sample(oracle_i8, cores, 3.0), "oracle_i8_1_thread": sample(oracle_i8, 1, 3.0)}
+    orc.cpu_set_threads(cores)
     return {
-        "value": round(LAYER_BYTES / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-        "sample": f"{reps} passes over one layer's 7 projections at batch 1 (dequantise to f32 + f32 GEMV per call, "
-                  f"{orc.cpu_isa()}), {dt * 1e3:.2f} ms per layer",
-        "ms_per_step": round(dt * 1e3, 3),
+        "value": main_leg["gbs"], "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": f"{main_leg['passes']} passes over one layer's 7 projections at batch 1 (dequantise to f32 + f32 GEMV per call, "
+                  f"{orc.cpu_isa()}), {main_leg['ms_per_layer']:.2f} ms per layer",
+        "ms_per_step": main_leg["ms_per_layer"], "variants": variants,
     }
 
 
@@ -315,16 +358,23 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    run_steps(0, LAYERS)  # residency: every layer's weights touched once, untimed
     run_steps(0, args.warmup)
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    start.record()
-    run_steps(args.warmup, args.steps)
-    stop.record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    event_ms = start.elapsed_time(stop)
+    regions = []  # (host seconds, event milliseconds) of each region of exactly args.steps steps
+    first = args.warmup
+    for _ in range(REPEATS):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        start.record()
+        run_steps(first, args.steps)
+        stop.record()
+        torch.cuda.synchronize()
+        regions.append((time.perf_counter() - t0, start.elapsed_time(stop)))
+        first += args.steps
+    regions_sorted = sorted(regions)
+    elapsed, event_ms = regions_sorted[len(regions_sorted) // 2]  # the median region by host time
 
     value = args.steps * LAYER_BYTES / elapsed / 1e9
     line = {
@@ -336,13 +386,16 @@ def main():
                                "(hidden 2560, ffn 6912, 20q/5kv heads), weights rotating over a 30-layer stack; "
                                "a step = one layer = four kernel launches, up to 30 consecutive steps per host call",
                    "bytes_per_step": LAYER_BYTES, "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-                   "event_ms_per_step": round(event_ms / args.steps, 5), "device": bh.device_info()},
+                   "event_ms_per_step": round(event_ms / args.steps, 5), "repeats": REPEATS, "reported": "median region",
+                   "region_ms": [round(r[0] * 1e3, 4) for r in regions], "sum_order": "block256 (the build's declared order)",
+                   "device": bh.device_info()},
     }
     line["roofline"] = decode_roofline(event_ms, args.steps)
     if not args.no_extras:
         line["gemv_only"] = gemv_only(bh, torch, dec, gen, reps=5)
         line["prefill"] = prefill_rates(bh, torch, dec, gen, reps=5)
         line["other_configs"] = stack_latency(bh, torch, dec, gen)
+        line["other_configs"]["decode_layer_b1_sum_order_sequential"] = sequential_order_decode(bh, torch, dec, gen)
         if not args.no_cpu_baseline:
             line["cpu_baseline"] = cpu_baseline(torch, dec)
     print(json.dumps(line))

@@ -8,6 +8,11 @@
 //   bitnet::BitLinear                 bitnet-quant/src/bitlinear/layer.rs:82-109,113-179,299-352 and the
 //                                     BitLinearForward trait, bitnet-quant/src/bitlinear/forward.rs:14-51
 //   bitnet::TernaryProcessor          bitnet-inference/src/engine/ternary_operations.rs:56-172
+//   bitnet::QuantizedActivation, absmax_quantize_activations
+//                                     bitnet-quant/src/quantization/activations.rs:95-112,530-641
+//   bitnet::WeightQuantizationConfig, BitNetWeightQuantizer, QuantizedWeight
+//                                     bitnet-quant/src/quantization/weights.rs:58-95,158-175,341-611
+//   bitnet::HipInferenceBackend       the InferenceBackend trait, bitnet-inference/src/engine/mod.rs:126-148
 //   bitnet::BitLinearLayer            bitnet-inference/src/engine/transformer_layers.rs:68-202
 //   bitnet::FeedForwardNetwork        bitnet-inference/src/engine/transformer_layers.rs:553-623
 //
@@ -19,6 +24,7 @@
 
 #include <cstdint>
 #include <memory>
+#include <mutex>
 #include <optional>
 #include <string>
 #include <utility>
@@ -131,7 +137,11 @@ public:
         if (rc != BITNET_HIP_OK) return last_error(rc);
         return std::shared_ptr<BitLinear>(new BitLinear(config, std::move(layer_name), h));
     }
-    ~BitLinear() { bitnet_hip_bitlinear_destroy(handle_); }
+    ~BitLinear()
+    {
+        bitnet_hip_bitlinear_destroy(handle_);
+        if (workspace_) (void)hipFree(workspace_);
+    }
     BitLinear(const BitLinear &) = delete;
     BitLinear &operator=(const BitLinear &) = delete;
 
@@ -160,9 +170,22 @@ public:
         if (!out_dims.empty()) out_dims.back() = config_.out_features;
         auto out = DeviceTensor::zeros(out_dims.empty() ? std::vector<size_t>{config_.out_features} : out_dims);
         if (out.is_err()) return out;
+        // the scratch for the quantised activations is kept by the layer and grown on demand: no allocation per call
+        size_t rows = input.dims().empty() ? 0 : input.elem_count() / (input.dims().back() ? input.dims().back() : 1);
+        std::lock_guard<std::mutex> guard(workspace_lock_);
+        const size_t need = bitnet_hip_bitlinear_workspace_size(handle_, rows);
+        if (need > workspace_bytes_) {
+            (void)hipDeviceSynchronize();
+            if (workspace_) (void)hipFree(workspace_);
+            workspace_ = nullptr;
+            workspace_bytes_ = 0;
+            if (hipMalloc(&workspace_, need) != hipSuccess)
+                return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
+            workspace_bytes_ = need;
+        }
         int rc = bitnet_hip_bitlinear_forward(handle_, input.data(), input.dims().data(), (int)input.dims().size(), gamma,
                                               config_.rms_norm_eps, config_.sum_order, nullptr, out.unwrap().data(),
-                                              nullptr, 0, nullptr, nullptr, nullptr, stream);
+                                              workspace_, workspace_bytes_, nullptr, nullptr, nullptr, stream);
         if (rc != BITNET_HIP_OK) return last_error(rc);
         return out;
     }
@@ -179,6 +202,9 @@ private:
     BitLinearConfig config_;
     std::string layer_name_;
     bitnet_hip_bitlinear *handle_;
+    mutable std::mutex workspace_lock_;  // forward calls of one layer share the scratch: one at a time through this mirror
+    mutable void *workspace_ = nullptr;
+    mutable size_t workspace_bytes_ = 0;
 };
 
 // TernaryProcessor: per-token int8 absmax quantisation and the ternary matmul on top of it.
@@ -287,6 +313,199 @@ public:
         (void)hipStreamSynchronize(stream);
         return out;
     }
+};
+
+// absmax_quantize_activations: ONE scale for the whole tensor, ternary codes (the default precision) or 8-bit values.
+enum class QuantizationPrecision { OneFiveFiveBit = BITNET_HIP_PRECISION_ONE_FIVE_FIVE_BIT, EightBit = BITNET_HIP_PRECISION_EIGHT_BIT };
+struct QuantizationStats {
+    size_t elements_count = 0;
+    float quantization_error = 0.f, compression_ratio = 0.f, min_value = 0.f, max_value = 0.f, scale_factor = 1.f;
+};
+struct QuantizedActivation {
+    std::shared_ptr<int8_t> values;  // device, original_shape elements (signed: the reference's U8 cast loses the sign)
+    float scales = 1.f;              // the one scale of the tensor
+    std::vector<size_t> original_shape;
+    QuantizationPrecision precision = QuantizationPrecision::OneFiveFiveBit;
+    QuantizationStats stats;
+    float effective_bit_width() const { return precision == QuantizationPrecision::OneFiveFiveBit ? 1.58f : 8.0f; }
+};
+inline Result<QuantizedActivation> absmax_quantize_activations(const DeviceTensor &activations,
+                                                               std::optional<QuantizationPrecision> precision = std::nullopt,
+                                                               hipStream_t stream = nullptr)
+{
+    QuantizedActivation q;
+    q.precision = precision.value_or(QuantizationPrecision::OneFiveFiveBit);
+    q.original_shape = activations.dims();
+    const size_t n = activations.elem_count();
+    int8_t *v = nullptr;
+    float *st = nullptr;
+    if (hipMalloc(reinterpret_cast<void **>(&v), n ? n : 1) != hipSuccess || hipMalloc(reinterpret_cast<void **>(&st), 4 * sizeof(float)) != hipSuccess)
+        return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
+    q.values.reset(v, [](int8_t *p) { (void)hipFree(p); });
+    std::shared_ptr<float> st_guard(st, [](float *p) { (void)hipFree(p); });
+    int rc = bitnet_hip_absmax_quantize_activations(activations.data(), n, static_cast<int>(q.precision), v, st, stream);
+    if (rc != BITNET_HIP_OK) return last_error(rc);
+    float h[4];
+    (void)hipMemcpy(h, st, sizeof h, hipMemcpyDeviceToHost);
+    q.scales = h[0];
+    q.stats = {n, h[1], 32.0f / q.effective_bit_width(), h[2], h[3], h[0]};
+    return q;
+}
+
+// BitNetWeightQuantizer::quantize with its whole configuration (weights.rs:568-611).
+enum class TernaryMethod { MeanThreshold = 0, MedianThreshold, AdaptiveThreshold, OptimalThreshold, DetSTE };
+struct WeightQuantizationConfig {
+    bool normalize_weights = true;
+    float outlier_threshold = 3.0f;
+    TernaryMethod ternary_method = TernaryMethod::MeanThreshold;
+    std::optional<float> custom_threshold_factor;
+};
+struct QuantizedWeight {
+    std::vector<int8_t> values;   // ternary, [rows * cols]
+    std::vector<uint8_t> packed;  // the reference's 2-bit bytes
+    float scales = 1.f;
+    std::vector<size_t> original_shape;
+};
+class BitNetWeightQuantizer {
+public:
+    explicit BitNetWeightQuantizer(WeightQuantizationConfig c = {}) : config_(c) {}
+    const WeightQuantizationConfig &config() const { return config_; }
+    // weights: [rows, cols] f32 on the device
+    Result<QuantizedWeight> quantize(const DeviceTensor &weights, hipStream_t stream = nullptr) const
+    {
+        if (weights.dims().size() < 2)
+            return BitLinearError{BitLinearError::QuantizationError, "Weight tensor must have at least 2 dimensions", {}, {}};
+        const size_t rows = weights.dims()[0], cols = weights.elem_count() / (rows ? rows : 1), n = rows * cols;
+        uint8_t *packed = nullptr;
+        int8_t *q = nullptr;
+        float *scale = nullptr;
+        if (hipMalloc(reinterpret_cast<void **>(&packed), (n + 3) / 4 + 1) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&q), n + 1) != hipSuccess || hipMalloc(reinterpret_cast<void **>(&scale), sizeof(float)) != hipSuccess)
+            return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
+        int rc = bitnet_hip_quantize_weights_reference(weights.data(), rows, cols, static_cast<int>(config_.ternary_method),
+                                                       config_.normalize_weights, config_.outlier_threshold,
+                                                       config_.custom_threshold_factor.value_or(0.0f), packed, scale, q, nullptr, stream);
+        QuantizedWeight out;
+        if (rc == BITNET_HIP_OK) {
+            out.values.resize(n);
+            out.packed.resize((n + 3) / 4);
+            out.original_shape = weights.dims();
+            (void)hipMemcpy(out.values.data(), q, n, hipMemcpyDeviceToHost);
+            (void)hipMemcpy(out.packed.data(), packed, out.packed.size(), hipMemcpyDeviceToHost);
+            (void)hipMemcpy(&out.scales, scale, sizeof(float), hipMemcpyDeviceToHost);
+        }
+        (void)hipFree(packed); (void)hipFree(q); (void)hipFree(scale);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return out;
+    }
+
+private:
+    WeightQuantizationConfig config_;
+};
+
+// The projections of a stack of decoder blocks, and the InferenceBackend that executes batches through them.
+class DecoderProjections {
+public:
+    static Result<std::shared_ptr<DecoderProjections>> create(size_t layers, size_t hidden, size_t ffn, size_t q_heads, size_t kv_heads,
+                                                              size_t head_dim, float eps, size_t max_tokens)
+    {
+        bitnet_hip_decoder *h = nullptr;
+        int rc = bitnet_hip_decoder_create(layers, hidden, ffn, q_heads, kv_heads, head_dim, eps, BITNET_HIP_SUM_BLOCK256, max_tokens, &h);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        auto d = std::shared_ptr<DecoderProjections>(new DecoderProjections());
+        d->handle_ = h; d->hidden = hidden; d->max_tokens = max_tokens; d->layers = layers;
+        return d;
+    }
+    ~DecoderProjections() { bitnet_hip_decoder_destroy(handle_); }
+    // latent f32 weights [out, in] of projection `proj` (BITNET_HIP_PROJ_*) of block `layer`, host memory
+    Result<Unit> update_weights(size_t layer, int proj, const std::vector<float> &w, size_t rows, size_t cols)
+    {
+        bitnet_hip_bitlinear *bl = nullptr;
+        int rc = bitnet_hip_decoder_projection(handle_, layer, proj, &bl);
+        if (rc == BITNET_HIP_OK)
+            rc = bitnet_hip_bitlinear_set_weights_f32(bl, w.data(), rows, cols, BITNET_HIP_LAYOUT_OUT_IN, 0,
+                                                      BITNET_HIP_TERNARY_ABSMEAN_ROUNDCLIP, 0.5f, nullptr);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return Unit{};
+    }
+    Result<DeviceTensor> decode(const DeviceTensor &x) const
+    {
+        auto out = DeviceTensor::zeros(x.dims());
+        if (out.is_err()) return out;
+        int rc = bitnet_hip_decoder_decode(handle_, x.data(), x.dims().empty() ? 0 : x.dims()[0], out.unwrap().data(), nullptr, nullptr, nullptr);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return out;
+    }
+    bitnet_hip_decoder *handle() const { return handle_; }
+    size_t hidden = 0, max_tokens = 0, layers = 0;
+
+private:
+    DecoderProjections() = default;
+    bitnet_hip_decoder *handle_ = nullptr;
+};
+
+struct BackendCapabilities {
+    bool supports_batching = false, supports_streaming = false;
+    size_t max_batch_size = 0;
+    std::optional<size_t> memory_limit;
+    int device = 0;
+};
+class HipInferenceBackend {
+public:
+    static Result<std::shared_ptr<HipInferenceBackend>> create(int device = 0)
+    {
+        bitnet_hip_backend *h = nullptr;
+        int rc = bitnet_hip_backend_create(device, &h);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        auto b = std::shared_ptr<HipInferenceBackend>(new HipInferenceBackend());
+        b->handle_ = h;
+        return b;
+    }
+    ~HipInferenceBackend() { bitnet_hip_backend_destroy(handle_); }
+    Result<Unit> optimize_model(std::shared_ptr<DecoderProjections> model)
+    {
+        int rc = bitnet_hip_backend_optimize_model(handle_, model ? model->handle() : nullptr);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        model_ = std::move(model);
+        return Unit{};
+    }
+    // execute_batch(&[Tensor]) -> Vec<Tensor>: every input [rows, hidden]
+    Result<std::vector<DeviceTensor>> execute_batch(const std::vector<DeviceTensor> &inputs, hipStream_t stream = nullptr) const
+    {
+        std::vector<DeviceTensor> outs;
+        std::vector<const float *> in_ptrs;
+        std::vector<float *> out_ptrs;
+        std::vector<size_t> rows;
+        for (const DeviceTensor &t : inputs) {
+            if (model_ && (t.dims().size() != 2 || t.dims()[1] != model_->hidden))
+                return BitLinearError{BitLinearError::ShapeMismatch, "execute_batch input", {t.dims().empty() ? 1 : t.dims()[0], model_->hidden}, t.dims()};
+            auto o = DeviceTensor::zeros(t.dims());
+            if (o.is_err()) return o.unwrap_err();
+            outs.push_back(o.unwrap());
+            in_ptrs.push_back(t.data());
+            out_ptrs.push_back(outs.back().data());
+            rows.push_back(t.dims().empty() ? 0 : t.dims()[0]);
+        }
+        int rc = bitnet_hip_backend_execute_batch(handle_, in_ptrs.data(), rows.data(), inputs.size(), out_ptrs.data(), stream);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return outs;
+    }
+    size_t get_memory_usage() const { return bitnet_hip_backend_get_memory_usage(handle_); }
+    BackendCapabilities capabilities() const
+    {
+        BackendCapabilities c;
+        int sb = 0, ss = 0;
+        size_t ml = 0;
+        (void)bitnet_hip_backend_capabilities(handle_, &sb, &ss, &c.max_batch_size, &ml, &c.device);
+        c.supports_batching = sb != 0; c.supports_streaming = ss != 0;
+        if (ml) c.memory_limit = ml;
+        return c;
+    }
+
+private:
+    HipInferenceBackend() = default;
+    bitnet_hip_backend *handle_ = nullptr;
+    std::shared_ptr<DecoderProjections> model_;
 };
 
 }  // namespace bitnet

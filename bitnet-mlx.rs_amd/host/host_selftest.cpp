@@ -110,6 +110,64 @@ int main()
         auto y2 = net.down_proj->forward(ht.unwrap());
         CHECK(y.unwrap().to_vec() == y2.unwrap().to_vec());
     }
+    {  // absmax_quantize_activations: the reference's vectors (activations.rs:815-865)
+        auto x = DeviceTensor::from_vec({100.0f, -50.0f, 25.0f, -75.0f}, {4});
+        auto q8 = absmax_quantize_activations(x.unwrap(), QuantizationPrecision::EightBit);
+        CHECK(q8.is_ok() && q8.unwrap().scales == 100.0f / 127.0f && q8.unwrap().effective_bit_width() == 8.0f);
+        int8_t h[4];
+        (void)hipMemcpy(h, q8.unwrap().values.get(), 4, hipMemcpyDeviceToHost);
+        CHECK(h[0] == 127 && h[1] == -64 && h[2] == 32 && h[3] == -95);
+        auto y = DeviceTensor::from_vec({4.0f, -2.0f, 1.0f, -3.0f}, {4});
+        auto qt = absmax_quantize_activations(y.unwrap());
+        CHECK(qt.is_ok() && qt.unwrap().stats.scale_factor == 4.0f && qt.unwrap().stats.elements_count == 4);
+        (void)hipMemcpy(h, qt.unwrap().values.get(), 4, hipMemcpyDeviceToHost);
+        CHECK(h[0] == 1 && h[1] == 0 && h[2] == 0 && h[3] == -1);  // |x| / 4 > 0.5 only for 4 and -3
+    }
+    {  // BitNetWeightQuantizer: the packed bytes loaded into a layer give the forward the quantiser's codes imply
+        const size_t n = 48, k = 256;
+        auto w = DeviceTensor::from_vec(randn(n * k, 21, 1.0f), {n, k});
+        BitNetWeightQuantizer quantizer;  // normalise, clip at 3.0, MeanThreshold
+        auto qw = quantizer.quantize(w.unwrap());
+        CHECK(qw.is_ok() && qw.unwrap().scales > 0.0f && qw.unwrap().values.size() == n * k);
+        bool ternary = true, packs = true;
+        for (size_t i = 0; i < n * k; ++i) {
+            const int v = qw.unwrap().values[i];
+            ternary = ternary && v >= -1 && v <= 1;
+            packs = packs && ((qw.unwrap().packed[i / 4] >> (2 * (i % 4))) & 3) == v + 1;
+        }
+        CHECK(ternary && packs);
+        BitLinearConfig c; c.in_features = k; c.out_features = n; c.ternary_method = BITNET_HIP_TERNARY_REF_MEAN_THRESHOLD; c.threshold_factor = 0.0f;
+        auto layer = BitLinear::create(c, "refq");
+        CHECK(layer.unwrap()->update_weights(w.unwrap().to_vec(), n, k).is_ok());
+        float ws = 0.f;
+        std::vector<uint8_t> held(n * k / 4);
+        CHECK(bitnet_hip_bitlinear_get_quantized(layer.unwrap()->handle(), &ws, held.data(), held.size()) == BITNET_HIP_OK);
+        CHECK(ws == qw.unwrap().scales && held == qw.unwrap().packed);
+    }
+    {  // HipInferenceBackend::execute_batch == one decode per input
+        auto dec = DecoderProjections::create(2, 256, 512, 4, 2, 64, 1e-5f, 8);
+        CHECK(dec.is_ok());
+        const size_t outs[7] = {256, 128, 128, 256, 512, 512, 256}, ins[7] = {256, 256, 256, 256, 256, 256, 512};
+        for (size_t l = 0; l < 2; ++l)
+            for (int p = 0; p < 7; ++p)
+                CHECK(dec.unwrap()->update_weights(l, p, randn(outs[p] * ins[p], 30 + (unsigned)(7 * l + p), 0.02f), outs[p], ins[p]).is_ok());
+        auto backend = HipInferenceBackend::create(0);
+        CHECK(backend.is_ok() && backend.unwrap()->get_memory_usage() == 0);
+        std::vector<DeviceTensor> batch;
+        for (size_t r : {size_t(1), size_t(3), size_t(2), size_t(8)}) batch.push_back(DeviceTensor::from_vec(randn(r * 256, 50 + (unsigned)r, 1.0f), {r, 256}).unwrap());
+        auto none = backend.unwrap()->execute_batch(batch);
+        CHECK(none.is_err() && none.unwrap_err().kind == BitLinearError::NotInitialized);
+        CHECK(backend.unwrap()->optimize_model(dec.unwrap()).is_ok());
+        auto caps = backend.unwrap()->capabilities();
+        CHECK(caps.supports_batching && !caps.supports_streaming && caps.max_batch_size == 8 && caps.memory_limit.has_value());
+        CHECK(backend.unwrap()->get_memory_usage() > 0);
+        auto res = backend.unwrap()->execute_batch(batch);
+        CHECK(res.is_ok() && res.unwrap().size() == batch.size());
+        for (size_t i = 0; res.is_ok() && i < batch.size(); ++i) {
+            auto one = dec.unwrap()->decode(batch[i]);
+            CHECK(one.is_ok() && one.unwrap().to_vec() == res.unwrap()[i].to_vec());
+        }
+    }
     std::printf(failures ? "host selftest: %d FAILED\n" : "host selftest: all passed\n", failures);
     return failures ? 1 : 0;
 }

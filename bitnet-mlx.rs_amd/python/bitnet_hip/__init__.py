@@ -231,8 +231,12 @@ def quantize_activations_i8(x: torch.Tensor, gamma: Optional[torch.Tensor] = Non
     """Fused RMSNorm (if gamma) + per-token absmax int8 quantisation of a [m, k] f32 matrix."""
     lib = load_library()
     _dev(x, torch.float32, "x")
+    if x.dim() != 2:
+        raise BitLinearError(SHAPE_MISMATCH, "x must be a [m, k] matrix", [1, x.shape[-1] if x.dim() else 1], list(x.shape))
     m, src_cols = x.shape
     k = src_cols * gqa_group if input_mode == INPUT_GQA_BROADCAST else src_cols
+    _opt_dev(gamma, torch.float32, "gamma", k, x)
+    _opt_dev(x2, torch.float32, "x2", x.numel(), x)
     q = torch.empty((m, k), dtype=torch.int8, device=x.device)
     a_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
     a_sum = torch.empty((m,), dtype=torch.int32, device=x.device) if want_sum else None
@@ -459,9 +463,16 @@ def matmul_w2a8(tiled: torch.Tensor, a: torch.Tensor, n: int, w_scale: Optional[
     """acc[m,n] (int32) and/or out[m,n] (f32) from re-tiled weights and int8 activations [m, k]."""
     _dev(tiled, torch.uint8, "tiled")
     _dev(a, torch.int8, "a")
+    if a.dim() != 2:
+        raise BitLinearError(SHAPE_MISMATCH, "a must be a [m, k] matrix", [1, a.shape[-1] if a.dim() else 1], list(a.shape))
     m, k = a.shape
     if tiled.numel() < tiled_size(n, k):
         raise BitLinearError(SHAPE_MISMATCH, "tiled buffer too short", [tiled_size(n, k)], [tiled.numel()])
+    _opt_dev(w_scale, torch.float32, "w_scale", 1, a)
+    _opt_dev(a_scale, torch.float32, "a_scale", m, a)
+    _opt_dev(a_sum, torch.int32, "a_sum", m, a)
+    _opt_dev(bias, torch.float32, "bias", n, a)
+    _opt_dev(residual, torch.float32, "residual", m * n, a)
     acc = torch.empty((m, n), dtype=torch.int32, device=a.device) if want_acc else None
     out = torch.empty((m, n), dtype=torch.float32, device=a.device) if want_out else None
     _check(load_library().bitnet_hip_matmul_w2a8(_ptr(tiled), _ptr(a), _ptr(a_sum), m, n, k, _ptr(acc), _ptr(w_scale), _ptr(a_scale),
@@ -634,6 +645,7 @@ class BitLinear:
         """BitLinearForward::forward (forward.rs:55-92).  x: [m,in] or [b,s,in] f32 on the GPU.  out and workspace
         (uint8, at least workspace_size(m) bytes) may be supplied by callers that must not allocate per call."""
         _dev(x, torch.float32, "input")
+        _check_optional_operands(self, x, gamma, residual)
         lib = load_library()
         dims = (C.c_size_t * max(x.dim(), 1))(*x.shape)
         nout = self.config.out_features
@@ -691,11 +703,19 @@ class BitLinear:
         """Contraction + epilogue on already-quantised activations (TernaryProcessor::ternary_matmul,
         ternary_operations.rs:87-113, minus its quantiser).  a: [m, in] int8, a_scale: [m] f32."""
         _dev(a, torch.int8, "a")
+        if a.dim() != 2 or a.shape[1] != self.config.in_features:
+            raise BitLinearError(SHAPE_MISMATCH, "activation width", [a.shape[0] if a.dim() else 1, self.config.in_features],
+                                 list(a.shape))
         m = a.shape[0]
-        if a.shape[1] != self.config.in_features:
-            raise BitLinearError(SHAPE_MISMATCH, "activation width", [m, self.config.in_features], list(a.shape))
+        _opt_dev(a_scale, torch.float32, "a_scale", m, a)
+        _opt_dev(a_sum, torch.int32, "a_sum", m, a)
+        _opt_dev(residual, torch.float32, "residual", m * self.config.out_features, a)
+        if a_scale is None:
+            raise BitLinearError(NULL_POINTER, "a_scale is required")
         if out is None:
             out = torch.empty((m, self.config.out_features), dtype=torch.float32, device=a.device)
+        else:
+            _opt_dev(out, torch.float32, "out", m * self.config.out_features, a)
         acc = torch.empty((m, self.config.out_features), dtype=torch.int32, device=a.device) if want_acc else None
         _check(load_library().bitnet_hip_bitlinear_matmul(self._h, _ptr(a), _ptr(a_sum), m, _ptr(a_scale), _ptr(residual), _ptr(acc),
                                                           _ptr(out), _stream(stream)))
@@ -716,9 +736,10 @@ def forward_multi(layers: Sequence["BitLinear"], x: torch.Tensor, gamma: Optiona
         raise BitLinearError(SHAPE_MISMATCH, "forward_multi takes a [m, in] input", [1, layers[0].config.in_features],
                              list(x.shape))
     m = x.shape[0]
-    outs = [torch.empty((m, l.config.out_features), dtype=torch.float32, device=x.device) for l in layers]
     if x.shape[1] != layers[0].config.in_features:
         raise BitLinearError(SHAPE_MISMATCH, "last input dimension", [m, layers[0].config.in_features], list(x.shape))
+    _opt_dev(gamma, torch.float32, "gamma", layers[0].config.in_features, x)
+    outs = [torch.empty((m, l.config.out_features), dtype=torch.float32, device=x.device) for l in layers]
     hs = (C.c_void_p * len(layers))(*[l._h for l in layers])
     os_ = (C.c_void_p * len(layers))(*[o.data_ptr() for o in outs])
     cfg = layers[0].config
@@ -773,9 +794,18 @@ class DecoderProjections:
                layers: Optional[Sequence[int]] = None):
         """One decode step through all blocks, or through blocks layers[0] .. layers[1]-1 only."""
         _dev(x, torch.float32, "x")
+        if x.dim() != 2 or x.shape[1] != self.hidden:
+            raise BitLinearError(SHAPE_MISMATCH, "decode input", [x.shape[0] if x.dim() else 1, self.hidden], list(x.shape))
         m = x.shape[0]
+        lo_hi = (0, self.layers) if layers is None else tuple(layers)
+        if len(lo_hi) != 2 or not (0 <= lo_hi[0] <= lo_hi[1] <= self.layers):
+            raise BitLinearError(INVALID_CONFIG, f"layer range {lo_hi} outside [0, {self.layers}]")
         if out is None:
             out = torch.empty_like(x)
+        else:
+            _dev(out, torch.float32, "out")
+            if tuple(out.shape) != tuple(x.shape) or out.device != x.device:
+                raise BitLinearError(SHAPE_MISMATCH, "decode output", list(x.shape), list(out.shape))
         q = torch.empty((m, self.hidden), dtype=torch.float32, device=x.device) if want_qk else None
         k = torch.empty((m, self.kv_dim), dtype=torch.float32, device=x.device) if want_qk else None
         lo, hi = (0, self.layers) if layers is None else layers

@@ -46,6 +46,8 @@ pub const BITNET_HIP_PRECISION_EIGHT_BIT: c_int = 1;
 pub const BITNET_HIP_LOOKUP_TERNARY: c_int = 0;
 pub const BITNET_HIP_LOOKUP_I2S: c_int = 1;
 
+// Only with the `hip` feature: without it nothing of the library is referenced, so the crate links without it.
+#[cfg(feature = "hip")]
 extern "C" {
     pub fn bitnet_hip_last_error() -> *const c_char;
     pub fn bitnet_hip_last_shape_mismatch(expected: *mut usize, actual: *mut usize, actual_rank: *mut c_int) -> c_int;

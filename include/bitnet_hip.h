@@ -198,7 +198,10 @@ int bitnet_hip_untile_weights(const uint8_t *tiled, size_t n, size_t k, uint8_t 
  *   CudaBackend::w2a8_gemv + validate_w2a8_dimensions (bitnet-cuda/src/backend.rs:129-157,217-257).
  *   weights [(m*k+3)/4] u8, activations [k] i8, output [m] i32; m = output features, k = input features
  *   (the reference's naming).  The *_checked form also takes the element counts of the three buffers
- *   and returns BITNET_HIP_SHAPE_MISMATCH exactly where validate_w2a8_dimensions errs. */
+ *   and returns BITNET_HIP_SHAPE_MISMATCH exactly where validate_w2a8_dimensions errs.
+ *   Code 3 (which no packer of the reference emits) counts as weight 0, as every Rust decoder of the reference
+ *   decodes it (weight_conversion.rs:175-181, gguf.rs:1130-1141); the CUDA kernel this call replaces clamps
+ *   code 3 - 1 = 2 to +1 instead (w2a8_gemv.cu:32-41).  The two differ only on bytes holding code 3. */
 int bitnet_hip_gemv_w2a8(const uint8_t *weights, const int8_t *activations, int32_t *output, size_t m,
                          size_t k, void *stream);
 int bitnet_hip_gemv_w2a8_checked(const uint8_t *weights, size_t weights_len, const int8_t *activations,

@@ -111,6 +111,71 @@ def test_binding_rejects_host_tensors_loudly():
     assert ei.value.kind == "DeviceError"
 
 
+class _FakeDeviceTensor:
+    """Stands in for a CUDA tensor so that the binding's host-side checks can be exercised without a device: the checks
+    must raise before any pointer reaches the library."""
+
+    def __init__(self, shape, dtype, device="cuda:0", contiguous=True):
+        import torch
+
+        self._t = torch.zeros(shape, dtype=dtype)
+        self.shape, self.dtype, self.is_cuda = self._t.shape, dtype, True
+        self.device = torch.device(device)
+        self._contig = contiguous
+
+    def dim(self):
+        return self._t.dim()
+
+    def numel(self):
+        return self._t.numel()
+
+    def is_contiguous(self):
+        return self._contig
+
+    def data_ptr(self):
+        raise AssertionError("a pointer was taken before validation finished")
+
+
+def test_binding_validates_operands_before_any_pointer_reaches_a_kernel():
+    """A wrong optional tensor (host memory, wrong dtype, too short, wrong shape, non-contiguous) is a BitLinearError raised
+    by the binding, never a launch with a wild pointer."""
+    import torch
+
+    F = _FakeDeviceTensor
+    f32, i8, i32 = torch.float32, torch.int8, torch.int32
+    layer = bh.BitLinear.__new__(bh.BitLinear)
+    layer.config, layer._h, layer._owner = bh.BitLinearConfig(in_features=16, out_features=8), None, object()
+    x = F((2, 16), f32)
+    cases = [
+        lambda: layer.forward(x, gamma=torch.ones(16)),                      # gamma in host memory
+        lambda: layer.forward(x, gamma=F((15,), f32)),                       # gamma too short
+        lambda: layer.forward(x, gamma=F((16,), torch.float64)),             # wrong dtype
+        lambda: layer.forward(x, residual=F((2, 7), f32)),                   # residual of the wrong size
+        lambda: layer.forward(x, residual=F((2, 8), f32, device="cuda:1")),  # another device
+        lambda: layer.forward_noalloc(x, F((2, 7), f32)),                    # out of the wrong size
+        lambda: layer.matmul_quantized(F((2, 16), i8), F((3,), f32)),        # a_scale length
+        lambda: layer.matmul_quantized(F((2, 16), i8), F((2,), f32), a_sum=F((2,), f32)),  # a_sum dtype
+        lambda: layer.matmul_quantized(F((2, 15), i8), F((2,), f32)),        # activation width
+        lambda: bh.quantize_activations_i8(F((2, 16), f32), gamma=F((8,), f32)),
+        lambda: bh.quantize_activations_i8(F((2, 16), f32), x2=F((2, 8), f32), input_mode=bh.INPUT_RELU2_MUL),
+        lambda: bh.quantize_activations_i8(F((16,), f32)),
+        lambda: bh.quantize_activations_i8(F((2, 16), f32, contiguous=False)),
+        lambda: bh.matmul_w2a8(F((1024,), torch.uint8), F((2, 16), i8), 8, a_scale=F((1,), f32)),
+        lambda: bh.matmul_w2a8(F((1024,), torch.uint8), F((2, 16), i8), 8, bias=F((7,), f32)),
+        lambda: bh.forward_multi([layer], x, gamma=F((4,), f32)),
+    ]
+    for i, case in enumerate(cases):
+        with pytest.raises(bh.BitLinearError):
+            case()
+    dec = bh.DecoderProjections.__new__(bh.DecoderProjections)
+    dec._h, dec.layers, dec.hidden, dec.kv_dim = None, 2, 16, 8
+    for bad in (lambda: dec.decode(F((2, 15), f32)), lambda: dec.decode(F((16,), f32)),
+                lambda: dec.decode(F((2, 16), f32), out=F((3, 16), f32)), lambda: dec.decode(F((2, 16), f32), layers=(1, 3)),
+                lambda: dec.decode(F((2, 16), torch.float64))):
+        with pytest.raises(bh.BitLinearError):
+            bad()
+
+
 def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
     monkeypatch.setattr(bh, "_lib", None)
     monkeypatch.setattr(bh, "LIB_PATH", tmp_path / "libbitnet_hip.so")

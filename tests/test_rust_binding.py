@@ -53,3 +53,52 @@ def test_rust_build_script_compiles_the_same_sources_with_the_same_flags():
     for flag in ("--offload-arch=gfx950", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-packed-fp32-ops",
                  "-amdgpu-kernarg-preload-count=10"):
         assert flag in build_rs and flag.lstrip("-") in makefile.replace("$(ARCH)", "gfx950")
+
+
+def _trait_methods(text, header_regex):
+    """{method: [argument names]} of the trait / impl block that starts at header_regex (brace matched)."""
+    m = re.search(header_regex, text)
+    assert m, header_regex
+    i = text.index("{", m.end() - 1)
+    depth, j = 0, i
+    while True:
+        depth += text[j] == "{"
+        depth -= text[j] == "}"
+        if depth == 0:
+            break
+        j += 1
+    body = re.sub(r"//[^\n]*", "", text[i:j])
+    out = {}
+    for fm in re.finditer(r"\bfn\s+([a-z_0-9]+)\s*\(([^)]*)\)", body, flags=re.S):
+        args = [a.strip() for a in fm.group(2).split(",") if a.strip()]
+        out[fm.group(1)] = [a if a.startswith("&") else a.split(":")[0].strip() for a in args]
+    return out
+
+
+def test_rust_crate_implements_the_reference_traits():
+    """impl BitLinearForward / TernaryLookupKernel / I2SLookupKernel / InferenceBackend for the wrapper types: same
+    method names, same receivers, same argument names and counts as the traits of the reference (transcribed with
+    their file:line into tests/golden; compared with the reference's own text where that is present)."""
+    import json
+
+    traits = json.loads((ROOT / "tests" / "golden" / "reference_vectors.json").read_text())["rust_traits"]
+    lib = (FFI.parent / "lib.rs").read_text()
+    for trait, spec in traits.items():
+        got = _trait_methods(lib, rf"impl\s+{trait}\s+for\s+{spec['for']}\s*\{{")
+        assert got == spec["methods"], (trait, got)
+        ref_file = Path("/root/reference") / spec["source"].split(":")[0]
+        if ref_file.exists():
+            assert _trait_methods(ref_file.read_text(), rf"pub\s+trait\s+{trait}\b[^{{]*\{{") == spec["methods"], trait
+
+
+def test_rust_crate_gates_the_library_behind_its_feature_and_keeps_raw_pointers_unsafe():
+    ffi = FFI.read_text()
+    assert re.search(r'#\[cfg\(feature = "hip"\)\]\s*extern "C" \{', ffi)
+    lib = (FFI.parent / "lib.rs").read_text()
+    # every function that takes raw device pointers is an unsafe fn; DeviceTensor's fields are private
+    for m in re.finditer(r"pub (unsafe )?fn ([a-z_0-9]+)\s*\(([^)]*)\)", lib, flags=re.S):
+        if "*const" in m.group(3) or "*mut" in m.group(3):
+            assert m.group(1), m.group(2)
+    tensor = re.search(r"pub struct DeviceTensor \{(.*?)\}", lib, flags=re.S).group(1)
+    assert "pub " not in tensor
+    assert "HipNotEnabled" in lib and '#[cfg(not(feature = "hip"))]' in lib
