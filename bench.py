@@ -67,7 +67,7 @@ LAUNCHES_PER_STEP = 4  # q+k+v | o | gate+up | down, each one gemv_fused16_kerne
 # script with --no-extras --calibration-copy), each scaled by what the same counter reads for the plain
 # 256 MiB copy: FETCH_SIZE reads 0.5 KiB per KiB fetched (factor 2.0), WRITE_SIZE 1.0 (factor 1.0).
 # Summary: profiles/decode_layer_b1_gemv_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_684_954
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_684_498
 
 
 def decode_roofline(event_ms, steps):
@@ -142,6 +142,13 @@ def prefill_rates(bh, torch, dec, gen, reps):
         ms = min(time_events(torch, lambda: [bh.forward_multi(layers, x) for _ in range(reps)]) for _ in range(3)) / reps
         ops = 2.0 * m * HIDDEN * sum(dec.proj_shape(p)[0] for p in projs)
         res[name] = {"forward_f32_in_ms": round(ms, 4), "tops_incl_quantiser": round(ops / (ms * 1e-3) / 1e12, 1)}
+    # what the matrix unit of this device sustains when it does nothing but v_mfma_i32_16x16x64_i8 from registers: the
+    # practical ceiling under the published 5.0 POP/s (its clock under load and the operands' switching activity included)
+    rand_tops, const_tops = bh.measure_mfma_i8_rate(True), bh.measure_mfma_i8_rate(False)
+    res["mfma_loop_ceiling"] = {"tops_random_operands": round(rand_tops, 1), "tops_constant_operands": round(const_tops, 1),
+                                "frac_int8_mfma_peak": round(rand_tops / INT8_PEAK_TOPS, 4)}
+    for name in ("2048x2560x6912", "2048x6912x2560"):
+        res[name]["frac_of_mfma_loop"] = round(res[name]["tops"] / rand_tops, 4)
     return res
 
 

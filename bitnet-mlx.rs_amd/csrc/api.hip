@@ -272,6 +272,38 @@ int bitnet_hip_device_info(char *arch_name, size_t arch_name_len, int *compute_u
     return BITNET_HIP_OK;
 }
 
+int bitnet_hip_measure_mfma_i8_rate(int random_operands, double *tera_ops_per_second, void *stream)
+{
+    if (!tera_ops_per_second) return fail(BITNET_HIP_NULL_POINTER, "measure_mfma_i8_rate: the result pointer is required");
+    int device = 0, units = 0;
+    BITNET_HIP_TRY(hipGetDevice(&device));
+    BITNET_HIP_TRY(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device));
+    DeviceTemp sink;
+    int rc = sink.alloc((size_t)units * MFMA_RATE_THREADS * sizeof(int));
+    if (rc != BITNET_HIP_OK) return rc;
+    struct Events {
+        hipEvent_t e[2] = {nullptr, nullptr};
+        ~Events() { for (hipEvent_t v : e) if (v) (void)hipEventDestroy(v); }
+    } ev;
+    BITNET_HIP_TRY(hipEventCreate(&ev.e[0]));
+    BITNET_HIP_TRY(hipEventCreate(&ev.e[1]));
+    hipStream_t s = as_stream(stream);
+    const int iters = 20000;  // about 2.5 ms
+    rc = launch_mfma_rate(random_operands != 0, 200, units, static_cast<int *>(sink.ptr), s);  // warm-up
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipEventRecord(ev.e[0], s));
+    rc = launch_mfma_rate(random_operands != 0, iters, units, static_cast<int *>(sink.ptr), s);
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipEventRecord(ev.e[1], s));
+    BITNET_HIP_TRY(hipEventSynchronize(ev.e[1]));  // the sink is freed on return: nothing of the launch is left running
+    float ms = 0.0f;
+    BITNET_HIP_TRY(hipEventElapsedTime(&ms, ev.e[0], ev.e[1]));
+    // 2 * 16 * 16 * 64 operations per instruction
+    const double ops = 32768.0 * MFMA_RATE_PER_ITER * (double)iters * (MFMA_RATE_THREADS / 64) * (double)units;
+    *tera_ops_per_second = ops / ((double)ms * 1e-3) / 1e12;
+    return BITNET_HIP_OK;
+}
+
 // ---- activation side ------------------------------------------------------------------------------
 
 int bitnet_hip_quantize_activations_i8(const float *x, const float *x2, size_t ldx, size_t m, size_t k,

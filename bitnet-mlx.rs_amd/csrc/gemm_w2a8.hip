@@ -895,4 +895,47 @@ int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_su
     return launch_tile<128, 128>(p, stream);
 }
 
+// ---- matrix-unit rate (diagnostic) -----------------------------------------------------------------------------
+// A loop of nothing but v_mfma_i32_16x16x64_i8 with its operands in registers: eight independent accumulators per
+// wavefront, two wavefronts per SIMD on every compute unit.  What it sustains is the ceiling of the GEMM above on the
+// device at hand (clock under a matrix load included); RANDOM gives every lane different int8 activations and 2-bit
+// codes 0..2 as weights, as the GEMM's operands are, otherwise every byte of both operands is 1.
+namespace {
+template <bool RANDOM>
+__global__ __launch_bounds__(512, 1) void mfma_rate_kernel(int iters, int *sink, unsigned seed)
+{
+    v4i acc[8], a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = (v4i){0, 0, 0, 0};
+    unsigned w = seed * (threadIdx.x + 1) * 2654435761u + blockIdx.x * 97u + 12345u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            w = w * 1664525u + 1013904223u;
+            a[i][c] = RANDOM ? (int)w : 0x01010101;
+            w = w * 1664525u + 1013904223u;
+            const unsigned two = (w >> 8) & 0x03030303u;  // bytes 0..3; 3 becomes 2 (no carry between bytes)
+            b[i][c] = RANDOM ? (int)(two - ((two >> 1) & two & 0x01010101u)) : 0x01010101;
+        }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b[i & 3], a[(i + (i >> 2)) & 3], acc[i], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+}  // namespace
+
+int launch_mfma_rate(bool random_operands, int iters, int compute_units, int *sink, hipStream_t stream)
+{
+    const dim3 grid((unsigned)compute_units), block(MFMA_RATE_THREADS);
+    if (random_operands) hipLaunchKernelGGL((mfma_rate_kernel<true>), grid, block, 0, stream, iters, sink, 7u);
+    else hipLaunchKernelGGL((mfma_rate_kernel<false>), grid, block, 0, stream, iters, sink, 7u);
+    BITNET_HIP_CHECK_LAUNCH("mfma_rate_kernel");
+    return BITNET_HIP_OK;
+}
+
 }  // namespace bitnet

@@ -84,4 +84,10 @@ int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_su
                       int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,
                       const float *residual, float *out, hipStream_t stream);
 
+// Diagnostic: `iters` rounds of eight v_mfma_i32_16x16x64_i8 per wavefront, MFMA_RATE_THREADS / 64 wavefronts on each of
+// `compute_units` workgroups, operands in registers; sink receives compute_units * MFMA_RATE_THREADS ints.
+constexpr int MFMA_RATE_THREADS = 512;
+constexpr int MFMA_RATE_PER_ITER = 8;
+int launch_mfma_rate(bool random_operands, int iters, int compute_units, int *sink, hipStream_t stream);
+
 }  // namespace bitnet

@@ -88,6 +88,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_last_shape_mismatch": (i32, [C.POINTER(sz), C.POINTER(sz), C.POINTER(i32)]),
         "bitnet_hip_init": (i32, [i32]),
         "bitnet_hip_device_info": (i32, [C.c_char_p, sz, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz)]),
+        "bitnet_hip_measure_mfma_i8_rate": (i32, [i32, C.POINTER(C.c_double), vp]),
         "bitnet_hip_quantize_activations_i8": (i32, [vp, vp, sz, sz, sz, i32, sz, sz, vp, f32, i32, vp, vp, vp, vp, vp]),
         "bitnet_hip_absmax_quantize_activations": (i32, [vp, sz, i32, vp, vp, vp]),
         "bitnet_hip_lookup_compute": (i32, [i32, vp, sz, vp, sz, vp, sz, vp]),
@@ -220,6 +221,15 @@ def device_info():
     cus, mhz, mem = C.c_int(0), C.c_int(0), C.c_size_t(0)
     _check(lib.bitnet_hip_device_info(name, 64, C.byref(cus), C.byref(mhz), C.byref(mem)))
     return {"arch": name.value.decode(), "compute_units": cus.value, "clock_mhz": mhz.value, "total_mem": mem.value}
+
+
+def measure_mfma_i8_rate(random_operands: bool = True, stream=None) -> float:
+    """10^12 int8 operations per second of a loop of nothing but v_mfma_i32_16x16x64_i8 on the current device (about
+    1.5 ms): the practical ceiling of the prefill GEMM there.  random_operands: int8 activations and 2-bit codes that
+    differ from lane to lane, as the GEMM's do; otherwise every operand byte is 1."""
+    tops = C.c_double(0.0)
+    _check(load_library().bitnet_hip_measure_mfma_i8_rate(1 if random_operands else 0, C.byref(tops), _stream(stream)))
+    return tops.value
 
 
 # ---- raw operators ------------------------------------------------------------------------------

@@ -89,6 +89,15 @@ int bitnet_hip_init(int device);
 int bitnet_hip_device_info(char *arch_name, size_t arch_name_len, int *compute_units, int *clock_mhz,
                            size_t *total_mem_bytes);
 
+/* Diagnostic: the int8 rate, in 10^12 operations per second, that a loop of nothing but v_mfma_i32_16x16x64_i8
+ * (operands in registers, two wavefronts per SIMD on every compute unit, about 2.5 ms) sustains on the current
+ * device: the practical ceiling of bitnet_hip_gemm_w2a8 there, clock under a matrix load included.
+ * random_operands != 0: every lane holds different int8 activations and 2-bit codes 0..2 as weights, as the GEMM's
+ * operands are; 0: every byte of both operands is 1.  Allocates a small buffer and waits for the result
+ * (tera_ops_per_second is a HOST pointer).  No counterpart in the reference; bench.py reports it beside the
+ * prefill rates. */
+int bitnet_hip_measure_mfma_i8_rate(int random_operands, double *tera_ops_per_second, void *stream);
+
 /* ---- activation side -------------------------------------------------------------------------- */
 
 /* Fused RMSNorm + per-token absmax int8 quantiser (one wavefront per token row).

@@ -1093,3 +1093,11 @@ def test_cpp_host_mirror_selftest():
     proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=110)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "all passed" in proc.stdout
+
+
+def test_mfma_rate_diagnostic_is_plausible():
+    """The matrix-unit loop bench.py quotes beside the prefill rates: between a tenth of and the published dense int8
+    peak (5.0 POP/s), and constant operands are not slower than switching ones beyond run-to-run noise."""
+    rand, const = bh.measure_mfma_i8_rate(True), bh.measure_mfma_i8_rate(False)
+    assert 500.0 < rand < 5100.0 and 500.0 < const < 5100.0
+    assert const > 0.9 * rand
