@@ -225,7 +225,7 @@ def device_info():
 
 def measure_mfma_i8_rate(random_operands: bool = True, stream=None) -> float:
     """10^12 int8 operations per second of a loop of nothing but v_mfma_i32_16x16x64_i8 on the current device (about
-    1.5 ms): the practical ceiling of the prefill GEMM there.  random_operands: int8 activations and 2-bit codes that
+    2.5 ms): the practical ceiling of the prefill GEMM there.  random_operands: int8 activations and 2-bit codes that
     differ from lane to lane, as the GEMM's do; otherwise every operand byte is 1."""
     tops = C.c_double(0.0)
     _check(load_library().bitnet_hip_measure_mfma_i8_rate(1 if random_operands else 0, C.byref(tops), _stream(stream)))
