@@ -3,18 +3,20 @@
 
     python bench.py --gpus 1 --steps K --warmup W
 
-A step is one decode pass (batch 1) through the seven BitLinear projections of one BitNet-b1.58-2B
-decoder layer (hidden 2560, FFN 6912, 20 query / 5 KV heads): fused RMSNorm + int8 quantisation before
+A step is one token at batch 1 through the decode projections of a BitNet-b1.58-2B stack: 30 passes of the
+decoder-layer workload (hidden 2560, FFN 6912, 20 query / 5 KV heads: fused RMSNorm + int8 quantisation before
 q/k/v and before gate/up, int8 quantisation before o and down, seven packed-ternary GEMVs with the scale
-epilogue.  Consecutive steps use the weights of consecutive layers of a 30-layer stack (521 MB of packed
-weights in total), so no step finds its weights in cache.  Inputs and weights are resident in HBM before
-the timed region: an untimed pass over all 30 layers comes first (first touch of every weight page), then the
-warm-up steps, then the region of exactly K steps, which is run REPEATS times back to back; the line reports the
-median region (every region's time is listed under config.region_ms), so that a short run (--steps 20) and a long one
-agree.  value = packed-weight bytes streamed per second over that region, by the host's clock around it.
+epilogue), each over the weights of its own layer (521 MB of packed weights per step, more than the last-level
+cache holds, so no pass finds its weights cached), the hidden state carried from layer to layer.  Inputs and
+weights are resident in HBM before the timed region: one untimed step comes first (first touch of every weight
+page), then the warm-up steps, then the region of exactly K steps, which is run REPEATS times back to back; the
+line reports the median region (every region's time is listed under config.region_ms).  A step is long enough
+(about 0.5 ms) for the cost of starting and stopping a region to vanish, so a short run (--steps 20) and a long
+one agree.  value = packed-weight bytes streamed per second over that region, by the host's clock around it;
+config.us_per_layer is the same figure per decoder layer.
 
 The timed region contains one kernel family only, the decode GEMV with the activation quantiser fused into
-its prologue (four launches per step: q+k+v, o, gate+up, down), so the roofline of the dominant kernel comes
+its prologue (four launches per layer: q+k+v, o, gate+up, down), so the roofline of the dominant kernel comes
 straight from the HIP events around the timed region: achieved = packed-weight bytes per launch / average
 launch duration.  The line also carries the GEMV alone on pre-quantised activations (graph replays over the
 same 210 matrices), the prefill GEMM rate (M = 2048) at the two FFN shapes, and a CPU baseline (a C
@@ -62,26 +64,33 @@ def time_events(torch, fn):
 
 
 REPEATS = 7  # timed regions of --steps steps each; the median is reported
-LAUNCHES_PER_STEP = 4  # q+k+v | o | gate+up | down, each one gemv_fused16_kernel<MODE, NORM, NCHB, RBW> launch
+LAUNCHES_PER_LAYER = 4  # q+k+v | o | gate+up | down, each one gemv_fused16_kernel<MODE, NORM, NCHB, RBW> launch
+# A step is one token at batch 1 through the decode projections of all 30 layers (30 passes of the decoder-layer
+# workload, each over its own weights, the hidden state carried from layer to layer): 120 dependent launches, 521 MB
+# of packed weights, about 0.5 ms.  Starting and stopping a timed region costs 20 to 90 us on the boxes measured
+# (event records, the first launch into an idle queue, the wake-up of the waiting host thread); with a step this
+# long that is under 1 % of a region of 20 steps, so the figure does not depend on --steps.
+LAUNCHES_PER_STEP = LAUNCHES_PER_LAYER * LAYERS
+STEP_BYTES = LAYER_BYTES * LAYERS
 # HBM bytes per launch of that kernel from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (two runs of this
 # script with --no-extras --calibration-copy), each scaled by what the same counter reads for the plain
 # 256 MiB copy: FETCH_SIZE reads 0.5 KiB per KiB fetched (factor 2.0), WRITE_SIZE 1.0 (factor 1.0).
 # Summary: profiles/decode_layer_b1_gemv_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_684_498
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_684_520
 
 
 def decode_roofline(event_ms, steps):
     launches = steps * LAUNCHES_PER_STEP
-    total_bytes = steps * LAYER_BYTES
+    total_bytes = steps * STEP_BYTES
     achieved = total_bytes / (event_ms * 1e-3) / 1e9
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
         "kernel": "gemv_fused16_kernel<MODE, NORM, NCHB, RBW> (decode GEMV, activation quantiser in the prologue)",
         "launches": launches, "avg_launch_us": round(event_ms * 1e3 / launches, 3),
-        "bytes_per_launch": LAYER_BYTES // LAUNCHES_PER_STEP,
+        "bytes_per_launch": LAYER_BYTES // LAUNCHES_PER_LAYER,
         "how": "HIP events on the launch stream around the timed region, which holds only this kernel "
-               "(4 launches per step, back to back); algorithmic bytes = packed weights n*k/4",
+               "(4 launches per layer, 120 per step, back to back); algorithmic bytes = packed weights n*k/4",
     }
 
 
@@ -321,8 +330,8 @@ def cpu_baseline(torch, dec, budget_s=8.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=600)
-    ap.add_argument("--warmup", type=int, default=60)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip roofline / prefill / CPU legs (profiling runs)")
     ap.add_argument("--only-prefill", type=int, default=0, metavar="REPS",
@@ -347,16 +356,11 @@ def main():
         return
     x = torch.randn((1, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
 
-    def run_steps(first, count):
-        """Steps first .. first+count-1; step i is decoder layer i % LAYERS.  Consecutive steps up to the end of the
-        stack go through one call of the boundary (the same four launches per step either way): with one call per
-        step the Python host, not the GPU, sets the pace once a step is under ~18 us."""
-        i, end = first, first + count
-        while i < end:
-            l = i % LAYERS
-            n = min(LAYERS - l, end - i)
-            dec.decode(x, out=x, layers=(l, l + n))
-            i += n
+    def run_steps(count):
+        """`count` token steps, each one call of the boundary: the seven projections of layers 0..29 in turn, the hidden
+        state carried along (four launches per layer)."""
+        for _ in range(count):
+            dec.decode(x, out=x)
 
     if args.calibration_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
@@ -365,34 +369,35 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    run_steps(0, LAYERS)  # residency: every layer's weights touched once, untimed
-    run_steps(0, args.warmup)
+    run_steps(1)  # residency: every layer's weights touched once, untimed
+    run_steps(args.warmup)
     torch.cuda.synchronize()
     regions = []  # (host seconds, event milliseconds) of each region of exactly args.steps steps
-    first = args.warmup
     for _ in range(REPEATS):
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         start.record()
-        run_steps(first, args.steps)
+        run_steps(args.steps)
         stop.record()
         torch.cuda.synchronize()
         regions.append((time.perf_counter() - t0, start.elapsed_time(stop)))
-        first += args.steps
     regions_sorted = sorted(regions)
     elapsed, event_ms = regions_sorted[len(regions_sorted) // 2]  # the median region by host time
 
-    value = args.steps * LAYER_BYTES / elapsed / 1e9
+    value = args.steps * STEP_BYTES / elapsed / 1e9
     line = {
         "metric": "BitLinear decode GB/s (% HBM peak) + prefill int8 TOPS (% MFMA peak)",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(elapsed * 1e3 / args.steps, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "i8", "data": "synthetic",
         "config": {"workload": "configs[1]: one decoder layer's 7 decode projections at batch 1 "
-                               "(hidden 2560, ffn 6912, 20q/5kv heads), weights rotating over a 30-layer stack; "
-                               "a step = one layer = four kernel launches, up to 30 consecutive steps per host call",
-                   "bytes_per_step": LAYER_BYTES, "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+                               "(hidden 2560, ffn 6912, 20q/5kv heads), passed 30 times per step over the 30 distinct "
+                               "weight sets of a BitNet-2B stack (= one token step of configs[4] at batch 1); "
+                               "a step = 30 layers = 120 dependent kernel launches, one host call",
+                   "layers_per_step": LAYERS, "bytes_per_step": STEP_BYTES, "bytes_per_layer": LAYER_BYTES,
+                   "us_per_layer": round(elapsed * 1e6 / args.steps / LAYERS, 3),
+                   "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
                    "event_ms_per_step": round(event_ms / args.steps, 5), "repeats": REPEATS, "reported": "median region",
                    "region_ms": [round(r[0] * 1e3, 4) for r in regions], "sum_order": "block256 (the build's declared order)",
                    "device": bh.device_info()},
