@@ -842,17 +842,21 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
     if (nproj > GEMM_MAX_PROJ) return BITNET_HIP_UNSUPPORTED;
     bool dma_ok = a_sum != nullptr && m >= 96 && k % 256 == 0 && k >= 512 && (reinterpret_cast<uintptr_t>(a) & 15) == 0 &&
                   m * k < (1ull << 32);  // 32-bit lane offsets
-    size_t tiles = 0;
+    size_t tiles = 0, tiles128 = 0;  // 128 x 160 tiles; 128 x 128 tiles, or 0 if a projection is not a multiple of 128 wide
+    bool all128 = true;
     GemmParams p = {};
     for (int j = 0; j < nproj && dma_ok; ++j) {
         const GemvProj &s = projs[j];
         dma_ok = s.n > 0 && s.n <= 0x7fffffffu && tiled_bytes(s.n, k) < (1ull << 32);
         tiles += ((m + 127) / 128) * ((s.n + 159) / 160);
+        tiles128 += ((m + 127) / 128) * ((s.n + 127) / 128);
+        all128 = all128 && s.n % 128 == 0;
         GemmProjDev &d = p.proj[j];
         d.w = s.tiled; d.w_scale = s.w_scale; d.bias = s.bias; d.residual = s.residual; d.out = s.out; d.acc = s.acc;
         d.n = (int)s.n; d.tn_end = 0;
     }
     if (!dma_ok) return BITNET_HIP_UNSUPPORTED;
+    if (!all128) tiles128 = 0;
     for (int j = nproj; j < GEMM_MAX_PROJ; ++j) p.proj[j] = p.proj[nproj - 1];
     p.nproj = nproj; p.a = a; p.a_sum = a_sum; p.a_scale = a_scale; p.m = (int)m; p.k = (int)k; p.kt_count = (int)k_tiles(k);
     // Three shapes of the LDS-direct kernel, chosen by how many 128 x 160 tiles the outputs hold (256 compute
@@ -866,6 +870,9 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
     //   otherwise                            -> 64 x 160, four workgroups of 4 wavefronts per compute unit.
     if (tiles >= 640) return launch_dma<128, 160, 2, 3>(p, stream);
     if (tiles >= 100 && tiles <= 256) return launch_ld8<128, 160>(p, stream);
+    // between one and 2.5 tiles of 128 x 160 per compute unit: 128 x 128 tiles when they divide every projection and
+    // fill the 768 workgroup slots almost three times (q + k + v at 3072 tokens: 33.0 us against 37.9 us with 64 x 160)
+    if (tiles > 256 && tiles128 >= 640) return launch_dma<128, 128, 2, 3>(p, stream);
     return launch_dma<64, 160, 2, 4>(p, stream);
 }
 

@@ -727,6 +727,32 @@ def test_forward_multi_prefill_gate_up_one_launch():
         assert np.array_equal(got, host(layer.forward(dev(x), gamma=dev(g))))
 
 
+def test_forward_multi_prefill_qkv_128x128_tiles():
+    """q, k and v at M = 3072 (and a ragged M just below) share one launch of the 128 x 128 instance of the prefill GEMM
+    (720 tiles): sampled rows against the oracle, everything against the single-layer forwards, which take other
+    instances (q alone 480 tiles, k and v alone 120)."""
+    rng = np.random.default_rng(3072)
+    k, ns = 2560, [2560, 640, 640]
+    g = (1 + 0.1 * rng.standard_normal(k, dtype=f32)).astype(f32)
+    layers, packed = [], []
+    for i, n in enumerate(ns):
+        w = synth_weights(rng, n, k)
+        layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), f"qkv{i}")
+        layer.update_weights(dev(w))
+        layers.append(layer)
+        qw, ws = orc.quantize_weights_absmean(w)
+        packed.append((orc.pack_2bit(qw), n, ws))
+    for m in (3072, 3072 - 37):
+        x = synth_activations(rng, m, k, outliers=True)
+        rows = np.sort(rng.choice(m, size=24, replace=False))
+        rows[-1] = m - 1
+        outs = bh.forward_multi(layers, dev(x), gamma=dev(g))
+        for layer, out, (pk, n, ws) in zip(layers, outs, packed):
+            got = host(out)
+            assert np.array_equal(got[rows], orc.bitlinear_forward(x[rows], pk, n, ws, g=g, eps=1e-5)[0])
+            assert np.array_equal(got, host(layer.forward(dev(x), gamma=dev(g))))
+
+
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 7])
 @pytest.mark.parametrize("n,k", [(1, 4), (17, 260), (1000, 2560), (2560, 6912), (6912 + 5, 2560), (40, 8192), (13824, 2560)])
 def test_forward_fused_rows_bit_exact(m, n, k):
