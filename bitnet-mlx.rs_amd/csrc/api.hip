@@ -991,6 +991,9 @@ int bitnet_hip_decoder_set_norm(bitnet_hip_decoder *dec, size_t layer, int which
     if (layer >= dec->layers || which < 0 || which > 1)
         return fail(BITNET_HIP_INVALID_CONFIG, "decoder_set_norm: layer %zu / which %d out of range", layer, which);
     float *dst = dec->gamma + (layer * 2 + (size_t)which) * dec->hidden;
+    // as a weight update: no decode is being enqueued, and those already queued (on any stream) have finished
+    std::lock_guard<std::mutex> one_decode(dec->decode_lock);
+    BITNET_HIP_TRY(hipDeviceSynchronize());
     BITNET_HIP_TRY(hipMemcpyAsync(dst, gamma, sizeof(float) * dec->hidden,
                                   on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, as_stream(stream)));
     BITNET_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
@@ -1088,11 +1091,16 @@ struct bitnet_hip_backend {
     float *stage_in = nullptr, *stage_out = nullptr;  // [max_tokens, hidden] each
     size_t stage_bytes = 0;
     std::mutex lock;  // execute_batch calls share the staging buffers
+    // recorded behind the last call that used the staging buffers: a call on another stream waits for it
+    hipEvent_t done = nullptr;
+    hipStream_t done_stream = nullptr;
+    bool done_recorded = false;
 
     ~bitnet_hip_backend()
     {
         if (stage_in) (void)hipFree(stage_in);
         if (stage_out) (void)hipFree(stage_out);
+        if (done) (void)hipEventDestroy(done);
     }
 };
 
@@ -1130,6 +1138,11 @@ int bitnet_hip_backend_create(int device, bitnet_hip_backend **backend)
         return fail(BITNET_HIP_DEVICE_ERROR, "backend_create: hipGetDeviceProperties failed: %s", hipGetErrorString(e));
     }
     b->total_mem = prop.totalGlobalMem;
+    e = hipEventCreateWithFlags(&b->done, hipEventDisableTiming);
+    if (e != hipSuccess) {
+        delete b;
+        return fail(BITNET_HIP_DEVICE_ERROR, "backend_create: hipEventCreate failed: %s", hipGetErrorString(e));
+    }
     *backend = b;
     return BITNET_HIP_OK;
 }
@@ -1176,6 +1189,11 @@ int bitnet_hip_backend_execute_batch(bitnet_hip_backend *backend, const float *c
             return fail_shape(e, 2, a, 2, "rows of one input exceed the model's max_tokens");
         }
     }
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(s, &capturing);
+    if (backend->done_recorded && backend->done_stream != s && capturing == hipStreamCaptureStatusNone)
+        BITNET_HIP_TRY(hipStreamWaitEvent(s, backend->done, 0));  // the staging buffers were last used on another stream
+    bool staged = false;
     size_t i = 0;
     while (i < count) {
         // the longest run of inputs from i on whose rows fit one pass
@@ -1187,6 +1205,7 @@ int bitnet_hip_backend_execute_batch(bitnet_hip_backend *backend, const float *c
             if (rc != BITNET_HIP_OK) return rc;
         } else {
             size_t at = 0;
+            staged = true;
             for (size_t t = i; t < j; ++t) {
                 if (rows[t] == 0) continue;
                 BITNET_HIP_TRY(hipMemcpyAsync(backend->stage_in + at * H, inputs[t], sizeof(float) * rows[t] * H, hipMemcpyDeviceToDevice, s));
@@ -1202,6 +1221,11 @@ int bitnet_hip_backend_execute_batch(bitnet_hip_backend *backend, const float *c
             }
         }
         i = j;
+    }
+    if (staged && capturing == hipStreamCaptureStatusNone) {
+        BITNET_HIP_TRY(hipEventRecord(backend->done, s));
+        backend->done_stream = s;
+        backend->done_recorded = true;
     }
     return BITNET_HIP_OK;
 }
