@@ -22,6 +22,7 @@ struct ActQuantParams {
     int32_t *a_sum;
     float *y;
     size_t m;
+    int seq_in_lds;  // the launch carries LDS for the row's squares (literal summation order: sum_sequential_lds)
 };
 
 // NCH > 0: a lane keeps its NCH chunks in registers (K <= 256*NCH).  NCH == 0: any K, the row is
@@ -153,7 +154,18 @@ __global__ __launch_bounds__(256) void act_quant_block_kernel(ActQuantParams p)
     if (norm) {
         float ss;
         if (src.sum_order == BITNET_HIP_SUM_SEQUENTIAL) {
-            ss = sum_squares_sequential<MODE>(src, row);
+            if (p.seq_in_lds) {
+                extern __shared__ float sq_lds[];  // squares_lds_bytes(k)
+#pragma unroll
+                for (int i = 0; i < nloop; ++i) {
+                    const int c = tid + 256 * i;
+                    if (c < chunks) store_squares4(sq_lds, c, chunk_at(i, c));
+                }
+                __syncthreads();
+                ss = sum_sequential_lds(sq_lds, k);
+            } else {
+                ss = sum_squares_sequential<MODE>(src, row);
+            }
         } else {
             float part = 0.0f;  // thread tid is virtual lane tid
 #pragma unroll
@@ -263,7 +275,16 @@ __global__ __launch_bounds__(1024) void act_quant_block16_kernel(const float *ho
     if (norm) {
         float ss;
         if (src.sum_order == BITNET_HIP_SUM_SEQUENTIAL) {
-            ss = sum_squares_sequential<MODE>(src, row);
+            if (p.seq_in_lds) {
+                extern __shared__ float sq_lds[];  // squares_lds_bytes(k)
+#pragma unroll
+                for (int i = 0; i < NCHB; ++i)
+                    if (tid + 1024 * i < chunks) store_squares4(sq_lds, tid + 1024 * i, v[i]);
+                lds_barrier();
+                ss = sum_sequential_lds(sq_lds, k);
+            } else {
+                ss = sum_squares_sequential<MODE>(src, row);
+            }
         } else {
             if (chain) {  // thread tid < 256 is virtual lane tid
                 float part = 0.0f;
@@ -325,10 +346,20 @@ void launch_wave(const ActQuantParams &p, hipStream_t s)
     hipLaunchKernelGGL((act_quant_wave_kernel<MODE, NCH, VEC>), grid, block, 0, s, p);
 }
 
-template <int MODE, int NCH, bool VEC>
-void launch_block(const ActQuantParams &p, hipStream_t s)
+// LDS for the row's squares where the literal summation order is asked for and a row fits the default limit
+inline size_t launch_squares_lds(const ActQuantParams &p)
 {
-    hipLaunchKernelGGL((act_quant_block_kernel<MODE, NCH, VEC>), dim3((unsigned)p.m), dim3(256), 0, s, p);
+    if (!p.src.gamma || p.src.sum_order != BITNET_HIP_SUM_SEQUENTIAL) return 0;
+    const size_t bytes = squares_lds_bytes(p.src.k);
+    return bytes <= 60 * 1024 ? bytes : 0;
+}
+
+template <int MODE, int NCH, bool VEC>
+void launch_block(ActQuantParams p, hipStream_t s)
+{
+    const size_t lds = launch_squares_lds(p);
+    p.seq_in_lds = lds != 0;
+    hipLaunchKernelGGL((act_quant_block_kernel<MODE, NCH, VEC>), dim3((unsigned)p.m), dim3(256), lds, s, p);
 }
 
 template <int MODE>
@@ -338,8 +369,11 @@ void launch_mode(const ActQuantParams &p, bool vec, hipStream_t s)
     // Few rows (a decode batch): 16 wavefronts per row.
     if (p.m <= 16 && vec && chunks <= 2048 && p.src.ldx < (1u << 31)) {
 #define BITNET_HOT_ARGS p.src.x, (int)p.src.ldx, p.src.k, p.src.x2, p.src.gamma, p.src.head_dim, p.src.gqa_group
-        if (chunks <= 1024) hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 1>), dim3((unsigned)p.m), dim3(1024), 0, s, BITNET_HOT_ARGS, p);
-        else hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 2>), dim3((unsigned)p.m), dim3(1024), 0, s, BITNET_HOT_ARGS, p);
+        ActQuantParams q = p;
+        const size_t lds = launch_squares_lds(p);
+        q.seq_in_lds = lds != 0;
+        if (chunks <= 1024) hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 1>), dim3((unsigned)p.m), dim3(1024), lds, s, BITNET_HOT_ARGS, q);
+        else hipLaunchKernelGGL((act_quant_block16_kernel<MODE, 2>), dim3((unsigned)p.m), dim3(1024), lds, s, BITNET_HOT_ARGS, q);
 #undef BITNET_HOT_ARGS
         return;
     }
@@ -506,7 +540,7 @@ int launch_act_quant(const float *x, const float *x2, size_t ldx, size_t m, size
     p.src.x = x; p.src.x2 = x2; p.src.gamma = gamma; p.src.ldx = ldx; p.src.k = (int)k;
     p.src.head_dim = (int)(head_dim ? head_dim : 1); p.src.gqa_group = (int)(gqa_group ? gqa_group : 1);
     p.src.sum_order = sum_order; p.src.eps = eps;
-    p.q = q; p.a_scale = a_scale; p.a_sum = a_sum; p.y = y; p.m = m;
+    p.q = q; p.a_scale = a_scale; p.a_sum = a_sum; p.y = y; p.m = m; p.seq_in_lds = 0;
 
     bool vec = (k % 4 == 0) && (ldx % 4 == 0) && aligned(x, 16) && aligned(q, 4) && (!x2 || aligned(x2, 16)) &&
                (!y || aligned(y, 16)) && (!gamma || aligned(gamma, 16));

@@ -341,7 +341,14 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
     if constexpr (NORM) {
         float ss;
         if (p.src.sum_order == BITNET_HIP_SUM_SEQUENTIAL) {
-            ss = sum_squares_sequential<MODE>(p.src, 0);
+            // the reference's literal order: the squares go through LDS (the launch sizes it for them; the int8 row
+            // takes the same place later, behind the barrier of the absmax reduction) and every wavefront runs the chain
+            float *sq_lds = reinterpret_cast<float *>(lds_a);
+#pragma unroll
+            for (int i = 0; i < NCH; ++i)
+                if (tid + 256 * i < chunks) store_squares4(sq_lds, tid + 256 * i, v[i]);
+            lds_barrier();
+            ss = sum_sequential_lds(sq_lds, p.k);
         } else {
             float part = 0.0f;
 #pragma unroll
@@ -1226,9 +1233,11 @@ int launch_mode(const GemvParams &p, hipStream_t stream)
 template <int MODE, int RBW>
 int launch_fused_mode(const GemvParams &p, hipStream_t stream)
 {
-    const size_t lds = (size_t)p.kt_count * 16 * sizeof(uint4);
-    const dim3 grid((unsigned)p.proj[p.nproj - 1].rb_end);
     const bool norm = p.src.gamma != nullptr, small = p.k <= 3 * 1024;
+    // the int8 row, or (first) the f32 squares of the row for the literal summation order
+    const size_t lds_q = (size_t)p.kt_count * 16 * sizeof(uint4), lds_sq = squares_lds_bytes(p.k);
+    const size_t lds = (norm && p.src.sum_order == BITNET_HIP_SUM_SEQUENTIAL && lds_sq > lds_q) ? lds_sq : lds_q;
+    const dim3 grid((unsigned)p.proj[p.nproj - 1].rb_end);
     if (norm && small) hipLaunchKernelGGL((gemv_fused_kernel<MODE, true, 3, RBW>), grid, dim3(256), lds, stream, p);
     else if (norm) hipLaunchKernelGGL((gemv_fused_kernel<MODE, true, FUSED_NCH, RBW>), grid, dim3(256), lds, stream, p);
     else if (small) hipLaunchKernelGGL((gemv_fused_kernel<MODE, false, 3, RBW>), grid, dim3(256), lds, stream, p);

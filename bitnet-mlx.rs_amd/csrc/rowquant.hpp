@@ -191,6 +191,30 @@ __device__ __forceinline__ float sum_squares_sequential(const RowSource &p, size
     return ss;
 }
 
+// The same literal order with the squares of the row staged in LDS: sq[i] = x[i] * x[i] in element order, written by
+// the workgroup (store_squares4) and made visible by a barrier before the call.  Every lane runs the same chain of k
+// additions; its reads are broadcasts (one address for all lanes), 16 bytes at a time.  What is left is the latency of
+// a dependent v_add_f32, about 8.5 cycles an element (measured; reading further ahead of the additions gains nothing).
+__host__ __device__ inline size_t squares_lds_bytes(int k) { return (size_t)((k + 3) >> 2) * 16; }
+__device__ __forceinline__ void store_squares4(float *sq, int c, const float4 &e)  // chunk c: elements 4c .. 4c + 3
+{
+    *reinterpret_cast<float4 *>(sq + 4 * (size_t)c) =
+        make_float4(f32_mul(e.x, e.x), f32_mul(e.y, e.y), f32_mul(e.z, e.z), f32_mul(e.w, e.w));
+}
+__device__ __forceinline__ float sum_sequential_lds(const float *sq, int k)
+{
+    float ss = 0.0f;
+    const int full = k >> 2;
+    const float4 *sq4 = reinterpret_cast<const float4 *>(sq);
+#pragma unroll 8
+    for (int c = 0; c < full; ++c) {
+        const float4 s = sq4[c];
+        ss = f32_add(f32_add(f32_add(f32_add(ss, s.x), s.y), s.z), s.w);
+    }
+    for (int i = full * 4; i < k; ++i) ss = f32_add(ss, sq[i]);
+    return ss;
+}
+
 __device__ __forceinline__ float rms_from_ss(float ss, int k, float eps)
 {
     return f32_sqrt(f32_add(f32_div(ss, (float)k), eps));

@@ -206,11 +206,14 @@ def test_activation_quant_bit_exact(m, k, norm):
         assert np.array_equal(host(y), orc.rmsnorm(x, g, 1e-5, orc.SUM_BLOCK256))
 
 
-@pytest.mark.parametrize("k", [2560, 300])
-def test_activation_quant_sequential_order_bit_exact(k):
-    """The reference's literal summation order (one running f32 sum) is available and also bit-exact."""
-    rng = np.random.default_rng(k)
-    x = synth_activations(rng, 3, k)
+@pytest.mark.parametrize("m,k", [(3, 2560), (3, 300), (40, 2560), (40, 6912), (5, 12000), (2, 20000), (40, 301), (64, 8192),
+                                 (300, 2560), (16, 6912)])
+def test_activation_quant_sequential_order_bit_exact(m, k):
+    """The reference's literal summation order (one running f32 sum) is available and also bit-exact: the kernels with
+    16 and 4 wavefronts per row (the row's squares staged in LDS, every lane running the chain), unaligned rows, rows
+    too long for the staging (the chain then reads global memory) and the wavefront-per-row kernel."""
+    rng = np.random.default_rng(k + m)
+    x = synth_activations(rng, m, k)
     g = rng.standard_normal(k, dtype=f32)
     q, s, _, y = bh.quantize_activations_i8(dev(x), dev(g), eps=1e-6, sum_order=bh.SUM_SEQUENTIAL, want_y=True)
     q_ref, s_ref, _ = orc.rmsnorm_quantize_i8(x, g, 1e-6, orc.SUM_SEQUENTIAL)
