@@ -148,6 +148,17 @@ public:
     const BitLinearConfig &config() const { return config_; }
     const std::string &layer_name() const { return layer_name_; }
     bitnet_hip_bitlinear *handle() const { return handle_; }
+    // BitLinear::device (layer.rs:223): the ordinal of the GPU the layer's buffers were allocated on
+    int device() const { return device_; }
+    // BitLinear::clear_cache (layer.rs:353-361): the reference caches the quantised form of its latent f32 weights;
+    // this layer holds only the quantised weights (update_weights quantises at once), so there is nothing to clear
+    Result<Unit> clear_cache() const { return Unit{}; }
+    // BitLinear::to_device (layer.rs:376-411): the same device is the reference's no-op, any other is refused
+    Result<Unit> to_device(int device)
+    {
+        if (device == device_) return Unit{};
+        return BitLinearError{BitLinearError::DeviceError, "Failed to move weights to device: the layer lives on one GPU", {}, {}};
+    }
 
     // update_weights: latent f32 [out_features, in_features] in host memory
     Result<Unit> update_weights(const std::vector<float> &w, size_t rows, size_t cols)
@@ -198,10 +209,14 @@ public:
     }
 
 private:
-    BitLinear(BitLinearConfig c, std::string n, bitnet_hip_bitlinear *h) : config_(c), layer_name_(std::move(n)), handle_(h) {}
+    BitLinear(BitLinearConfig c, std::string n, bitnet_hip_bitlinear *h) : config_(c), layer_name_(std::move(n)), handle_(h)
+    {
+        (void)hipGetDevice(&device_);
+    }
     BitLinearConfig config_;
     std::string layer_name_;
     bitnet_hip_bitlinear *handle_;
+    int device_ = 0;
     mutable std::mutex workspace_lock_;  // forward calls of one layer share the scratch: one at a time through this mirror
     mutable void *workspace_ = nullptr;
     mutable size_t workspace_bytes_ = 0;
@@ -317,9 +332,11 @@ public:
 
 // absmax_quantize_activations: ONE scale for the whole tensor, ternary codes (the default precision) or 8-bit values.
 enum class QuantizationPrecision { OneFiveFiveBit = BITNET_HIP_PRECISION_ONE_FIVE_FIVE_BIT, EightBit = BITNET_HIP_PRECISION_EIGHT_BIT };
+// QuantizationStats (bitnet-quant/src/quantization/mod.rs:118-148) with its defaults
 struct QuantizationStats {
     size_t elements_count = 0;
-    float quantization_error = 0.f, compression_ratio = 0.f, min_value = 0.f, max_value = 0.f, scale_factor = 1.f;
+    float quantization_error = 0.f, compression_ratio = 1.f, min_value = 0.f, max_value = 0.f, scale_factor = 1.f;
+    std::optional<int> zero_point;
 };
 struct QuantizedActivation {
     std::shared_ptr<int8_t> values;  // device, original_shape elements (signed: the reference's U8 cast loses the sign)
@@ -370,6 +387,23 @@ class BitNetWeightQuantizer {
 public:
     explicit BitNetWeightQuantizer(WeightQuantizationConfig c = {}) : config_(c) {}
     const WeightQuantizationConfig &config() const { return config_; }
+    // Quantizer::validate_input (weights.rs:625-639)
+    Result<Unit> validate_input(const DeviceTensor &weights) const
+    {
+        if (weights.dims().size() < 2)
+            return BitLinearError{BitLinearError::QuantizationError, "Weight tensor must have at least 2 dimensions", {}, {}};
+        return Unit{};
+    }
+    // Quantizer::dequantize (weights.rs:616-619): values * scales, on the host
+    std::vector<float> dequantize(const QuantizedWeight &q) const
+    {
+        std::vector<float> out(q.values.size());
+        for (size_t i = 0; i < out.size(); ++i) out[i] = static_cast<float>(q.values[i]) * q.scales;
+        return out;
+    }
+    // Quantizer::get_stats (weights.rs:638-640): the quantizer's own record, which quantize(&self) never updates in the
+    // reference, so the defaults
+    QuantizationStats get_stats() const { return QuantizationStats{}; }
     // weights: [rows, cols] f32 on the device
     Result<QuantizedWeight> quantize(const DeviceTensor &weights, hipStream_t stream = nullptr) const
     {
@@ -380,8 +414,10 @@ public:
         int8_t *q = nullptr;
         float *scale = nullptr;
         if (hipMalloc(reinterpret_cast<void **>(&packed), (n + 3) / 4 + 1) != hipSuccess ||
-            hipMalloc(reinterpret_cast<void **>(&q), n + 1) != hipSuccess || hipMalloc(reinterpret_cast<void **>(&scale), sizeof(float)) != hipSuccess)
+            hipMalloc(reinterpret_cast<void **>(&q), n + 1) != hipSuccess || hipMalloc(reinterpret_cast<void **>(&scale), sizeof(float)) != hipSuccess) {
+            (void)hipFree(packed); (void)hipFree(q); (void)hipFree(scale);  // hipFree(nullptr) is a no-op
             return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
+        }
         int rc = bitnet_hip_quantize_weights_reference(weights.data(), rows, cols, static_cast<int>(config_.ternary_method),
                                                        config_.normalize_weights, config_.outlier_threshold,
                                                        config_.custom_threshold_factor.value_or(0.0f), packed, scale, q, nullptr, stream);

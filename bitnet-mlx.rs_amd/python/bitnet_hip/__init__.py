@@ -407,6 +407,18 @@ WQ_STATS = ("mean", "sd", "clip_mean", "clip_mad", "lo", "hi", "mean_abs", "max_
 
 
 @dataclass
+class QuantizationStats:
+    """QuantizationStats (bitnet-quant/src/quantization/mod.rs:118-148) with its defaults."""
+    elements_count: int = 0
+    quantization_error: float = 0.0
+    compression_ratio: float = 1.0
+    min_value: float = 0.0
+    max_value: float = 0.0
+    scale_factor: float = 1.0
+    zero_point: Optional[int] = None
+
+
+@dataclass
 class QuantizedWeight:
     """QuantizedWeight (weights.rs:158-175): ternary values (int8, the reference stores them as f32 in a tensor),
     the scalar scale, the original shape; plus the packed bytes the BitLinear layer takes."""
@@ -448,6 +460,11 @@ class BitNetWeightQuantizer:
     def dequantize(self, quantized: QuantizedWeight) -> torch.Tensor:
         """weights.rs:616-619: values * scales (a host-side convenience through torch; not on the forward path)."""
         return quantized.values.to(torch.float32) * quantized.scales
+
+    def get_stats(self) -> QuantizationStats:
+        """Quantizer::get_stats (weights.rs:638-640): the quantizer's own record, which `quantize(&self)` never updates
+        in the reference, so the defaults; the figures of a call are in QuantizedWeight.stats."""
+        return QuantizationStats()
 
 
 def retile_weights(packed: torch.Tensor, n: int, k: int, layout: int = LAYOUT_OUT_IN, stream=None) -> torch.Tensor:
@@ -730,6 +747,29 @@ class BitLinear:
         _check(load_library().bitnet_hip_bitlinear_matmul(self._h, _ptr(a), _ptr(a_sum), m, _ptr(a_scale), _ptr(residual), _ptr(acc),
                                                           _ptr(out), _stream(stream)))
         return (out, acc) if want_acc else out
+
+    @property
+    def device(self) -> str:
+        """BitLinear::device (layer.rs:223): always the GPU the library was initialised on."""
+        return f"hip:{torch.cuda.current_device()}" if torch.cuda.is_available() else "hip"
+
+    def clear_cache(self):
+        """BitLinear::clear_cache (layer.rs:353-361).  The reference caches the quantised weights of the latent f32
+        tensor; here the layer holds nothing but the quantised weights (update_weights quantises at once), so there is
+        no cache to clear and the call succeeds without effect."""
+        return None
+
+    def cache_stats(self):
+        """BitLinear::cache_stats (layer.rs:364-368): None, as for a reference layer built without a cache."""
+        return None
+
+    def to_device(self, device) -> None:
+        """BitLinear::to_device (layer.rs:376-411).  A layer lives on the one GPU this library drives: a move to that
+        device is the reference's same-device no-op, anything else is refused."""
+        name = str(device)
+        if name in ("hip", "cuda", self.device, self.device.replace("hip", "cuda")):
+            return None
+        raise BitLinearError(DEVICE_ERROR, f"Failed to move weights to device: {name} (this layer lives on {self.device})")
 
     def forward_batch(self, x: torch.Tensor):
         """BitLinear::forward_batch (forward.rs:270-297): rank >= 2 required."""

@@ -191,6 +191,7 @@ mod imp {
         layer_name: String,
         handle: *mut ffi::bitnet_hip_bitlinear,
         stream: *mut c_void,
+        device: i32,  // the library drives one GPU per process: the ordinal given to `HipBackend::new`, 0 by default
         // scratch for the quantised activations and the staging buffers of the host-tensor entry points: grown on
         // demand, never allocated per call once warm
         scratch: Mutex<Scratch>,
@@ -212,7 +213,7 @@ mod imp {
                 ffi::bitnet_hip_bitlinear_create(config.in_features, config.out_features, config.use_bias as c_int, &mut handle)
             })?;
             let scratch = Scratch { workspace: DeviceBuffer::new(0)?, input: DeviceBuffer::new(0)?, output: DeviceBuffer::new(0)? };
-            Ok(Self { config, layer_name, handle, stream: ptr::null_mut(), scratch: Mutex::new(scratch) })
+            Ok(Self { config, layer_name, handle, stream: ptr::null_mut(), device: 0, scratch: Mutex::new(scratch) })
         }
         pub fn config(&self) -> &BitLinearConfig { &self.config }
         pub fn layer_name(&self) -> &str { &self.layer_name }
@@ -236,6 +237,23 @@ mod imp {
         pub fn update_bias(&self, bias: &[f32]) -> HipResult<()> {
             check(unsafe { ffi::bitnet_hip_bitlinear_set_bias(self.handle, bias.as_ptr(), bias.len(), 0, self.stream) })
         }
+        /// `BitLinear::clear_cache` (layer.rs:353-361).  The reference caches the quantised form of its latent f32
+        /// weights; this layer holds only the quantised weights (`update_weights` quantises at once), so there is
+        /// nothing to clear.
+        pub fn clear_cache(&self) -> HipResult<()> {
+            Ok(())
+        }
+        /// `BitLinear::to_device` (layer.rs:376-411): the layer lives on the GPU the library was initialised on; that
+        /// device is the reference's same-device no-op, any other ordinal is refused.
+        pub fn to_device(&mut self, device: i32) -> HipResult<()> {
+            if device == self.device {
+                Ok(())
+            } else {
+                Err(HipError::DeviceError(format!("Failed to move weights to device: {device} (the layer lives on {})", self.device)))
+            }
+        }
+        /// `BitLinear::device` (layer.rs:223): the ordinal of the GPU the layer was created on.
+        pub fn device(&self) -> i32 { self.device }
 
         /// The forward on device tensors: input [.., in_features] -> output [.., out_features]; `gamma` is the RMSNorm
         /// weight [in_features] applied before quantisation, if any.  The output's dims are checked here, so safe code

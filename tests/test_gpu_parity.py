@@ -1130,3 +1130,17 @@ def test_mfma_rate_diagnostic_is_plausible():
     rand, const = bh.measure_mfma_i8_rate(True), bh.measure_mfma_i8_rate(False)
     assert 500.0 < rand < 5100.0 and 500.0 < const < 5100.0
     assert const > 0.9 * rand
+
+
+def test_bitlinear_housekeeping_methods_of_the_reference():
+    """clear_cache / cache_stats / to_device / device (layer.rs:223,353-411) and Quantizer::get_stats (weights.rs:638-640)
+    as the reference's call sites use them: nothing to clear, the same device is a no-op, another device is refused."""
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=64, out_features=32), "api")
+    assert layer.clear_cache() is None and layer.cache_stats() is None
+    assert layer.device.startswith("hip")
+    assert layer.to_device(layer.device) is None and layer.to_device("cuda") is None
+    with pytest.raises(bh.BitLinearError) as ei:
+        layer.to_device("cpu")
+    assert ei.value.kind == "DeviceError"
+    stats = bh.BitNetWeightQuantizer().get_stats()
+    assert (stats.elements_count, stats.quantization_error, stats.compression_ratio, stats.scale_factor, stats.zero_point) == (0, 0.0, 1.0, 1.0, None)
