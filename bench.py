@@ -336,6 +336,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip roofline / prefill / CPU legs (profiling runs)")
     ap.add_argument("--only-prefill", type=int, default=0, metavar="REPS",
                     help="run only the two M=2048 prefill GEMMs REPS times each and print their rates (profiling runs)")
+    ap.add_argument("--only-batch8", type=int, default=0, metavar="STEPS",
+                    help="run only STEPS token steps of the 30-layer stack at batch 8 (profiling runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -353,6 +355,18 @@ def main():
     dec, gen = build_stack(bh, torch, LAYERS)
     if args.only_prefill > 0:
         print(json.dumps({"prefill": prefill_rates(bh, torch, dec, gen, reps=args.only_prefill)}))
+        return
+    if args.only_batch8 > 0:
+        big = bh.DecoderProjections(LAYERS, HIDDEN, FFN, Q_HEADS, KV_HEADS, HEAD_DIM, eps=1e-5, max_tokens=8)
+        for l in range(LAYERS):
+            for p in range(7):
+                packed, scale = dec.projection(l, p).get_quantized_weights()
+                big.projection(l, p).set_quantized_weights(packed.cuda(), scale)
+        x8 = torch.randn((8, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
+        y8 = torch.empty_like(x8)
+        big.decode(x8, out=y8)
+        ms = time_events(torch, lambda: [big.decode(x8, out=y8) for _ in range(args.only_batch8)]) / args.only_batch8
+        print(json.dumps({"stack30_batch8": {"us_per_token_step": round(ms * 1e3, 1), "steps": args.only_batch8}}))
         return
     x = torch.randn((1, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
 
