@@ -319,11 +319,18 @@ def cpu_baseline(torch, dec, budget_s=8.0):
                 "ref_simd_all_cores": sample(ref_simd, cores, 3.0), "ref_simd_1_thread": sample(ref_simd, 1, 3.0),
                 "oracle_i8_all_cores": sample(oracle_i8, cores, 3.0), "oracle_i8_1_thread": sample(oracle_i8, 1, 3.0)}
     orc.cpu_set_threads(cores)
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((line.split(":", 1)[1].strip() for line in f if line.startswith("model name")), model)
+    except OSError:
+        pass
     return {
-        "value": main_leg["gbs"], "unit": "GB/s", "cores": cores, "kind": "port",
+        "value": main_leg["gbs"], "unit": "GB/s", "cores": cores, "kind": "port", "cpu_model": model,
         "sample": f"{main_leg['passes']} passes over one layer's 7 projections at batch 1 (dequantise to f32 + f32 GEMV per call, "
-                  f"{orc.cpu_isa()}), {main_leg['ms_per_layer']:.2f} ms per layer",
-        "ms_per_step": main_leg["ms_per_layer"], "variants": variants,
+                  f"{orc.cpu_isa()}), {main_leg['ms_per_layer']:.2f} ms per layer = {main_leg['ms_per_layer'] * LAYERS:.1f} ms per "
+                  f"30-layer step of the GPU figure",
+        "ms_per_layer": main_leg["ms_per_layer"], "ms_per_step": round(main_leg["ms_per_layer"] * LAYERS, 2), "variants": variants,
     }
 
 
