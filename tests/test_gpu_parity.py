@@ -428,6 +428,22 @@ def test_token_group_gemv_bit_exact(m, n, k):
     assert np.array_equal(host(acc2), acc_ref)
 
 
+@pytest.mark.parametrize("m,n,k", [(96, 2560, 6912), (130, 2560, 6912), (256, 2560, 6912), (128, 6912, 2560), (200, 650, 2560),
+                                   (256, 4800, 3072), (257, 2560, 6912), (192, 6912, 2560)])
+def test_token_group_gemv_takes_small_prefill_launches(m, n, k):
+    """96 to 256 tokens on matrices that would give the prefill GEMM fewer than 64 tiles of 128 x 160: the token-group
+    GEMV runs instead (the last two cases stay with the GEMM: 257 tokens, and 88 tiles).  Same results either way."""
+    rng = np.random.default_rng(m + n + k)
+    packed, ws, a, a_scale = make_problem(rng, m, n, k, outliers=True)
+    tiled = bh.retile_weights(dev(packed), n, k)
+    res = rng.standard_normal((m, n), dtype=f32)
+    a_sum = dev(a.astype(np.int32).sum(axis=1).astype(np.int32))
+    acc, out = bh.matmul_w2a8(tiled, dev(a), n, dev(np.array([ws], dtype=f32)), dev(a_scale), residual=dev(res), a_sum=a_sum)
+    acc_ref = orc.gemm_w2a8(packed, a, n)
+    assert np.array_equal(host(acc), acc_ref)
+    assert np.array_equal(host(out), orc.epilogue(acc_ref, ws, a_scale, None, res))
+
+
 @pytest.mark.parametrize("n,k", [(6912, 2560), (2560, 6912)])
 @pytest.mark.parametrize("with_sum", [True, False], ids=["lds_direct_kernel", "register_staged_kernel"])
 def test_prefill_gemm_full_size(n, k, with_sum):
@@ -679,10 +695,11 @@ def test_bitlinear_forward_shapes_bias_norm_and_layouts():
     assert np.array_equal(host(layer_p.forward(dev(x))), ref0)
 
 
-@pytest.mark.parametrize("m", [1, 3, 8, 20, 40, 64, 200, 1100])
+@pytest.mark.parametrize("m", [1, 3, 8, 20, 40, 64, 200, 300, 1100])
 def test_forward_multi_matches_single_forwards(m):
     """q/k/v-style: several layers on one input give exactly what each layer gives alone, and what the oracle gives.
-    (m = 200 and 1100: the projections share launches of the 64 x 160 and of the eight-wavefront prefill GEMM.)"""
+    (m = 200: the token-group GEMV, which takes prefill launches too small for the GEMM to fill the chip; m = 300 and
+    1100: the projections share launches of the 64 x 160 and of the eight-wavefront prefill GEMM.)"""
     rng = np.random.default_rng(40 + m)
     k = 2560
     ns = [2560, 640, 640, 96]
