@@ -178,9 +178,9 @@ int run_projections(bitnet_hip_bitlinear *const *layers, int count, const float 
     int rc = launch_act_quant(x, x2, ldx, m, k, input_mode, gqa_group, head_dim, gamma, eps, sum_order, q, a_scale, a_sum,
                               nullptr, s);
     if (rc != BITNET_HIP_OK) return rc;
-    size_t n_tiles = 0;  // 160-column tiles the prefill GEMM would cut the outputs into
-    for (int j = 0; j < count; ++j) n_tiles += (layers[j]->out_features + 159) / 160;
-    if (gemv_takes(m, k, n_tiles, q)) {
+    size_t n_blocks = 0;
+    for (int j = 0; j < count; ++j) n_blocks += row_blocks(layers[j]->out_features);
+    if (gemv_takes(m, k, n_blocks, q)) {
         for (int j0 = 0; j0 < count; j0 += GEMV_MAX_PROJ) {
             GemvProj pjs[GEMV_MAX_PROJ];
             const int nj = count - j0 < GEMV_MAX_PROJ ? count - j0 : GEMV_MAX_PROJ;
@@ -510,7 +510,7 @@ int bitnet_hip_matmul_w2a8(const uint8_t *tiled, const int8_t *a, const int32_t 
     if (reinterpret_cast<uintptr_t>(tiled) % 16)
         return fail(BITNET_HIP_INVALID_CONFIG, "matmul_w2a8: tiled weights must be 16-byte aligned");
     if (n > 0x7fffffffu || k > 0x7fffffffu) return fail(BITNET_HIP_UNSUPPORTED, "matmul_w2a8: dimension too large");
-    if (gemv_takes(m, k, (n + 159) / 160, a)) {
+    if (gemv_takes(m, k, row_blocks(n), a)) {
         GemvProj pj = {tiled, w_scale, bias, residual, out, acc, n};
         return launch_gemv_tiled(&pj, 1, a, a_scale, m, k, as_stream(stream));
     }

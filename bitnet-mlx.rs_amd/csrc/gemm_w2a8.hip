@@ -842,7 +842,7 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
     if (nproj > GEMM_MAX_PROJ) return BITNET_HIP_UNSUPPORTED;
     bool dma_ok = a_sum != nullptr && m >= 96 && k % 256 == 0 && k >= 512 && (reinterpret_cast<uintptr_t>(a) & 15) == 0 &&
                   m * k < (1ull << 32);  // 32-bit lane offsets
-    size_t tiles = 0, tiles128 = 0;  // 128 x 160 tiles; 128 x 128 tiles, or 0 if a projection is not a multiple of 128 wide
+    size_t tiles = 0, tiles128 = 0, tiles64 = 0, tiles32 = 0;  // 128 x 160 tiles; 128 x 128 tiles, or 0 if a projection is not a multiple of 128 wide
     bool all128 = true;
     GemmParams p = {};
     for (int j = 0; j < nproj && dma_ok; ++j) {
@@ -850,6 +850,8 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
         dma_ok = s.n > 0 && s.n <= 0x7fffffffu && tiled_bytes(s.n, k) < (1ull << 32);
         tiles += ((m + 127) / 128) * ((s.n + 159) / 160);
         tiles128 += ((m + 127) / 128) * ((s.n + 127) / 128);
+        tiles64 += ((m + 63) / 64) * ((s.n + 63) / 64);
+        tiles32 += ((m + 63) / 64) * ((s.n + 31) / 32);
         all128 = all128 && s.n % 128 == 0;
         GemmProjDev &d = p.proj[j];
         d.w = s.tiled; d.w_scale = s.w_scale; d.bias = s.bias; d.residual = s.residual; d.out = s.out; d.acc = s.acc;
@@ -869,6 +871,13 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
     //                                           and two loader wavefronts;
     //   otherwise                            -> 64 x 160, four workgroups of 4 wavefronts per compute unit.
     if (tiles >= 640) return launch_dma<128, 160, 2, 3>(p, stream);
+    // Few tiles: a workgroup walks the whole of k by itself and its time is a chain of load latencies, so small
+    // launches take narrow tiles (more workgroups, all resident at once) with four stages of loads in flight.
+    // tiles64 / tiles32: 64 x 64 and 64 x 32 tiles of the launch.  Measured at 6912 -> 2560: 384 tokens 35.4 -> 23.3 us,
+    // 512 tokens 36.6 -> 25.8 us (64 x 32), 768 tokens 38.0 -> 29.6 us, 1024 tokens 36.8 -> 34.3 us (64 x 64);
+    // 2560 -> 6912 at 192 tokens 17.5 -> 13.6 us, at 384 tokens 20.0 -> 17.7 us.
+    if (tiles < 100 && tiles32 <= 704) return launch_dma<64, 32, 4, 4>(p, stream);
+    if (tiles <= 140 && tiles64 <= 768) return launch_dma<64, 64, 4, 3>(p, stream);
     if (tiles >= 100 && tiles <= 256) return launch_ld8<128, 160>(p, stream);
     // between one and 2.5 tiles of 128 x 160 per compute unit: 128 x 128 tiles when they divide every projection and
     // fill the 768 workgroup slots almost three times (q + k + v at 3072 tokens: 33.0 us against 37.9 us with 64 x 160)

@@ -49,17 +49,20 @@ int launch_untile(const uint8_t *tiled, size_t n, size_t k, uint8_t *packed, hip
 int launch_gemv_rowmajor(const uint8_t *packed, const int8_t *a, int32_t *out, size_t n, size_t k,
                          hipStream_t stream);
 constexpr int GEMV_MAX_M = 95;      // token rows the decode-GEMV path always takes
-// More rows go to the prefill GEMM, unless that would have so few 128 x 160 tiles that most compute units idle while
-// each workgroup walks the whole of k (measured at 6912 -> 2560: 33 us at any token count from 96 to 1024): up to
-// GEMV_WIDE_MAX_M rows the token-group GEMV takes launches of fewer than GEMV_WIDE_TILES such tiles, where its
-// conditions hold (k a multiple of 256 up to 8192, 16-byte aligned rows).  At 128 tokens: 14.1 us against 16.8 us
-// (2560 -> 6912), 21.8 us against 33.1 us (6912 -> 2560); at 256 tokens 30.7 us against 33.8 us.
-constexpr int GEMV_WIDE_MAX_M = 256, GEMV_WIDE_TILES = 64;
-inline bool gemv_takes(size_t m, size_t k, size_t n_tiles_160, const void *a)
+// More rows go to the prefill GEMM, except where the token-group GEMV (gemv_mfma_tg_kernel: k a multiple of 256 up to
+// 8192, 16-byte aligned rows) runs as a single round of workgroups: it then beats a GEMM that is too small to fill the
+// chip (6912 -> 2560 at 96 tokens: 13.6 us against 18.9 us; 2560 -> 2560 up to 192 tokens: 8.4 .. 9.8 us against
+// 10.7 .. 11.0 us), and loses as soon as its workgroups need a second round (6912 -> 2560 at 112 tokens: 21.6 us
+// against 19.1 us).  n_blocks: 16-row blocks of all projections of the launch.  The row blocks per workgroup and
+// the workgroup slots follow launch_gemv_tiled.
+constexpr int GEMV_WIDE_MAX_M = 512;
+inline bool gemv_takes(size_t m, size_t k, size_t n_blocks, const void *a)
 {
     if (m <= (size_t)GEMV_MAX_M) return true;
-    return m <= (size_t)GEMV_WIDE_MAX_M && ((m + 127) / 128) * n_tiles_160 < (size_t)GEMV_WIDE_TILES && k % 256 == 0 && k <= 8192 &&
-           (reinterpret_cast<uintptr_t>(a) & 15) == 0;
+    if (m > (size_t)GEMV_WIDE_MAX_M || k % 256 != 0 || k > 8192 || (reinterpret_cast<uintptr_t>(a) & 15) != 0) return false;
+    const size_t tgroups = (m + 15) / 16, slots = k <= 3072 ? 768 : 256;
+    const size_t rb = n_blocks * tgroups > 2 * slots ? 4 : (n_blocks * tgroups > slots ? 2 : 1);
+    return (n_blocks + rb - 1) / rb * tgroups <= slots;
 }
 constexpr int GEMV_MFMA_MAX_M = 64; // rows per launch of the MFMA variant of the decode GEMV (2 and more rows)
 constexpr int GEMV_MAX_PROJ = 3;  // projections sharing one input row per launch (q,k,v / gate,up)

@@ -429,10 +429,12 @@ def test_token_group_gemv_bit_exact(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(96, 2560, 6912), (130, 2560, 6912), (256, 2560, 6912), (128, 6912, 2560), (200, 650, 2560),
-                                   (256, 4800, 3072), (257, 2560, 6912), (192, 6912, 2560)])
-def test_token_group_gemv_takes_small_prefill_launches(m, n, k):
-    """96 to 256 tokens on matrices that would give the prefill GEMM fewer than 64 tiles of 128 x 160: the token-group
-    GEMV runs instead (the last two cases stay with the GEMM: 257 tokens, and 88 tiles).  Same results either way."""
+                                   (256, 4800, 3072), (257, 2560, 6912), (192, 6912, 2560), (500, 2560, 6912), (700, 2577, 6912),
+                                   (384, 6912, 2560), (1000, 2560, 2560), (160, 2560, 2560)])
+def test_small_prefill_launches_bit_exact(m, n, k):
+    """96 to 257 tokens, where the launch is too small for the 128 x 160 GEMM tiles to fill the chip: the token-group GEMV
+    while its workgroups fit one round (96 tokens at 6912 -> 2560, 200 tokens at 650 rows), else the GEMM with narrow
+    tiles and four stages of loads in flight (64 x 32 or 64 x 64).  Same results whichever runs."""
     rng = np.random.default_rng(m + n + k)
     packed, ws, a, a_scale = make_problem(rng, m, n, k, outliers=True)
     tiled = bh.retile_weights(dev(packed), n, k)
