@@ -142,6 +142,18 @@ def prefill_rates(bh, torch, dec, gen, reps):
         bl.forward(x)
         fwd_ms = min(time_events(torch, lambda: [bl.forward(x) for _ in range(reps)]) for _ in range(3)) / reps
         res[name]["forward_f32_in_ms"] = round(fwd_ms, 4)
+        # calibration only: the vendor library's int8 GEMM (torch._int_mm -> hipBLASLt) at the same shape, on weights
+        # expanded to one int8 per value and without the scale epilogue (int32 output); not part of the measured path
+        try:
+            w8 = torch.randint(-1, 2, (n, k), generator=gen, device="cuda", dtype=torch.int8)
+            torch._int_mm(a, w8.t())
+            lib_ms = min(time_events(torch, lambda: [torch._int_mm(a, w8.t()) for _ in range(reps)]) for _ in range(3)) / reps
+            res[name]["vendor_int8_gemm_ms"] = round(lib_ms, 4)
+            res[name]["vendor_int8_gemm_tops"] = round(2.0 * m * n * k / (lib_ms * 1e-3) / 1e12, 1)
+            del w8
+        except Exception as exc:  # the calibration must never fail the benchmark
+            res[name]["vendor_int8_gemm_ms"] = None
+            res[name]["vendor_int8_gemm_note"] = repr(exc)[:120]
         del a, out, x
     # projections that share their input in one call: one quantiser pass, one GEMM launch for all of them
     x = torch.randn((m, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
