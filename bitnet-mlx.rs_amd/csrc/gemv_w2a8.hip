@@ -425,15 +425,23 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
     }
 }
 
-// The same launch with 16 wavefronts per workgroup.  The prologue of gemv_fused_kernel is redundant arithmetic on
-// one wavefront per SIMD (normalise, absmax, quantise: about half of the dependent work of a launch); 1024 threads
-// do the element-wise part four times faster.  Thread t owns chunks t, t + 1024 (NCHB of them); the sum of squares
+// The same launch with up to 16 wavefronts per workgroup.  The prologue of gemv_fused_kernel is redundant arithmetic on
+// one wavefront per SIMD (normalise, absmax, quantise: about half of the dependent work of a launch); a thread per
+// chunk does the element-wise part four times faster.  A workgroup has nw wavefronts (bs = 64 nw threads), thread t
+// owns chunks t, t + bs (NCHB of them) and wavefront w the k-tiles w, w + nw; the sum of squares
 // keeps the declared order: chunk c belongs to virtual lane c % 256, whose chain runs over its chunks in ascending
 // order, so threads 0..255 (one per virtual lane) also fetch their lane's chunks (from L2, with the first loads of the
 // kernel) and add the squares up in that order, then the four 64-lane butterflies as before.
 // A 256-column k-tile is the 64 chunks one wavefront quantises, so every wavefront multiplies the tiles of its own
 // chunks (for each of the workgroup's RBW row blocks) straight after writing them to LDS, without a workgroup barrier
 // between quantiser and dot products; the partial sums of a row meet in LDS atomics.
+
+// Wavefronts per workgroup of gemv_fused16_kernel for a row of k columns.
+__host__ __device__ inline int fused16_waves(int k)
+{
+    const int kt = (k + 255) >> 8;
+    return kt > 16 ? 16 : (kt < 4 ? 4 : kt);
+}
 
 template <int MODE, bool NORM, int NCHB, int RBW>
 __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, const float *hot_x2, const float *hot_gamma, int hot_k, int hot_head_dim,
@@ -447,7 +455,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     // load from the argument buffer that the first address computation would have to wait for.
     RowSource hot;
     hot.x = hot_x; hot.x2 = hot_x2; hot.gamma = hot_gamma; hot.ldx = (size_t)hot_ldx; hot.k = hot_k; hot.head_dim = hot_head_dim;
-    hot.gqa_group = hot_gqa_group; hot.sum_order = BITNET_HIP_SUM_BLOCK256; hot.eps = 0.0f;
+    hot.gqa_group = hot_gqa_group & 0xffff; hot.sum_order = BITNET_HIP_SUM_BLOCK256; hot.eps = 0.0f;
     const size_t tok = blockIdx.x >> 3;
     const int group = (int)blockIdx.y * 8 + (int)(blockIdx.x & 7);  // may lie past the last group: such workgroups leave below
     extern __shared__ uint4 lds_a[];  // int8 activations, zero past K
@@ -457,6 +465,14 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int chunks = hot_k >> 2;
+    // A row of at most 1024 chunks is launched with one wavefront per k-tile (at least the four of the summation order)
+    // instead of 16: wavefronts without a chunk would only add their share of the redundant arithmetic between the
+    // barriers to the SIMDs' queues.  Their slots of the cross-wavefront reductions hold the neutral element.
+    const int nw = hot_gqa_group >> 16, bs = nw << 6;  // wavefronts and threads of the workgroup (preloaded with the GQA group)
+    if (tid < 16 && tid >= nw) {
+        red_f[1][tid] = 0.0f;
+        red_i[tid] = 0;
+    }
 
     // Every load is unconditional (clamped indices, values discarded), in the order in which the data is needed.
     // First what the preloaded arguments alone address: the input row and the RMSNorm weights.  The argument buffer is
@@ -465,7 +481,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     float4 v[NCHB], gm[NORM ? NCHB : 1];
     constexpr int NSS = NORM ? 4 * NCHB : 1;  // chunks per virtual lane of the summation order
 #pragma unroll
-    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(hot, tok, min(tid + 1024 * i, chunks - 1));
+    for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(hot, tok, min(tid + bs * i, chunks - 1));
     if constexpr (NORM) {
         float4 vs[NSS];
         if (wave < 4) {  // thread tid < 256 is virtual lane tid: it fetches the lane's chunks itself (from L2)
@@ -473,7 +489,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
             for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(hot, tok, min(tid + 256 * i, chunks - 1));
         }
 #pragma unroll
-        for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(hot, min(tid + 1024 * i, chunks - 1), true);
+        for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(hot, min(tid + bs * i, chunks - 1), true);
         if (wave < 4) {
             float part = 0.0f;
 #pragma unroll
@@ -506,7 +522,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
         for (int r = 0; r < RBW; ++r)
 #pragma unroll
             for (int i = 0; i < NCHB; ++i)
-                wt[r][i] = load_weight_slot(tiles + ((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + 16 * i, p.kt_count - 1)) * 64);
+                wt[r][i] = load_weight_slot(tiles + ((size_t)min(rb0 + r, rb_count - 1) * p.kt_count + min(wave + nw * i, p.kt_count - 1)) * 64);
         __builtin_amdgcn_sched_barrier(0);
     };
     // epilogue operands: absent ones read the input row instead (always there) and are not used; the weight scale goes
@@ -520,7 +536,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     if (tid < RBW * TILE_ROWS) tot[tid >> 4][tid & 15] = 0;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i)
-        if (tid + 1024 * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (tid + bs * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     if constexpr (NORM) {
         lds_barrier();
@@ -529,7 +545,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
         const RowDivisor rdiv = make_row_divisor(rms_from_ss(ss, p.k, p.src.eps));
 #pragma unroll
         for (int i = 0; i < NCHB; ++i)
-            if (tid + 1024 * i < chunks) v[i] = normalize4(v[i], rdiv, gm[i]);
+            if (tid + bs * i < chunks) v[i] = normalize4(v[i], rdiv, gm[i]);
     }
     float amax = 0.0f;
 #pragma unroll
@@ -546,7 +562,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     int isum = 0;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i) {
-        const int c = tid + 1024 * i;
+        const int c = tid + bs * i;
         if (c < chunks) {
             const uint32_t packed = quant4_packed(v[i], scale, &isum);
             lds_w[c] = packed;
@@ -570,7 +586,7 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     const bool row0 = (lane & 15) == 0;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i) {
-        const int kt = wave + 16 * i;
+        const int kt = wave + nw * i;
         if (kt < p.kt_count) {  // uniform over the wavefront
             v4i_t acc[RBW];
 #pragma unroll
@@ -1249,14 +1265,25 @@ int launch_fused_mode(const GemvParams &p, hipStream_t stream)
 template <int MODE, int RBW>
 int launch_fused16_mode(const GemvParams &p, hipStream_t stream)
 {
-    const bool norm = p.src.gamma != nullptr, one = (p.k >> 2) <= 1024;
+    const bool norm = p.src.gamma != nullptr;
     const size_t lds = (size_t)p.kt_count * 16 * sizeof(uint4);
     const dim3 grid(8u * (unsigned)p.m, ((unsigned)p.proj[p.nproj - 1].rb_end + 7u) / 8u);
-#define BITNET_HOT_ARGS p.src.x, p.src.x2, p.src.gamma, p.src.k, p.src.head_dim, p.src.gqa_group, (int)p.src.ldx
-    if (norm && one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 1, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
-    else if (norm) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, 2, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
-    else if (one) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, 1, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
-    else hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, 2, RBW>), grid, dim3(1024), lds, stream, BITNET_HOT_ARGS, p);
+    // One wavefront per k-tile (at least the four of the summation order) for rows of up to 16 k-tiles, one chunk per
+    // thread; 16 wavefronts and two chunks per thread above.  Fewer wavefronts with more chunks each are slower (the
+    // element-wise steps lose their parallelism: 2560 columns on 5 wavefronts 581 us per 30-layer step against 507 on 10).
+    const int nchb = p.kt_count <= 16 ? 1 : 2;
+    const int nw = p.kt_count <= 16 ? fused16_waves(p.src.k) : 16;
+    if (p.src.gqa_group < 0 || p.src.gqa_group > 0xffff) return fail(BITNET_HIP_INVALID_CONFIG, "GQA group %d out of range", p.src.gqa_group);
+    const dim3 block(64u * (unsigned)nw);
+#define BITNET_HOT_ARGS p.src.x, p.src.x2, p.src.gamma, p.src.k, p.src.head_dim, p.src.gqa_group | (nw << 16), (int)p.src.ldx
+#define BITNET_F16_LAUNCH(NCHB) \
+    do { \
+        if (norm) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, NCHB, RBW>), grid, block, lds, stream, BITNET_HOT_ARGS, p); \
+        else hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, NCHB, RBW>), grid, block, lds, stream, BITNET_HOT_ARGS, p); \
+    } while (0)
+    if (nchb == 1) BITNET_F16_LAUNCH(1);
+    else BITNET_F16_LAUNCH(2);
+#undef BITNET_F16_LAUNCH
 #undef BITNET_HOT_ARGS
     BITNET_HIP_CHECK_LAUNCH("gemv_fused16_kernel");
     return BITNET_HIP_OK;
