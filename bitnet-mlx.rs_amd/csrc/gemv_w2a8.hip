@@ -436,13 +436,6 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvParams p)
 // chunks (for each of the workgroup's RBW row blocks) straight after writing them to LDS, without a workgroup barrier
 // between quantiser and dot products; the partial sums of a row meet in LDS atomics.
 
-// Wavefronts per workgroup of gemv_fused16_kernel for a row of k columns.
-__host__ __device__ inline int fused16_waves(int k)
-{
-    const int kt = (k + 255) >> 8;
-    return kt > 16 ? 16 : (kt < 4 ? 4 : kt);
-}
-
 template <int MODE, bool NORM, int NCHB, int RBW>
 __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, const float *hot_x2, const float *hot_gamma, int hot_k, int hot_head_dim,
                                                            int hot_gqa_group, int hot_ldx, GemvParams p)
@@ -1272,7 +1265,7 @@ int launch_fused16_mode(const GemvParams &p, hipStream_t stream)
     // thread; 16 wavefronts and two chunks per thread above.  Fewer wavefronts with more chunks each are slower (the
     // element-wise steps lose their parallelism: 2560 columns on 5 wavefronts 581 us per 30-layer step against 507 on 10).
     const int nchb = p.kt_count <= 16 ? 1 : 2;
-    const int nw = p.kt_count <= 16 ? fused16_waves(p.src.k) : 16;
+    const int nw = p.kt_count <= 16 ? row_workgroup_waves(p.src.k) : 16;
     if (p.src.gqa_group < 0 || p.src.gqa_group > 0xffff) return fail(BITNET_HIP_INVALID_CONFIG, "GQA group %d out of range", p.src.gqa_group);
     const dim3 block(64u * (unsigned)nw);
 #define BITNET_HOT_ARGS p.src.x, p.src.x2, p.src.gamma, p.src.k, p.src.head_dim, p.src.gqa_group | (nw << 16), (int)p.src.ldx

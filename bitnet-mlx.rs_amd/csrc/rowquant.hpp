@@ -36,6 +36,15 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Wavefronts per workgroup of gemv_fused16_kernel for a row of k columns: one per 256 columns, at least the four of
+// the declared summation order, at most 16.  (The stand-alone quantiser with a workgroup per row gains nothing from
+// the same rule: measured on the 8- to 16-token decoder stack.)
+__host__ __device__ inline int row_workgroup_waves(int k)
+{
+    const int kt = (k + 255) >> 8;
+    return kt > 16 ? 16 : (kt < 4 ? 4 : kt);
+}
+
 struct RowSource {
     const float *x;      // [m, ldx]
     const float *x2;     // second operand of RELU2_MUL
