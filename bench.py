@@ -76,7 +76,7 @@ STEP_BYTES = LAYER_BYTES * LAYERS
 # script with --no-extras --calibration-copy), each scaled by what the same counter reads for the plain
 # 256 MiB copy: FETCH_SIZE reads 0.5 KiB per KiB fetched (factor 2.0), WRITE_SIZE 1.0 (factor 1.0).
 # Summary: profiles/decode_layer_b1_gemv_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_685_792
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_685_968
 
 
 def decode_roofline(event_ms, steps):
@@ -186,9 +186,15 @@ def stack_latency(bh, torch, dec, gen, reps=20):
         x = torch.randn((m, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
         y = torch.empty_like(x)
         big.decode(x, out=y)
-        ms = time_events(torch, lambda: [big.decode(x, out=y) for _ in range(reps)]) / reps
+        eager_ms = time_events(torch, lambda: [big.decode(x, out=y) for _ in range(reps)]) / reps
+        recorded = big.record(x, out=y)
+        recorded.replay()
+        ms = sorted(time_events(torch, lambda: [recorded.replay() for _ in range(reps)]) / reps for _ in range(3))[1]
         out[f"stack30_batch{m}"] = {"us_per_token_step": round(ms * 1e3, 1),
-                                    "gbs_packed_weights": round(dec.weight_bytes() / (ms * 1e-3) / 1e9, 1)}
+                                    "gbs_packed_weights": round(dec.weight_bytes() / (ms * 1e-3) / 1e9, 1),
+                                    "eager_launches_us_per_token_step": round(eager_ms * 1e3, 1),
+                                    "timed": "the recorded step replayed (HIP graph); eager = launches enqueued one by one"}
+        del recorded
     del big
     # the decode GEMV where a launch is large enough to be bound by bandwidth rather than by launch latency:
     # 32768 x 16384 ternary weights (128 MiB packed), int8 activations already quantised, one token
@@ -238,6 +244,25 @@ def sequential_order_decode(bh, torch, dec, gen, reps=20):
     ms = times[len(times) // 2]
     return {"us_per_layer_step": round(ms * 1e3 / dec.layers, 2), "gbs_packed_weights": round(dec.weight_bytes() / (ms * 1e-3) / 1e9, 1),
             "timed": f"median of 5 loops of {reps} 30-layer token steps"}
+
+
+def eager_decode(torch, dec, x, reps=20):
+    """The headline step with its 120 launches enqueued one by one by the host, and what that enqueue costs the host:
+    where the host needs longer per launch than the GPU, the loop runs at the host's pace."""
+    dec.decode(x, out=x)
+    torch.cuda.synchronize()
+    host = []
+    for _ in range(9):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.decode(x, out=x)
+        host.append(time.perf_counter() - t0)
+    host_us = sorted(host)[len(host) // 2] * 1e6
+    times = sorted(time_events(torch, lambda: [dec.decode(x, out=x) for _ in range(reps)]) / reps for _ in range(5))
+    ms = times[len(times) // 2]
+    return {"us_per_token_step": round(ms * 1e3, 1), "gbs_packed_weights": round(dec.weight_bytes() / (ms * 1e-3) / 1e9, 1),
+            "host_enqueue_us_per_step": round(host_us, 1), "host_enqueue_us_per_launch": round(host_us / LAUNCHES_PER_STEP, 2),
+            "timed": f"median of 5 loops of {reps} steps; enqueue = host time of one decode call into an idle queue"}
 
 
 def time_forward_graph(torch, bls, x, y, ws, replays=10):
@@ -353,6 +378,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip roofline / prefill / CPU legs (profiling runs)")
+    ap.add_argument("--eager", action="store_true",
+                    help="time the token step as 120 launches enqueued one by one from the host instead of replaying the "
+                         "recorded step (the eager loop is bound by the host's launch rate on most boxes)")
     ap.add_argument("--only-prefill", type=int, default=0, metavar="REPS",
                     help="run only the two M=2048 prefill GEMMs REPS times each and print their rates (profiling runs)")
     ap.add_argument("--only-batch8", type=int, default=0, metavar="STEPS",
@@ -383,17 +411,25 @@ def main():
                 big.projection(l, p).set_quantized_weights(packed.cuda(), scale)
         x8 = torch.randn((8, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
         y8 = torch.empty_like(x8)
-        big.decode(x8, out=y8)
-        ms = time_events(torch, lambda: [big.decode(x8, out=y8) for _ in range(args.only_batch8)]) / args.only_batch8
+        recorded8 = big.record(x8, out=y8)
+        recorded8.replay()
+        ms = time_events(torch, lambda: [recorded8.replay() for _ in range(args.only_batch8)]) / args.only_batch8
         print(json.dumps({"stack30_batch8": {"us_per_token_step": round(ms * 1e3, 1), "steps": args.only_batch8}}))
         return
     x = torch.randn((1, HIDDEN), generator=gen, device="cuda", dtype=torch.float32)
+
+    # The step is recorded once (bitnet_hip_decoder_graph_create: the 120 launches of decode() as a HIP graph) and
+    # replayed: the same kernels in the same order, enqueued by one host call.
+    recorded = None if args.eager else dec.record(x, out=x)
 
     def run_steps(count):
         """`count` token steps, each one call of the boundary: the seven projections of layers 0..29 in turn, the hidden
         state carried along (four launches per layer)."""
         for _ in range(count):
-            dec.decode(x, out=x)
+            if recorded is None:
+                dec.decode(x, out=x)
+            else:
+                recorded.replay()
 
     if args.calibration_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
@@ -427,7 +463,10 @@ def main():
         "config": {"workload": "configs[1]: one decoder layer's 7 decode projections at batch 1 "
                                "(hidden 2560, ffn 6912, 20q/5kv heads), passed 30 times per step over the 30 distinct "
                                "weight sets of a BitNet-2B stack (= one token step of configs[4] at batch 1); "
-                               "a step = 30 layers = 120 dependent kernel launches, one host call",
+                               "a step = 30 layers = 120 dependent kernel launches, one host call"
+                               + (" (launches enqueued one by one)" if args.eager else
+                                  " (bitnet_hip_decoder_graph_launch: the recorded step replayed)"),
+                   "enqueue": "eager launches" if args.eager else "recorded step (HIP graph)",
                    "layers_per_step": LAYERS, "bytes_per_step": STEP_BYTES, "bytes_per_layer": LAYER_BYTES,
                    "us_per_layer": round(elapsed * 1e6 / args.steps / LAYERS, 3),
                    "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
@@ -441,6 +480,7 @@ def main():
         line["prefill"] = prefill_rates(bh, torch, dec, gen, reps=5)
         line["other_configs"] = stack_latency(bh, torch, dec, gen)
         line["other_configs"]["decode_layer_b1_sum_order_sequential"] = sequential_order_decode(bh, torch, dec, gen)
+        line["other_configs"]["decode_b1_eager_launches"] = eager_decode(torch, dec, x)
         if not args.no_cpu_baseline:
             line["cpu_baseline"] = cpu_baseline(torch, dec)
     print(json.dumps(line))

@@ -472,6 +472,34 @@ public:
         if (rc != BITNET_HIP_OK) return last_error(rc);
         return out;
     }
+    // The decode step x -> out recorded as a HIP graph (the step runs once while it is recorded); replay() enqueues it
+    // with one call.  The graph shares ownership of nothing: keep the decoder and both tensors alive while it is used.
+    class Graph {
+    public:
+        Graph(Graph &&o) noexcept : handle_(o.handle_) { o.handle_ = nullptr; }
+        Graph(const Graph &) = delete;
+        Graph &operator=(const Graph &) = delete;
+        ~Graph() { if (handle_) bitnet_hip_decoder_graph_destroy(handle_); }
+        Result<Unit> replay(void *stream = nullptr) const
+        {
+            int rc = bitnet_hip_decoder_graph_launch(handle_, stream);
+            if (rc != BITNET_HIP_OK) return last_error(rc);
+            return Unit{};
+        }
+    private:
+        friend class DecoderProjections;
+        explicit Graph(bitnet_hip_decoder_graph *h) : handle_(h) {}
+        bitnet_hip_decoder_graph *handle_ = nullptr;
+    };
+    Result<Graph> record(const DeviceTensor &x, DeviceTensor &out) const
+    {
+        if (x.dims().size() != 2 || x.dims() != out.dims())
+            return BitLinearError{BitLinearError::ShapeMismatch, "record: x and out must be [m, hidden] tensors of one shape", x.dims(), out.dims()};
+        bitnet_hip_decoder_graph *g = nullptr;
+        int rc = bitnet_hip_decoder_graph_create(handle_, 0, layers, x.data(), x.dims()[0], out.data(), nullptr, nullptr, &g);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return Graph(g);
+    }
     bitnet_hip_decoder *handle() const { return handle_; }
     size_t hidden = 0, max_tokens = 0, layers = 0;
 

@@ -168,6 +168,25 @@ int main()
             CHECK(one.is_ok() && one.unwrap().to_vec() == res.unwrap()[i].to_vec());
         }
     }
+    {  // a recorded decode step replays to the bits of the eager step, also after its input has changed
+        auto dec = DecoderProjections::create(2, 256, 512, 4, 2, 64, 1e-5f, 4);
+        CHECK(dec.is_ok());
+        const size_t outs[7] = {256, 128, 128, 256, 512, 512, 256}, ins[7] = {256, 256, 256, 256, 256, 256, 512};
+        for (size_t l = 0; l < 2; ++l)
+            for (int p = 0; p < 7; ++p)
+                CHECK(dec.unwrap()->update_weights(l, p, randn(outs[p] * ins[p], 70 + (unsigned)(7 * l + p), 0.02f), outs[p], ins[p]).is_ok());
+        auto x = DeviceTensor::from_vec(randn(3 * 256, 90, 1.0f), {3, 256}).unwrap();
+        auto out = DeviceTensor::zeros({3, 256}).unwrap();
+        auto graph = dec.unwrap()->record(x, out);
+        CHECK(graph.is_ok());
+        for (unsigned round = 0; graph.is_ok() && round < 3; ++round) {
+            auto fresh = randn(3 * 256, 91 + round, 1.0f);
+            (void)hipMemcpy(x.data(), fresh.data(), fresh.size() * sizeof(float), hipMemcpyHostToDevice);
+            auto eager = dec.unwrap()->decode(x);
+            CHECK(graph.unwrap().replay().is_ok());
+            CHECK(eager.is_ok() && eager.unwrap().to_vec() == out.to_vec());
+        }
+    }
     std::printf(failures ? "host selftest: %d FAILED\n" : "host selftest: all passed\n", failures);
     return failures ? 1 : 0;
 }

@@ -127,6 +127,9 @@ def load_library() -> C.CDLL:
         "bitnet_hip_decoder_set_norm": (i32, [vp, sz, i32, vp, i32, vp]),
         "bitnet_hip_decoder_weight_bytes": (sz, [vp]),
         "bitnet_hip_decoder_decode": (i32, [vp, vp, sz, vp, vp, vp, vp]),
+        "bitnet_hip_decoder_graph_create": (i32, [vp, sz, sz, vp, sz, vp, vp, vp, C.POINTER(vp)]),
+        "bitnet_hip_decoder_graph_launch": (i32, [vp, vp]),
+        "bitnet_hip_decoder_graph_destroy": (None, [vp]),
         "bitnet_hip_backend_create": (i32, [i32, C.POINTER(vp)]),
         "bitnet_hip_backend_destroy": (None, [vp]),
         "bitnet_hip_backend_optimize_model": (i32, [vp, vp]),
@@ -862,6 +865,47 @@ class DecoderProjections:
         _check(load_library().bitnet_hip_decoder_decode_layers(self._h, lo, hi, _ptr(x), m, _ptr(out), _ptr(q), _ptr(k),
                                                                _stream(stream)))
         return (out, q, k) if want_qk else out
+
+    def record(self, x: torch.Tensor, out: Optional[torch.Tensor] = None, want_qk: bool = False,
+               layers: Optional[Sequence[int]] = None) -> "DecoderGraph":
+        """The decode step on these tensors recorded as a HIP graph (the step runs once while it is recorded); replay() then
+        reads x and writes out in place, for the price of one host call instead of four launches a block."""
+        _dev(x, torch.float32, "x")
+        if x.dim() != 2 or x.shape[1] != self.hidden:
+            raise BitLinearError(SHAPE_MISMATCH, "decode input", [x.shape[0] if x.dim() else 1, self.hidden], list(x.shape))
+        lo_hi = (0, self.layers) if layers is None else tuple(layers)
+        if len(lo_hi) != 2 or not (0 <= lo_hi[0] < lo_hi[1] <= self.layers):
+            raise BitLinearError(INVALID_CONFIG, f"layer range {lo_hi} outside [0, {self.layers}] or empty")
+        if out is None:
+            out = torch.empty_like(x)
+        else:
+            _dev(out, torch.float32, "out")
+            if tuple(out.shape) != tuple(x.shape) or out.device != x.device:
+                raise BitLinearError(SHAPE_MISMATCH, "decode output", list(x.shape), list(out.shape))
+        m = x.shape[0]
+        q = torch.empty((m, self.hidden), dtype=torch.float32, device=x.device) if want_qk else None
+        k = torch.empty((m, self.kv_dim), dtype=torch.float32, device=x.device) if want_qk else None
+        h = C.c_void_p()
+        _check(load_library().bitnet_hip_decoder_graph_create(self._h, lo_hi[0], lo_hi[1], _ptr(x), m, _ptr(out), _ptr(q),
+                                                              _ptr(k), C.byref(h)))
+        return DecoderGraph(h, self, x, out, q, k)
+
+
+class DecoderGraph:
+    """A recorded decode step (bitnet_hip_decoder_graph): keeps the decoder and the tensors it reads and writes alive."""
+
+    def __init__(self, handle, decoder, x, out, q, k):
+        self._h, self._decoder = handle, decoder
+        self.x, self.out, self.q, self.k = x, out, q, k
+
+    def replay(self, stream=None) -> torch.Tensor:
+        _check(load_library().bitnet_hip_decoder_graph_launch(self._h, _stream(stream)))
+        return self.out
+
+    def __del__(self):
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.bitnet_hip_decoder_graph_destroy(self._h)
+            self._h = None
 
 
 @dataclass

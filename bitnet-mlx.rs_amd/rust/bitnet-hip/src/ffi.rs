@@ -12,6 +12,10 @@ pub struct bitnet_hip_decoder {
     _private: [u8; 0],
 }
 #[repr(C)]
+pub struct bitnet_hip_decoder_graph {
+    _private: [u8; 0],
+}
+#[repr(C)]
 pub struct bitnet_hip_backend {
     _private: [u8; 0],
 }
@@ -137,6 +141,11 @@ extern "C" {
     pub fn bitnet_hip_decoder_decode_layers(dec: *mut bitnet_hip_decoder, layer_begin: usize, layer_end: usize,
                                             x_in: *const f32, m: usize, x_out: *mut f32, q_last: *mut f32,
                                             k_last: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_decoder_graph_create(dec: *mut bitnet_hip_decoder, layer_begin: usize, layer_end: usize,
+                                           x_in: *const f32, m: usize, x_out: *mut f32, q_last: *mut f32,
+                                           k_last: *mut f32, graph: *mut *mut bitnet_hip_decoder_graph) -> c_int;
+    pub fn bitnet_hip_decoder_graph_launch(graph: *mut bitnet_hip_decoder_graph, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_decoder_graph_destroy(graph: *mut bitnet_hip_decoder_graph);
     pub fn bitnet_hip_backend_create(device: c_int, backend: *mut *mut bitnet_hip_backend) -> c_int;
     pub fn bitnet_hip_backend_destroy(backend: *mut bitnet_hip_backend);
     pub fn bitnet_hip_backend_optimize_model(backend: *mut bitnet_hip_backend, model: *mut bitnet_hip_decoder) -> c_int;

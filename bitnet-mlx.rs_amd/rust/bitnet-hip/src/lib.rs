@@ -424,6 +424,38 @@ mod imp {
         }
     }
 
+    /// A decode step of a `HipDecoder` recorded as a HIP graph (bitnet_hip_decoder_graph_*): `replay` enqueues the
+    /// whole step with one call.  It borrows the decoder, so it cannot outlive it.
+    pub struct HipDecoderGraph<'a> {
+        handle: *mut ffi::bitnet_hip_decoder_graph,
+        _decoder: std::marker::PhantomData<&'a HipDecoder>,
+    }
+    impl HipDecoder {
+        /// Records the step `x_in [m, hidden] -> x_out [m, hidden]` through blocks `layers.start .. layers.end`.
+        /// # Safety
+        /// `x_in` and `x_out` are device pointers to `m * hidden` floats that stay valid for the life of the graph.
+        pub unsafe fn record(&self, layers: std::ops::Range<usize>, x_in: *const f32, m: usize, x_out: *mut f32)
+                             -> HipResult<HipDecoderGraph<'_>> {
+            if m > self.max_tokens {
+                return Err(HipError::ShapeMismatch { expected: vec![self.max_tokens, self.hidden], actual: vec![m, self.hidden] });
+            }
+            let mut handle = ptr::null_mut();
+            check(ffi::bitnet_hip_decoder_graph_create(self.handle, layers.start, layers.end, x_in, m, x_out, ptr::null_mut(),
+                                                       ptr::null_mut(), &mut handle))?;
+            Ok(HipDecoderGraph { handle, _decoder: std::marker::PhantomData })
+        }
+    }
+    impl HipDecoderGraph<'_> {
+        pub fn replay(&self) -> HipResult<()> {
+            check(unsafe { ffi::bitnet_hip_decoder_graph_launch(self.handle, ptr::null_mut()) })
+        }
+    }
+    impl Drop for HipDecoderGraph<'_> {
+        fn drop(&mut self) {
+            unsafe { ffi::bitnet_hip_decoder_graph_destroy(self.handle) }
+        }
+    }
+
     /// `InferenceBackend` for this path (bitnet-inference/src/engine/mod.rs:126-138), selected where
     /// `InferenceEngine::create_backend` selects the CPU / Metal backends (api/mod.rs:426-460).
     pub struct HipInferenceBackend {

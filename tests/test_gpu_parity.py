@@ -1057,6 +1057,73 @@ def test_decoder_repeated_calls_subranges_and_streams(dims, layers):
         assert np.array_equal(host(o), r)
 
 
+@pytest.mark.parametrize("dims,layers,m", [((2560, 6912, 20, 5, 128), 3, 1), ((2560, 6912, 20, 5, 128), 2, 8),
+                                           ((256, 512, 4, 2, 64), 3, 3), ((1024, 2816, 8, 8, 128), 2, 1)])
+def test_decoder_recorded_step_replays_match_the_oracle(dims, layers, m):
+    """A decode step recorded as a HIP graph (bitnet_hip_decoder_graph_*): every replay, with eager work and host
+    synchronisations between the replays and with new inputs written into the recorded input tensor, equals the oracle's
+    chain bit for bit; so do a recorded sub-range in place, replays on another stream, replays interleaved with eager
+    decode calls on the same decoder, and replays after a weight update (the graph reads the layers' buffers, which an
+    update keeps)."""
+    rng = np.random.default_rng(17 * layers + m + dims[0])
+    dec, ref = build_decoder_packed(rng, layers, *dims, max_tokens=max(m, 2))
+    x = dev(synth_activations(rng, m, dims[0]))
+    graph = dec.record(x, want_qk=True)
+    other = torch.cuda.Stream()
+    for round_ in range(4):
+        fresh = synth_activations(rng, m, dims[0])
+        x_ref, q_ref, k_ref = oracle_stack(ref, fresh, *dims)
+        x.copy_(dev(fresh))
+        graph.out.zero_()
+        if round_ == 2:  # another stream, ordered behind the copy above by an explicit wait
+            other.wait_stream(torch.cuda.current_stream())
+            graph.replay(stream=other)
+            torch.cuda.current_stream().wait_stream(other)
+        else:
+            graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(graph.out), x_ref), f"replay {round_}"
+        assert np.array_equal(host(graph.q), q_ref) and np.array_equal(host(graph.k), k_ref)
+        # eager work on the same decoder between the replays
+        assert np.array_equal(host(dec.decode(dev(fresh))), x_ref)
+    # a sub-range of blocks, in place
+    if layers >= 3:
+        start = oracle_stack(ref[:1], host(x), *dims)[0]
+        want = oracle_stack(ref[1:], start, *dims)[0]
+        buf = dev(start.copy())
+        sub = dec.record(buf, out=buf, layers=(1, layers))
+        for _ in range(2):
+            buf.copy_(dev(start))
+            sub.replay()
+            assert np.array_equal(host(buf), want)
+    # new weights in one projection: the recorded step reads them
+    n, k = dec.proj_shape(6)  # down
+    pk = random_packed_ternary(rng, n, k)
+    dec.projection(layers - 1, 6).set_quantized_weights(torch.from_numpy(pk), 0.02)
+    packed, scales, ga, gf = ref[-1]
+    ref[-1] = (packed[:6] + [pk], scales[:6] + [f32(0.02)], ga, gf)
+    x_ref = oracle_stack(ref, host(x), *dims)[0]
+    graph.replay()
+    assert np.array_equal(host(graph.out), x_ref)
+
+
+def test_decoder_recorded_step_argument_errors():
+    dec = bh.DecoderProjections(2, 256, 512, 4, 2, 64, max_tokens=2)
+    x = torch.zeros((1, 256), device="cuda")
+    with pytest.raises(bh.BitLinearError) as ei:  # no weights yet: nothing is recorded
+        dec.record(x)
+    assert ei.value.kind == "NotInitialized"
+    with pytest.raises(bh.BitLinearError) as ei:
+        dec.record(torch.zeros((3, 256), device="cuda"))
+    assert ei.value.kind == "ShapeMismatch"
+    with pytest.raises(bh.BitLinearError) as ei:
+        dec.record(x, layers=(1, 1))
+    assert ei.value.kind == "InvalidConfig"
+    lib = bh.load_library()
+    assert lib.bitnet_hip_decoder_graph_launch(None, None) == bh.NULL_POINTER
+    lib.bitnet_hip_decoder_graph_destroy(None)
+
+
 @pytest.mark.parametrize("layout", [bh.LAYOUT_OUT_IN, bh.LAYOUT_IN_OUT])
 @pytest.mark.parametrize("n,k", [(1, 4), (48, 300), (640, 2560)])
 def test_gguf_ternary_tensor_ingestion(n, k, layout):
