@@ -469,28 +469,20 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
 
     // Every load is unconditional (clamped indices, values discarded), in the order in which the data is needed.
     // First what the preloaded arguments alone address: the input row and the RMSNorm weights.  The argument buffer is
-    // read only after these loads are on their way and after the wavefronts of the summation order have added up
-    // their squares, so that its latency hides behind theirs.
+    // read once these loads are on their way (it takes as long to arrive as the row: both come from memory), then
+    // the sum of squares, so that the two latencies run side by side.
     float4 v[NCHB], gm[NORM ? NCHB : 1];
     constexpr int NSS = NORM ? 4 * NCHB : 1;  // chunks per virtual lane of the summation order
 #pragma unroll
     for (int i = 0; i < NCHB; ++i) v[i] = load_chunk<MODE, true>(hot, tok, min(tid + bs * i, chunks - 1));
+    float4 vs[NSS];
     if constexpr (NORM) {
-        float4 vs[NSS];
         if (wave < 4) {  // thread tid < 256 is virtual lane tid: it fetches the lane's chunks itself (from L2)
 #pragma unroll
             for (int i = 0; i < NSS; ++i) vs[i] = load_chunk<MODE, true>(hot, tok, min(tid + 256 * i, chunks - 1));
         }
 #pragma unroll
         for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(hot, min(tid + bs * i, chunks - 1), true);
-        if (wave < 4) {
-            float part = 0.0f;
-#pragma unroll
-            for (int i = 0; i < NSS; ++i)
-                if (tid + 256 * i < chunks) part = sum_squares4(part, vs[i]);  // chunks past the end would add +0
-            part = wave_sum_f32(part);
-            if (lane == 0) red_f[0][wave] = part;
-        }
     }
     __builtin_amdgcn_sched_barrier(0);  // nothing below moves above: the first wait for the argument buffer comes here
 
@@ -505,9 +497,10 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     const uint4 *tiles = reinterpret_cast<const uint4 *>(P.w) + lane;
     // k-tile kt holds chunks 64*kt .. 64*kt + 63: exactly what wavefront kt % 16 quantises, so a wavefront multiplies
     // the tiles of its own chunks (tiles and row blocks past the end repeat the last one; their results are not added).
-    // The tiles are requested right after the first workgroup barrier, not here: the chain of reductions that starts
-    // from the input row is what the kernel's duration hangs on, and a weight stream requested before the row has
-    // been reduced once holds that chain up (in the memory system and in the L1 that every wavefront's loads share).
+    // When the tiles are requested (measured on the 30-block token step, replayed from a graph): with RMSNorm, once
+    // the argument buffer has arrived, ahead of the sum of squares (483.4 us a step against 489.7 behind the first
+    // barrier); without it, behind the absmax barrier (requested as early there the step takes 494 us: the weight
+    // stream then competes with the input row, which the kernel's chain of reductions hangs on).
     uint4 wt[RBW][NCHB];
     auto request_weight_tiles = [&]() {
         __builtin_amdgcn_sched_barrier(0);
@@ -532,8 +525,16 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
         if (tid + bs * i >= chunks) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     if constexpr (NORM) {
-        lds_barrier();
         request_weight_tiles();
+        if (wave < 4) {
+            float part = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NSS; ++i)
+                if (tid + 256 * i < chunks) part = sum_squares4(part, vs[i]);  // chunks past the end would add +0
+            part = wave_sum_f32(part);
+            if (lane == 0) red_f[0][wave] = part;
+        }
+        lds_barrier();
         const float ss = f32_add(f32_add(f32_add(red_f[0][0], red_f[0][1]), red_f[0][2]), red_f[0][3]);
         const RowDivisor rdiv = make_row_divisor(rms_from_ss(ss, p.k, p.src.eps));
 #pragma unroll
