@@ -1117,6 +1117,8 @@ int bitnet_hip_decoder_graph_create(bitnet_hip_decoder *dec, size_t layer_begin,
     if (!g) return fail(BITNET_HIP_MEMORY_ERROR, "decoder_graph_create: out of host memory");
     g->dec = dec; g->layer_begin = layer_begin; g->layer_end = layer_end;
     hipStream_t cs = nullptr;
+    // a one-off: work queued on other streams that still writes x_in or reads x_out finishes first
+    BITNET_HIP_TRY(hipDeviceSynchronize());
     BITNET_HIP_TRY(hipStreamCreateWithFlags(&cs, hipStreamNonBlocking));
     // The step runs once for real first: it validates the arguments, and every one-time set-up of the launchers
     // (a kernel's LDS limit) happens outside the recording.

@@ -366,8 +366,8 @@ int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin
                                      const float *x_in, size_t m, float *x_out, float *q_last, float *k_last,
                                      void *stream);
 /* A decode step recorded once and replayed: the launches of bitnet_hip_decoder_decode_layers(dec, layer_begin, layer_end,
- * x_in, m, x_out, q_last, k_last) as a HIP graph.  create runs the step once on a stream of its own (x_out is written),
- * records it and returns when both are done; launch replays it on `stream`, reading x_in and writing x_out (and q_last,
+ * x_in, m, x_out, q_last, k_last) as a HIP graph.  create waits for the device to be idle, runs the step once on a
+ * stream of its own (x_out is written), records it and returns when both are done; launch replays it on `stream`, reading x_in and writing x_out (and q_last,
  * k_last) at the addresses given to create, with the locking and ordering of a decode call.  Weight, bias and norm
  * updates of the decoder's layers keep their device buffers, so a graph stays valid across them and reads the new
  * values; it must be destroyed before the decoder.
