@@ -174,6 +174,13 @@ def test_binding_validates_operands_before_any_pointer_reaches_a_kernel():
                 lambda: dec.decode(F((2, 16), torch.float64))):
         with pytest.raises(bh.BitLinearError):
             bad()
+    # the recorded step takes the same operands through the same checks
+    for bad in (lambda: dec.record(F((2, 15), f32)), lambda: dec.record(F((16,), f32)),
+                lambda: dec.record(F((2, 16), f32), out=F((3, 16), f32)), lambda: dec.record(F((2, 16), f32), layers=(1, 3)),
+                lambda: dec.record(F((2, 16), f32), layers=(1, 1)), lambda: dec.record(F((2, 16), torch.float64)),
+                lambda: dec.record(torch.zeros(2, 16))):
+        with pytest.raises(bh.BitLinearError):
+            bad()
 
 
 def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
