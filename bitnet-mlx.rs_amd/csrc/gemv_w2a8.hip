@@ -1037,7 +1037,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_lds_kernel(const int8_t *hot_a,
 // groups of a row-block group placed on the same XCD, from HBM once and from that XCD's L2 afterwards.
 // The copy is made by LDS-direct loads, all in flight at once, and the wavefront's k-tiles (kt = wave + 4u, at most NT of
 // them) are requested as one batch right behind it, so the two latencies overlap.  k % 256 == 0, activations 16-byte
-// aligned, m * k < 4 GiB, 16 * (k + 16) bytes of dynamic LDS.
+// aligned, m * k < 4 GiB, 16 * (k + 16) bytes of dynamic LDS rounded up to a whole KiB (the copy stores whole loads).
 template <int RB, int NT>
 __global__ __launch_bounds__(256) void gemv_mfma_tg_kernel(const int8_t *hot_a, int hot_k, int hot_m, int hot_kt_count, int hot_groups,
                                                            int hot_tgroups, GemvMfmaParams p)
@@ -1350,6 +1350,9 @@ int launch_mfma_rb(const GemvProj *projs, int nproj, const int8_t *a, const floa
     return BITNET_HIP_OK;
 }
 
+// Dynamic LDS of gemv_mfma_tg_kernel: 16 token rows of k + 16 bytes, rounded up to the 1 KiB loads that fill it.
+constexpr size_t tg_lds_bytes(size_t k) { return (16 * (k + 16) + 1023) / 1024 * 1024; }
+
 // 17 and more token rows, k a multiple of 256 up to 8192, aligned activations: token groups of 16 (gemv_mfma_tg_kernel)
 template <int RB>
 int launch_mfma_tg(const GemvProj *projs, int nproj, const int8_t *a, const float *a_scale, size_t m, size_t k, hipStream_t stream)
@@ -1369,15 +1372,19 @@ int launch_mfma_tg(const GemvProj *projs, int nproj, const int8_t *a, const floa
     if (end == 0) return BITNET_HIP_OK;
     const int tgroups = (int)((m + 15) / 16), total = end * tgroups;
     const unsigned grid = (unsigned)((total + 7) / 8 * 8);
-    const size_t lds = 16 * (k + 16);
+    // The copy fills LDS in whole loads of 1 KiB (64 lanes x 16 bytes); the last one runs past the 16 * (k + 16) bytes
+    // of token rows, so the allocation is rounded up to whole loads.
+    const size_t lds = tg_lds_bytes(k);
+    if ((16 * (k / 16 + 1) + 63) / 64 * 1024 > lds)
+        return fail(BITNET_HIP_KERNEL_ERROR, "gemv_mfma_tg: the activation copy would overrun its LDS allocation");
     if (p.kt_count <= 12) {
         static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mfma_tg_kernel<RB, 3>),
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 16 * (3072 + 16));
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)tg_lds_bytes(3072));
         BITNET_HIP_TRY(attr);
         hipLaunchKernelGGL((gemv_mfma_tg_kernel<RB, 3>), dim3(grid), dim3(256), lds, stream, p.a, p.k, p.m, p.kt_count, end, tgroups, p);
     } else {
         static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mfma_tg_kernel<RB, 8>),
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 16 * (8192 + 16));
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)tg_lds_bytes(8192));
         BITNET_HIP_TRY(attr);
         hipLaunchKernelGGL((gemv_mfma_tg_kernel<RB, 8>), dim3(grid), dim3(256), lds, stream, p.a, p.k, p.m, p.kt_count, end, tgroups, p);
     }

@@ -4,8 +4,8 @@ use std::env;
 use std::path::PathBuf;
 use std::process::Command;
 
-const KERNELS: [&str; 6] =
-    ["api.hip", "act_quant.hip", "weight_prep.hip", "gemv_w2a8.hip", "gemm_w2a8.hip"];
+const KERNELS: &[&str] =
+    &["api.hip", "act_quant.hip", "weight_prep.hip", "gemv_w2a8.hip", "gemm_w2a8.hip"];
 
 fn main() {
     println!("cargo:rerun-if-changed=build.rs");

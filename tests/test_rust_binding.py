@@ -48,8 +48,18 @@ def test_rust_extern_block_matches_header():
 def test_rust_build_script_compiles_the_same_sources_with_the_same_flags():
     build_rs = (FFI.parents[1] / "build.rs").read_text()
     makefile = (ROOT / "bitnet-mlx.rs_amd" / "Makefile").read_text()
-    for src in re.findall(r"csrc/([a-z0-9_]+\.hip)", makefile):
-        assert f'"{src}"' in build_rs, src
+    make_srcs = re.findall(r"csrc/([a-z0-9_]+\.hip)", re.search(r"^SRCS\s*=(.*)$", makefile, flags=re.M).group(1))
+    decl = re.search(r"const KERNELS:\s*([^=]+?)\s*=\s*&?\[(.*?)\];", build_rs, flags=re.S)
+    assert decl, "build.rs declares no KERNELS list"
+    listed = re.findall(r'"([a-z0-9_]+\.hip)"', decl.group(2))
+    assert listed == make_srcs  # the same sources in the same order as the Makefile's SRCS
+    fixed_len = re.fullmatch(r"\[&str;\s*(\d+)\]", decl.group(1))
+    if fixed_len:  # a fixed-size array type must state the number of elements it holds (a mismatch does not compile)
+        assert int(fixed_len.group(1)) == len(listed)
+    else:
+        assert decl.group(1) == "&[&str]"
+    for src in listed:
+        assert (ROOT / "bitnet-mlx.rs_amd" / "csrc" / src).is_file(), src
     for flag in ("--offload-arch=gfx950", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-packed-fp32-ops",
                  "-amdgpu-kernarg-preload-count=10"):
         assert flag in build_rs and flag.lstrip("-") in makefile.replace("$(ARCH)", "gfx950")
