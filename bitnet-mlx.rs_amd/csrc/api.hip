@@ -885,6 +885,8 @@ int bitnet_hip_bitlinear_matmul(bitnet_hip_bitlinear *layer, const int8_t *a, co
 // ---------------------------------------------------------------------------------------------------
 // Decoder projections
 // ---------------------------------------------------------------------------------------------------
+constexpr size_t DECODER_MAX_CHAINS = 8;
+
 struct bitnet_hip_decoder {
     size_t layers = 0, hidden = 0, ffn = 0, q_heads = 0, kv_heads = 0, head_dim = 0, max_tokens = 0;
     float eps = 1e-5f;
@@ -903,6 +905,16 @@ struct bitnet_hip_decoder {
     hipEvent_t done = nullptr;
     hipStream_t done_stream = nullptr;
     bool done_recorded = false;
+    // Token rows never interact on this path (CpuInferenceBackend::execute_batch fans independent inputs out over
+    // threads, bitnet-inference/src/engine/cpu_backend.rs:206-238).  A step of several rows is therefore split into up
+    // to DECODER_MAX_CHAINS groups of rows can be run as chains of launches side by side, each through all blocks on a
+    // stream of its own (its rows of the activation buffers are its own), forked from and joined to the caller's stream
+    // by events.  Off unless asked for (chains <= 1 = one chain): on the part measured the command processor starts one
+    // kernel per 2.2 us whatever the number of queues, so chains of these short kernels take turns instead of
+    // overlapping (8 tokens, 30 blocks: 957 us as one chain, 918 as two, 1355 as four, 2155 as eight).
+    size_t chains = 0;
+    hipStream_t side[DECODER_MAX_CHAINS - 1] = {};
+    hipEvent_t fork = nullptr, join[DECODER_MAX_CHAINS - 1] = {};
 
     ~bitnet_hip_decoder()
     {
@@ -911,6 +923,11 @@ struct bitnet_hip_decoder {
         for (void *b : bufs)
             if (b) (void)hipFree(b);
         if (done) (void)hipEventDestroy(done);
+        if (fork) (void)hipEventDestroy(fork);
+        for (hipEvent_t e : join)
+            if (e) (void)hipEventDestroy(e);
+        for (hipStream_t st : side)
+            if (st) (void)hipStreamDestroy(st);
     }
 };
 
@@ -968,11 +985,31 @@ int bitnet_hip_decoder_create(size_t layers, size_t hidden, size_t ffn, size_t q
         hipError_t e = hipEventCreateWithFlags(&d->done, hipEventDisableTiming);
         if (e != hipSuccess) rc = fail(BITNET_HIP_DEVICE_ERROR, "decoder_create: hipEventCreate failed: %s", hipGetErrorString(e));
     }
+    // streams (default priority) and events of the row-group chains, made here so that no decode call creates any
+    const size_t side_streams = (max_tokens < DECODER_MAX_CHAINS ? max_tokens : DECODER_MAX_CHAINS) - 1;
+    if (rc == BITNET_HIP_OK && side_streams > 0) {
+        hipError_t e = hipEventCreateWithFlags(&d->fork, hipEventDisableTiming);
+        for (size_t i = 0; i < side_streams && e == hipSuccess; ++i) {
+            e = hipStreamCreateWithFlags(&d->side[i], hipStreamNonBlocking);
+            if (e == hipSuccess) e = hipEventCreateWithFlags(&d->join[i], hipEventDisableTiming);
+        }
+        if (e != hipSuccess) rc = fail(BITNET_HIP_DEVICE_ERROR, "decoder_create: chain streams: %s", hipGetErrorString(e));
+    }
     if (rc != BITNET_HIP_OK) {
         delete d;
         return rc;
     }
     *dec = d;
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_decoder_set_chains(bitnet_hip_decoder *dec, size_t chains)
+{
+    if (!dec) return fail(BITNET_HIP_NULL_POINTER, "decoder_set_chains: dec is NULL");
+    if (chains > DECODER_MAX_CHAINS)
+        return fail(BITNET_HIP_INVALID_CONFIG, "decoder_set_chains: %zu chains, at most %zu", chains, DECODER_MAX_CHAINS);
+    std::lock_guard<std::mutex> one_decode(dec->decode_lock);
+    dec->chains = chains;
     return BITNET_HIP_OK;
 }
 
@@ -1042,30 +1079,62 @@ int bitnet_hip_decoder_decode_layers(bitnet_hip_decoder *dec, size_t layer_begin
     (void)hipStreamIsCapturing(s, &capturing);
     if (dec->done_recorded && dec->done_stream != s && capturing == hipStreamCaptureStatusNone)
         BITNET_HIP_TRY(hipStreamWaitEvent(s, dec->done, 0));  // the previous decode used these buffers on another stream
-    // one launch group: `count` projections reading the same (transformed) input
-    auto run = [&](bitnet_hip_bitlinear *const *layers, int count, const float *x, const float *x2, size_t ldx, int mode,
-                   const float *gamma, const float *res0, float *const *outs) {
-        if (rc != BITNET_HIP_OK) return;
-        const float *res[GEMV_MAX_PROJ] = {res0, nullptr, nullptr};
-        rc = run_projections(layers, count, x, x2, ldx, m, mode, group, dec->head_dim, gamma, dec->eps, dec->sum_order, res,
-                             outs, nullptr, dec->a8, dec->a_scale, dec->a_sum, false, s);
+    // One chain: rows [row0, row0 + rows) through blocks layer_begin .. layer_end-1 on stream cs, in its own rows of the
+    // decoder's activation buffers.
+    const size_t widest = H > F ? H : F;
+    auto run_chain = [&](size_t row0, size_t rows, hipStream_t cs) {
+        // one launch group: `count` projections reading the same (transformed) input
+        auto run = [&](bitnet_hip_bitlinear *const *layers, int count, const float *x, const float *x2, size_t ldx, int mode,
+                       const float *gamma, const float *res0, float *const *outs) {
+            if (rc != BITNET_HIP_OK) return;
+            const float *res[GEMV_MAX_PROJ] = {res0, nullptr, nullptr};
+            rc = run_projections(layers, count, x, x2, ldx, rows, mode, group, dec->head_dim, gamma, dec->eps, dec->sum_order,
+                                 res, outs, nullptr, dec->a8 + row0 * widest, dec->a_scale + row0, dec->a_sum + row0, false, cs);
+        };
+        float *qb = dec->qb + row0 * H, *kb = dec->kb + row0 * KV, *vb = dec->vb + row0 * KV, *x1 = dec->x1 + row0 * H;
+        float *gate = dec->gate + row0 * F, *up = dec->up + row0 * F, *ping = dec->ping + row0 * H;
+        float *xo = x_out + row0 * H;
+        const float *x = x_in + row0 * H;
+        for (size_t l = layer_begin; l < layer_end; ++l) {
+            bitnet_hip_bitlinear **P = &dec->proj[l * 7];
+            const float *g_attn = dec->gamma + (l * 2) * H, *g_ffn = g_attn + H;
+            const bool last = l + 1 == layer_end;
+            // hidden states alternate between x_out and the internal buffer so that the last block writes x_out
+            float *x2 = ((layer_end - 1 - l) % 2 == 0) ? xo : ping;
+            float *qkv_out[3] = {(last && q_last) ? q_last + row0 * H : qb, (last && k_last) ? k_last + row0 * KV : kb, vb};
+            run(&P[BITNET_HIP_PROJ_Q], 3, x, nullptr, H, BITNET_HIP_INPUT_PLAIN, g_attn, nullptr, qkv_out);
+            float *o_out[1] = {x1};
+            run(&P[BITNET_HIP_PROJ_O], 1, vb, nullptr, KV, BITNET_HIP_INPUT_GQA_BROADCAST, nullptr, x, o_out);
+            float *gu_out[2] = {gate, up};
+            run(&P[BITNET_HIP_PROJ_GATE], 2, x1, nullptr, H, BITNET_HIP_INPUT_PLAIN, g_ffn, nullptr, gu_out);
+            float *d_out[1] = {x2};
+            run(&P[BITNET_HIP_PROJ_DOWN], 1, gate, up, F, BITNET_HIP_INPUT_RELU2_MUL, nullptr, x1, d_out);
+            x = x2;
+        }
     };
-    const float *x = x_in;
-    for (size_t l = layer_begin; l < layer_end; ++l) {
-        bitnet_hip_bitlinear **P = &dec->proj[l * 7];
-        const float *g_attn = dec->gamma + (l * 2) * H, *g_ffn = g_attn + H;
-        const bool last = l + 1 == layer_end;
-        // hidden states alternate between x_out and the internal buffer so that the last block writes x_out
-        float *x2 = ((layer_end - 1 - l) % 2 == 0) ? x_out : dec->ping;
-        float *qkv_out[3] = {(last && q_last) ? q_last : dec->qb, (last && k_last) ? k_last : dec->kb, dec->vb};
-        run(&P[BITNET_HIP_PROJ_Q], 3, x, nullptr, H, BITNET_HIP_INPUT_PLAIN, g_attn, nullptr, qkv_out);
-        float *o_out[1] = {dec->x1};
-        run(&P[BITNET_HIP_PROJ_O], 1, dec->vb, nullptr, KV, BITNET_HIP_INPUT_GQA_BROADCAST, nullptr, x, o_out);
-        float *gu_out[2] = {dec->gate, dec->up};
-        run(&P[BITNET_HIP_PROJ_GATE], 2, dec->x1, nullptr, H, BITNET_HIP_INPUT_PLAIN, g_ffn, nullptr, gu_out);
-        float *d_out[1] = {x2};
-        run(&P[BITNET_HIP_PROJ_DOWN], 1, dec->gate, dec->up, F, BITNET_HIP_INPUT_RELU2_MUL, nullptr, dec->x1, d_out);
-        x = x2;
+    size_t chains = dec->chains ? dec->chains : 1;
+    if (chains > m) chains = m;
+    if (chains > dec->max_tokens) chains = dec->max_tokens;  // side streams exist for min(max_tokens, 8) chains
+    if (chains <= 1) {
+        run_chain(0, m, s);
+    } else {
+        // fork: the side streams start behind whatever the caller's stream holds; join: it continues behind them all.
+        // Recorded into the caller's graph when s is being captured (the events pull the side streams into the capture).
+        BITNET_HIP_TRY(hipEventRecord(dec->fork, s));
+        const size_t base = m / chains, extra = m % chains;
+        size_t row0 = base + (extra ? 1 : 0);
+        for (size_t c = 1; c < chains; ++c) BITNET_HIP_TRY(hipStreamWaitEvent(dec->side[c - 1], dec->fork, 0));
+        // every fork that was opened is joined again, also after a failed launch (an open fork would poison a capture)
+        run_chain(0, row0, s);
+        for (size_t c = 1; c < chains; ++c) {
+            const size_t rows = base + (c < extra ? 1 : 0);
+            run_chain(row0, rows, dec->side[c - 1]);
+            row0 += rows;
+            hipError_t e = hipEventRecord(dec->join[c - 1], dec->side[c - 1]);
+            if (e == hipSuccess) e = hipStreamWaitEvent(s, dec->join[c - 1], 0);
+            if (e != hipSuccess && rc == BITNET_HIP_OK)
+                rc = fail(BITNET_HIP_DEVICE_ERROR, "decoder_decode: joining a row-group chain: %s", hipGetErrorString(e));
+        }
     }
     if (rc == BITNET_HIP_OK && capturing == hipStreamCaptureStatusNone) {
         BITNET_HIP_TRY(hipEventRecord(dec->done, s));

@@ -43,7 +43,7 @@ namespace bitnet {
 namespace {
 
 constexpr int MODE_PREQUANT = -1;
-constexpr int GEMV_FUSED_MAX_ROWS = 6;   // tokens per fused quantiser + GEMV launch (measured: 2..6 gain, 8 loses)
+constexpr int GEMV_FUSED_MAX_ROWS = 8;   // tokens per fused quantiser + GEMV launch (a set of workgroups per token)
 constexpr int GEMV_FUSED_MAX_WGS = 512;  // and its workgroups over all tokens: one round on 256 compute units
 constexpr int FUSED_NCH = 7;  // 16-byte f32 chunks per thread kept in registers: K <= 7168
 
@@ -440,7 +440,7 @@ template <int MODE, bool NORM, int NCHB, int RBW>
 __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, const float *hot_x2, const float *hot_gamma, int hot_k, int hot_head_dim,
                                                            int hot_gqa_group, int hot_ldx, GemvParams p)
 {
-    // A launch has one to six tokens (input rows), each with its own workgroups.  Workgroup (x, y) of the grid works on
+    // A launch has one to eight tokens (input rows), each with its own workgroups.  Workgroup (x, y) of the grid works on
     // token x / 8 and on group 8y + x % 8 of row blocks: the workgroups of one group are neighbours in dispatch order and,
     // workgroups going to the XCDs in turn, run on the same XCD, so its L2 fetches their weight tiles once.
     // The leading scalar arguments repeat what the first loads need (input rows, RMSNorm weights, k): the file is
@@ -582,28 +582,33 @@ __global__ __launch_bounds__(1024) void gemv_fused16_kernel(const float *hot_x, 
     for (int i = 0; i < NCHB; ++i) {
         const int kt = wave + nw * i;
         if (kt < p.kt_count) {  // uniform over the wavefront
-            v4i_t acc[RBW];
+            // row blocks in batches of at most four: the accumulators of a batch are 16 registers
+            constexpr int RBB = RBW < 4 ? RBW : 4;
 #pragma unroll
-            for (int r = 0; r < RBW; ++r) acc[r] = (v4i_t){0, 0, 0, 0};
+            for (int r0 = 0; r0 < RBW; r0 += RBB) {
+                v4i_t acc[RBB];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                v4i_t af = (v4i_t){0, 0, 0, 0};
-                if (row0) af = *reinterpret_cast<const v4i_t *>(lds_a + kt * 16 + 4 * t + kq);
+                for (int r = 0; r < RBB; ++r) acc[r] = (v4i_t){0, 0, 0, 0};
 #pragma unroll
-                for (int r = 0; r < RBW; ++r) {
-                    const uint4 w4 = wt[r][i];
-                    const uint32_t wd = t == 0 ? w4.x : (t == 1 ? w4.y : (t == 2 ? w4.z : w4.w));
-                    v4i_t bf;
-                    bf[0] = (int)(wd & 0x03030303u);
-                    bf[1] = (int)((wd >> 2) & 0x03030303u);
-                    bf[2] = (int)((wd >> 4) & 0x03030303u);
-                    bf[3] = (int)((wd >> 6) & 0x03030303u);
-                    acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf, acc[r], 0, 0, 0);
+                for (int t = 0; t < 4; ++t) {
+                    v4i_t af = (v4i_t){0, 0, 0, 0};
+                    if (row0) af = *reinterpret_cast<const v4i_t *>(lds_a + kt * 16 + 4 * t + kq);
+#pragma unroll
+                    for (int r = 0; r < RBB; ++r) {
+                        const uint4 w4 = wt[r0 + r][i];
+                        const uint32_t wd = t == 0 ? w4.x : (t == 1 ? w4.y : (t == 2 ? w4.z : w4.w));
+                        v4i_t bf;
+                        bf[0] = (int)(wd & 0x03030303u);
+                        bf[1] = (int)((wd >> 2) & 0x03030303u);
+                        bf[2] = (int)((wd >> 4) & 0x03030303u);
+                        bf[3] = (int)((wd >> 6) & 0x03030303u);
+                        acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf, acc[r], 0, 0, 0);
+                    }
                 }
-            }
 #pragma unroll
-            for (int r = 0; r < RBW; ++r)
-                if (lane < TILE_ROWS) atomicAdd(&tot[r][lane], acc[r][0]);  // int32: any order gives the same sum
+                for (int r = 0; r < RBB; ++r)
+                    if (lane < TILE_ROWS) atomicAdd(&tot[r0 + r][lane], acc[r][0]);  // int32: any order gives the same sum
+            }
         }
     }
     lds_barrier();
@@ -1275,8 +1280,13 @@ int launch_fused16_mode(const GemvParams &p, hipStream_t stream)
         if (norm) hipLaunchKernelGGL((gemv_fused16_kernel<MODE, true, NCHB, RBW>), grid, block, lds, stream, BITNET_HOT_ARGS, p); \
         else hipLaunchKernelGGL((gemv_fused16_kernel<MODE, false, NCHB, RBW>), grid, block, lds, stream, BITNET_HOT_ARGS, p); \
     } while (0)
-    if (nchb == 1) BITNET_F16_LAUNCH(1);
-    else BITNET_F16_LAUNCH(2);
+    if (nchb == 1) {
+        BITNET_F16_LAUNCH(1);
+    } else if constexpr (RBW <= 8) {  // two k-tiles per wavefront: the tiles of 16 row blocks would not fit the registers
+        BITNET_F16_LAUNCH(2);
+    } else {
+        return fail(BITNET_HIP_UNSUPPORTED, "gemv_fused16: %d row blocks per workgroup with %d k-tiles", RBW, p.kt_count);
+    }
 #undef BITNET_F16_LAUNCH
 #undef BITNET_HOT_ARGS
     BITNET_HIP_CHECK_LAUNCH("gemv_fused16_kernel");
@@ -1455,6 +1465,26 @@ int launch_gemv_tiled(const GemvProj *projs, int nproj, const int8_t *a, const f
     return launch_mode<MODE_PREQUANT>(p, stream);
 }
 
+// Row blocks per workgroup of gemv_fused16_kernel.  Every workgroup quantises its token's input row for itself: that
+// arithmetic is repeated by every workgroup of the launch, and two workgroups on one compute unit take turns on its
+// SIMDs, so the launch is sized to about one workgroup per compute unit where the registers allow (a wavefront holds
+// the tiles of all its row blocks: 16 of them for rows of up to 16 k-tiles, 8 above).
+int fused16_row_blocks_per_workgroup(size_t m, size_t k, size_t blocks)
+{
+    if (m == 1) {
+        // one token, gate alone, 432 row blocks: 4.50 us with one row block per workgroup, 3.82 us with two
+        if (blocks > 512 && k <= 4096) return 4;
+        return (blocks > 256 && k <= 4096) ? 2 : 1;
+    }
+    // Several tokens, each with its own workgroups: the fewest row blocks per workgroup that keep the launch within one
+    // workgroup per compute unit, at most 8 (16 lose: the dot products of 16 row blocks are a wavefront's serial work).
+    // 30-block step at 2 / 3 / 4 / 6 / 8 tokens: 578 / 662 / 713 / 778 / 901 us; with a limit of 512 workgroups and at
+    // most 4 row blocks each 646 / 733 / 779 / 1023 / 1150 us.
+    int rbw = 1;
+    while (rbw < 8 && (blocks + rbw - 1) / rbw * m > 256) rbw *= 2;
+    return rbw;
+}
+
 bool gemv_fused_supported(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
                           size_t head_dim, const float *gamma, int sum_order, size_t blocks)
 {
@@ -1465,7 +1495,7 @@ bool gemv_fused_supported(const float *x, const float *x2, size_t ldx, size_t m,
     if (m == 0 || m > (size_t)GEMV_FUSED_MAX_ROWS) return false;
     if (m > 1) {
         if (!((gamma == nullptr || sum_order == BITNET_HIP_SUM_BLOCK256) && k <= 8192 && ldx < ((size_t)1 << 31))) return false;
-        const size_t rbw = blocks * m > 512 ? 4 : 1;
+        const size_t rbw = (size_t)fused16_row_blocks_per_workgroup(m, k, blocks);
         if ((blocks + rbw - 1) / rbw * m > (size_t)GEMV_FUSED_MAX_WGS) return false;
     }
     if (k % 4 != 0 || ldx % 4 != 0 || k > (size_t)FUSED_NCH * 1024) return false;
@@ -1488,8 +1518,7 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
         // row blocks per workgroup: one round of workgroups on the 256 compute units where the row is short enough for
         // a wavefront to hold the tiles of several row blocks (one token, gate alone, 432 row blocks: 4.50 us with one
         // row block per workgroup, 3.82 us with two)
-        int rbw16 = ((m == 1 ? (blocks > 512 && k <= 4096) : blocks * m > 512)) ? 4 : 1;
-        if (m == 1 && rbw16 == 1 && blocks > 256 && k <= 4096) rbw16 = 2;
+        const int rbw16 = fused16_row_blocks_per_workgroup(m, k, blocks);
         GemvParams p = {};
         if (fill_projs(p, projs, nproj, 0, k, rbw16) == 0) return BITNET_HIP_OK;
         p.m = (int)m;
@@ -1497,25 +1526,20 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
         p.src.head_dim = (int)(head_dim ? head_dim : 1); p.src.gqa_group = (int)(gqa_group ? gqa_group : 1);
         p.src.sum_order = sum_order; p.src.eps = eps;
         p.q_out = q_out; p.a_scale_out = a_scale_out; p.a_sum_out = a_sum_out;
-        if (rbw16 == 2) {
-            switch (input_mode) {
-                case BITNET_HIP_INPUT_PLAIN: return launch_fused16_mode<BITNET_HIP_INPUT_PLAIN, 2>(p, stream);
-                case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused16_mode<BITNET_HIP_INPUT_RELU2_MUL, 2>(p, stream);
-                default: return launch_fused16_mode<BITNET_HIP_INPUT_GQA_BROADCAST, 2>(p, stream);
-            }
+#define BITNET_F16_MODES(RBW) \
+    switch (input_mode) { \
+        case BITNET_HIP_INPUT_PLAIN: return launch_fused16_mode<BITNET_HIP_INPUT_PLAIN, RBW>(p, stream); \
+        case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused16_mode<BITNET_HIP_INPUT_RELU2_MUL, RBW>(p, stream); \
+        default: return launch_fused16_mode<BITNET_HIP_INPUT_GQA_BROADCAST, RBW>(p, stream); \
+    }
+        switch (rbw16) {
+            case 16: BITNET_F16_MODES(16)
+            case 8: BITNET_F16_MODES(8)
+            case 4: BITNET_F16_MODES(4)
+            case 2: BITNET_F16_MODES(2)
+            default: BITNET_F16_MODES(1)
         }
-        if (rbw16 == 4) {
-            switch (input_mode) {
-                case BITNET_HIP_INPUT_PLAIN: return launch_fused16_mode<BITNET_HIP_INPUT_PLAIN, 4>(p, stream);
-                case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused16_mode<BITNET_HIP_INPUT_RELU2_MUL, 4>(p, stream);
-                default: return launch_fused16_mode<BITNET_HIP_INPUT_GQA_BROADCAST, 4>(p, stream);
-            }
-        }
-        switch (input_mode) {
-            case BITNET_HIP_INPUT_PLAIN: return launch_fused16_mode<BITNET_HIP_INPUT_PLAIN, 1>(p, stream);
-            case BITNET_HIP_INPUT_RELU2_MUL: return launch_fused16_mode<BITNET_HIP_INPUT_RELU2_MUL, 1>(p, stream);
-            default: return launch_fused16_mode<BITNET_HIP_INPUT_GQA_BROADCAST, 1>(p, stream);
-        }
+#undef BITNET_F16_MODES
     }
     const int rbw = (blocks > 512 && k <= 3 * 1024) ? 2 : 1;
     GemvParams p = {};

@@ -464,6 +464,13 @@ public:
         if (rc != BITNET_HIP_OK) return last_error(rc);
         return Unit{};
     }
+    // row groups a step of several token rows is split into, each a chain of launches on its own stream (0 and 1 = one chain, the default)
+    Result<Unit> set_chains(size_t chains)
+    {
+        int rc = bitnet_hip_decoder_set_chains(handle_, chains);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        return Unit{};
+    }
     Result<DeviceTensor> decode(const DeviceTensor &x) const
     {
         auto out = DeviceTensor::zeros(x.dims());

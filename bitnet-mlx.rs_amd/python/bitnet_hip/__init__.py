@@ -125,6 +125,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_decoder_destroy": (None, [vp]),
         "bitnet_hip_decoder_projection": (i32, [vp, sz, i32, C.POINTER(vp)]),
         "bitnet_hip_decoder_set_norm": (i32, [vp, sz, i32, vp, i32, vp]),
+        "bitnet_hip_decoder_set_chains": (i32, [vp, sz]),
         "bitnet_hip_decoder_weight_bytes": (sz, [vp]),
         "bitnet_hip_decoder_decode": (i32, [vp, vp, sz, vp, vp, vp, vp]),
         "bitnet_hip_decoder_graph_create": (i32, [vp, sz, sz, vp, sz, vp, vp, vp, C.POINTER(vp)]),
@@ -839,6 +840,11 @@ class DecoderProjections:
             raise BitLinearError(SHAPE_MISMATCH, "norm weight", [self.hidden], list(gamma.shape))
         _check(load_library().bitnet_hip_decoder_set_norm(self._h, layer, which, _ptr(gamma), int(gamma.is_cuda),
                                                           _stream(stream)))
+
+    def set_chains(self, chains: int):
+        """Row groups a decode step of several token rows is split into (each a chain of launches on its own stream);
+        0 and 1 keep all rows in one chain (the default, and the faster form on the device measured)."""
+        _check(load_library().bitnet_hip_decoder_set_chains(self._h, int(chains)))
 
     def weight_bytes(self) -> int:
         return load_library().bitnet_hip_decoder_weight_bytes(self._h)

@@ -135,6 +135,7 @@ extern "C" {
                                          out: *mut *mut bitnet_hip_bitlinear) -> c_int;
     pub fn bitnet_hip_decoder_set_norm(dec: *mut bitnet_hip_decoder, layer: usize, which: c_int, gamma: *const f32,
                                        on_device: c_int, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_decoder_set_chains(dec: *mut bitnet_hip_decoder, chains: usize) -> c_int;
     pub fn bitnet_hip_decoder_weight_bytes(dec: *const bitnet_hip_decoder) -> usize;
     pub fn bitnet_hip_decoder_decode(dec: *mut bitnet_hip_decoder, x_in: *const f32, m: usize, x_out: *mut f32,
                                      q_last: *mut f32, k_last: *mut f32, stream: *mut c_void) -> c_int;

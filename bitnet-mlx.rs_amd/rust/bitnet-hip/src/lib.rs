@@ -411,6 +411,11 @@ mod imp {
             check(unsafe { ffi::bitnet_hip_decoder_projection(self.handle, layer, proj, &mut bl) })?;
             check(unsafe { ffi::bitnet_hip_bitlinear_set_weights_packed(bl, packed.as_ptr(), packed.len(), w_scale, 0, ptr::null_mut()) })
         }
+        /// Row groups a step of several token rows is split into, each a chain of launches on its own stream
+        /// (0 and 1 = one chain, the default).
+        pub fn set_chains(&self, chains: usize) -> HipResult<()> {
+            check(unsafe { ffi::bitnet_hip_decoder_set_chains(self.handle, chains) })
+        }
         pub fn set_norm(&self, layer: usize, which: c_int, gamma: &[f32]) -> HipResult<()> {
             if gamma.len() != self.hidden {
                 return Err(HipError::ShapeMismatch { expected: vec![self.hidden], actual: vec![gamma.len()] });

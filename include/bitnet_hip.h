@@ -353,6 +353,14 @@ int bitnet_hip_decoder_projection(bitnet_hip_decoder *dec, size_t layer, int pro
 /* RMSNorm weights of a block: which = 0 (before attention) or 1 (before the FFN); [hidden] f32. */
 int bitnet_hip_decoder_set_norm(bitnet_hip_decoder *dec, size_t layer, int which, const float *gamma,
                                 int on_device, void *stream);
+/* Row groups of a decode step.  Token rows never interact on this path (the reference fans independent inputs out
+ * over threads, bitnet-inference/src/engine/cpu_backend.rs:206-238), so a step of m > 1 rows is run as `chains` groups
+ * of consecutive rows, each a dependent chain of launches through all blocks on a stream of the decoder's own, forked
+ * from and joined to the caller's stream by events (also inside a recorded step): the chains' launches overlap, the
+ * results are those of the single chain bit for bit.  chains = 0 (the default) and 1 keep every row in one chain on
+ * the caller's stream, which is the faster form on the device measured (kernels this short are started one at a time
+ * whatever the number of queues); at most 8. */
+int bitnet_hip_decoder_set_chains(bitnet_hip_decoder *dec, size_t chains);
 /* Packed-weight bytes one decode step streams (sum of n*k/4 over all projections). */
 size_t bitnet_hip_decoder_weight_bytes(const bitnet_hip_decoder *dec);
 /* One decode step: x_in [m, hidden] -> x_out [m, hidden] through all blocks.  A decoder owns one set of activation

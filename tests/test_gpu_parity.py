@@ -941,7 +941,7 @@ def oracle_stack(ref, x, hidden, ffn, qh, kvh, hd, eps=1e-5):
     return x, q, k
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_decoder_layer_config2_bit_exact(m):
     """BASELINE config 2: one decoder layer's seven projections at BitNet-2B shapes."""
     rng = np.random.default_rng(0)
@@ -1105,6 +1105,46 @@ def test_decoder_recorded_step_replays_match_the_oracle(dims, layers, m):
     x_ref = oracle_stack(ref, host(x), *dims)[0]
     graph.replay()
     assert np.array_equal(host(graph.out), x_ref)
+
+
+@pytest.mark.parametrize("dims,layers,m,chains", [((2560, 6912, 20, 5, 128), 2, 8, 2), ((2560, 6912, 20, 5, 128), 2, 8, 4),
+                                                  ((2560, 6912, 20, 5, 128), 2, 5, 8), ((256, 512, 4, 2, 64), 3, 3, 2),
+                                                  ((1024, 2816, 8, 8, 128), 3, 16, 3)])
+def test_decoder_row_group_chains_match_the_oracle(dims, layers, m, chains):
+    """bitnet_hip_decoder_set_chains: a step of several token rows run as groups of rows side by side, each group a chain
+    of launches on a stream of the decoder's own.  Eager calls, a recorded step replayed several times (with eager work
+    and host synchronisations between the replays), a sub-range in place and the last block's q / k equal the oracle's
+    chain bit for bit; more chains than rows are cut down to one row each; back to one chain afterwards."""
+    rng = np.random.default_rng(31 * layers + 7 * m + chains + dims[0])
+    dec, ref = build_decoder_packed(rng, layers, *dims, max_tokens=m)
+    dec.set_chains(chains)
+    xs = synth_activations(rng, m, dims[0])
+    x_ref, q_ref, k_ref = oracle_stack(ref, xs, *dims)
+    for _ in range(2):
+        out, q, k = dec.decode(dev(xs), want_qk=True)
+        assert np.array_equal(host(out), x_ref)
+        assert np.array_equal(host(q), q_ref) and np.array_equal(host(k), k_ref)
+    x = dev(xs)
+    graph = dec.record(x, want_qk=True)
+    for round_ in range(3):
+        fresh = synth_activations(rng, m, dims[0])
+        want, q_want, k_want = oracle_stack(ref, fresh, *dims)
+        x.copy_(dev(fresh))
+        graph.out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(graph.out), want), f"replay {round_}"
+        assert np.array_equal(host(graph.q), q_want) and np.array_equal(host(graph.k), k_want)
+        assert np.array_equal(host(dec.decode(dev(fresh))), want)  # eager work on the same decoder between the replays
+    start = oracle_stack(ref[:1], xs, *dims)[0]
+    buf = dev(start.copy())
+    dec.decode(buf, out=buf, layers=(1, layers))
+    assert np.array_equal(host(buf), x_ref)
+    dec.set_chains(1)
+    assert np.array_equal(host(dec.decode(dev(xs))), x_ref)
+    with pytest.raises(bh.BitLinearError) as ei:
+        dec.set_chains(9)
+    assert ei.value.kind == "InvalidConfig"
 
 
 def test_decoder_recorded_step_argument_errors():
