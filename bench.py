@@ -122,32 +122,43 @@ def gemv_only(bh, torch, dec, gen, reps):
             "bytes_per_launch": round(total_bytes / launches), "gbs": round(total_bytes / (ms * 1e-3) / 1e9, 1)}
 
 
+PREFILL_LOOPS, PREFILL_LAUNCHES = 7, 50  # the prefill GEMM is timed as the median of 7 loops of 50 back-to-back launches
+
+
+def median_loop_ms(torch, fn, launches, loops):
+    """Milliseconds per launch: the median over `loops` event-timed loops of `launches` back-to-back calls of fn."""
+    times = sorted(time_events(torch, lambda: [fn() for _ in range(launches)]) / launches for _ in range(loops))
+    return times[len(times) // 2], times
+
+
 def prefill_rates(bh, torch, dec, gen, reps):
+    """configs[3]: the M = 2048 prefill GEMM at the two FFN shapes, on the configuration's own operands: f32 rows ~ N(0,1)
+    quantised per token by the library's quantiser (int8, a_scale, a_sum), ternary weights from N(0, 0.02)."""
     m = 2048
     res = {}
+    launches, loops = max(reps, 1), (PREFILL_LOOPS if reps >= PREFILL_LAUNCHES else 3)
     for name, p in (("2048x2560x6912", 4), ("2048x6912x2560", 6)):
         n, k = dec.proj_shape(p)
         bl = dec.projection(0, p)
-        a = torch.randint(-127, 128, (m, k), generator=gen, device="cuda", dtype=torch.int8)
-        a_scale = torch.ones((m,), device="cuda", dtype=torch.float32)
-        a_sum = a.to(torch.int32).sum(dim=1).to(torch.int32).contiguous()  # what the activation quantiser emits
+        x = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32)
+        a, a_scale, a_sum, _ = bh.quantize_activations_i8(x, want_sum=True)
         out = torch.empty((m, n), device="cuda", dtype=torch.float32)
         bl.matmul_quantized(a, a_scale, out=out, a_sum=a_sum)
-        ms = min(time_events(torch, lambda: [bl.matmul_quantized(a, a_scale, out=out, a_sum=a_sum) for _ in range(reps)])
-                 for _ in range(3)) / reps  # best of three loops of `reps` back-to-back launches
+        ms, all_ms = median_loop_ms(torch, lambda: bl.matmul_quantized(a, a_scale, out=out, a_sum=a_sum), launches, loops)
         tops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
-        res[name] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+        res[name] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4),
+                     "timed": f"median of {loops} loops of {launches} launches, operands of configs[3] (quantised N(0,1) rows)",
+                     "loops_ms": [round(t, 4) for t in all_ms]}
         # the whole BitLinear forward on f32 activations (absmax int8 quantiser + GEMM + scale epilogue), for reference
-        x = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32)
         bl.forward(x)
-        fwd_ms = min(time_events(torch, lambda: [bl.forward(x) for _ in range(reps)]) for _ in range(3)) / reps
+        fwd_ms, _ = median_loop_ms(torch, lambda: bl.forward(x), min(launches, 20), 3)
         res[name]["forward_f32_in_ms"] = round(fwd_ms, 4)
         # calibration only: the vendor library's int8 GEMM (torch._int_mm -> hipBLASLt) at the same shape, on weights
         # expanded to one int8 per value and without the scale epilogue (int32 output); not part of the measured path
         try:
             w8 = torch.randint(-1, 2, (n, k), generator=gen, device="cuda", dtype=torch.int8)
             torch._int_mm(a, w8.t())
-            lib_ms = min(time_events(torch, lambda: [torch._int_mm(a, w8.t()) for _ in range(reps)]) for _ in range(3)) / reps
+            lib_ms, _ = median_loop_ms(torch, lambda: torch._int_mm(a, w8.t()), min(launches, 20), 3)
             res[name]["vendor_int8_gemm_ms"] = round(lib_ms, 4)
             res[name]["vendor_int8_gemm_tops"] = round(2.0 * m * n * k / (lib_ms * 1e-3) / 1e12, 1)
             del w8
@@ -160,7 +171,7 @@ def prefill_rates(bh, torch, dec, gen, reps):
     for name, projs in (("q_k_v_2048x3840x2560", (0, 1, 2)), ("gate_up_2048x13824x2560", (4, 5))):
         layers = [dec.projection(0, p) for p in projs]
         bh.forward_multi(layers, x)
-        ms = min(time_events(torch, lambda: [bh.forward_multi(layers, x) for _ in range(reps)]) for _ in range(3)) / reps
+        ms, _ = median_loop_ms(torch, lambda: bh.forward_multi(layers, x), min(launches, 20), 3)
         ops = 2.0 * m * HIDDEN * sum(dec.proj_shape(p)[0] for p in projs)
         res[name] = {"forward_f32_in_ms": round(ms, 4), "tops_incl_quantiser": round(ops / (ms * 1e-3) / 1e12, 1)}
     # what the matrix unit of this device sustains when it does nothing but v_mfma_i32_16x16x64_i8 from registers: the
@@ -226,6 +237,30 @@ def stack_latency(bh, torch, dec, gen, reps=20):
             out[f"{name}_m{m}"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1),
                                    "timed": how}
     return out
+
+
+def launch_floor(bh, torch, step_us):
+    """What a chain of 120 dependent launches costs on this device when the kernels do nothing, and when they only read the
+    bytes the launches of a token step read (q+k+v, o, gate+up, down of 30 layers: the same 521 MB, distinct memory every
+    launch): recorded as HIP graphs and replayed like the measured step, in this process.  The measured step cannot go
+    below the second figure; the gap between the two is what reading the bytes adds to a launch."""
+    per_launch = [(2560 * 2560 + 2 * 640 * 2560) // 4, 2560 * 2560 // 4, 2 * 6912 * 2560 // 4, 6912 * 2560 // 4]
+    assert sum(per_launch) == LAYER_BYTES
+    buf = torch.randint(0, 256, (STEP_BYTES,), device="cuda", dtype=torch.uint8)
+    empty = sorted(bh.measure_launch_chain(LAUNCHES_PER_STEP, replays=20) for _ in range(5))[2]
+    reads = sorted(bh.measure_launch_chain(LAUNCHES_PER_STEP, replays=20, buf=buf, bytes_per_launch=per_launch) for _ in range(5))[2]
+    one = sorted(bh.measure_launch_chain(1, replays=20, buf=buf, bytes_per_launch=[STEP_BYTES]) for _ in range(5))[2]
+    del buf
+    return {"launches": LAUNCHES_PER_STEP, "bytes": STEP_BYTES,
+            "empty_kernels_us_per_step": round(empty, 1), "empty_kernel_us_per_launch": round(empty / LAUNCHES_PER_STEP, 3),
+            "read_only_kernels_us_per_step": round(reads, 1), "read_only_kernel_us_per_launch": round(reads / LAUNCHES_PER_STEP, 3),
+            "read_only_frac_hbm_peak": round(STEP_BYTES / (reads * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "one_launch_reading_all_bytes_us": round(one, 1),
+            "one_launch_frac_hbm_peak": round(STEP_BYTES / (one * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "measured_step_us": round(step_us, 1), "measured_over_read_only_floor": round(step_us / reads, 3),
+            "how": "bitnet_hip_measure_launch_chain: a recorded chain of 120 dependent launches (kernels that do nothing / "
+                   "kernels that only read the step's packed-weight bytes, 3.7 + 1.6 + 8.8 + 4.4 MB per layer), median of 5 "
+                   "measurements of 20 replays each"}
 
 
 def sequential_order_decode(bh, torch, dec, gen, reps=20):
@@ -476,9 +511,25 @@ def main():
     }
     line["roofline"] = decode_roofline(event_ms, args.steps)
     if not args.no_extras:
+        # Both halves of the metric and the floors they are judged against live under "roofline": the decode GEMV chain
+        # above, the prefill GEMM at the two shapes of configs[3], the decode GEMV where a launch is large enough to be
+        # bound by bandwidth, and the cost of 120 dependent launches on this device.
+        line["roofline"]["launch_floor"] = launch_floor(bh, torch, event_ms * 1e3 / args.steps)
         line["gemv_only"] = gemv_only(bh, torch, dec, gen, reps=5)
-        line["prefill"] = prefill_rates(bh, torch, dec, gen, reps=5)
+        line["prefill"] = prefill_rates(bh, torch, dec, gen, reps=PREFILL_LAUNCHES)
+        line["roofline"]["prefill"] = {
+            name: {"us": round(line["prefill"][name]["ms"] * 1e3, 2), "tops": line["prefill"][name]["tops"],
+                   "frac": line["prefill"][name]["frac_int8_mfma_peak"]}
+            for name in ("2048x2560x6912", "2048x6912x2560")}
+        line["roofline"]["prefill"].update({
+            "bound": "mfma", "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "ops_per_launch": 2 * 2048 * 2560 * 6912,
+            "mfma_loop_ceiling_tops": line["prefill"]["mfma_loop_ceiling"]["tops_random_operands"],
+            "how": line["prefill"]["2048x2560x6912"]["timed"]})
         line["other_configs"] = stack_latency(bh, torch, dec, gen)
+        large = line["other_configs"]["gemv_32768x16384_m1"]
+        line["roofline"]["large_gemv_frac"] = large["frac_hbm_peak"]
+        line["roofline"]["large_gemv"] = {"shape": "32768x16384, one token", "us": large["us"], "gbs": large["gbs_packed_weights"],
+                                          "frac": large["frac_hbm_peak"], "bytes_per_launch": 32768 * 16384 // 4}
         line["other_configs"]["decode_layer_b1_sum_order_sequential"] = sequential_order_decode(bh, torch, dec, gen)
         line["other_configs"]["decode_b1_eager_launches"] = eager_decode(torch, dec, x)
         if not args.no_cpu_baseline:

@@ -89,6 +89,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_init": (i32, [i32]),
         "bitnet_hip_device_info": (i32, [C.c_char_p, sz, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz)]),
         "bitnet_hip_measure_mfma_i8_rate": (i32, [i32, C.POINTER(C.c_double), vp]),
+        "bitnet_hip_measure_launch_chain": (i32, [vp, C.POINTER(sz), sz, sz, sz, C.POINTER(C.c_double), vp]),
         "bitnet_hip_quantize_activations_i8": (i32, [vp, vp, sz, sz, sz, i32, sz, sz, vp, f32, i32, vp, vp, vp, vp, vp]),
         "bitnet_hip_absmax_quantize_activations": (i32, [vp, sz, i32, vp, vp, vp]),
         "bitnet_hip_lookup_compute": (i32, [i32, vp, sz, vp, sz, vp, sz, vp]),
@@ -234,6 +235,29 @@ def measure_mfma_i8_rate(random_operands: bool = True, stream=None) -> float:
     tops = C.c_double(0.0)
     _check(load_library().bitnet_hip_measure_mfma_i8_rate(1 if random_operands else 0, C.byref(tops), _stream(stream)))
     return tops.value
+
+
+def measure_launch_chain(launches: int, replays: int = 20, buf: Optional[torch.Tensor] = None,
+                         bytes_per_launch: Optional[Sequence[int]] = None, stream=None) -> float:
+    """Microseconds per replay of a recorded chain of `launches` dependent kernel launches on the current device: kernels
+    that do nothing (buf None), or kernels that only read bytes_per_launch[i % len] bytes of buf each, one region after
+    the other (the floor of a decode step with that many launches and those bytes)."""
+    us = C.c_double(0.0)
+    if buf is None:
+        _check(load_library().bitnet_hip_measure_launch_chain(None, None, 0, launches, replays, C.byref(us), _stream(stream)))
+        return us.value
+    if not buf.is_cuda or not buf.is_contiguous():
+        raise BitLinearError(INVALID_CONFIG, "measure_launch_chain: buf must be a contiguous device tensor")
+    sizes = [int(b) for b in (bytes_per_launch or [])]
+    if not sizes or any(b <= 0 or b % 16 for b in sizes):
+        raise BitLinearError(INVALID_CONFIG, "measure_launch_chain: bytes_per_launch must be positive multiples of 16")
+    total = sum(sizes[i % len(sizes)] for i in range(launches))
+    if total > buf.numel() * buf.element_size():
+        raise BitLinearError(SHAPE_MISMATCH, "measure_launch_chain buffer", [total], [buf.numel() * buf.element_size()])
+    arr = (C.c_size_t * len(sizes))(*sizes)
+    _check(load_library().bitnet_hip_measure_launch_chain(_ptr(buf), arr, len(sizes), launches, replays, C.byref(us),
+                                                          _stream(stream)))
+    return us.value
 
 
 # ---- raw operators ------------------------------------------------------------------------------

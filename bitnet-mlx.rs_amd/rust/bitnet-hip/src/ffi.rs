@@ -59,6 +59,9 @@ extern "C" {
     pub fn bitnet_hip_device_info(arch_name: *mut c_char, arch_name_len: usize, compute_units: *mut c_int,
                                   clock_mhz: *mut c_int, total_mem_bytes: *mut usize) -> c_int;
     pub fn bitnet_hip_measure_mfma_i8_rate(random_operands: c_int, tera_ops_per_second: *mut f64, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_measure_launch_chain(buf: *const c_void, bytes_per_launch: *const usize, pattern_len: usize,
+                                           launches: usize, replays: usize, us_per_replay: *mut f64,
+                                           stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_quantize_activations_i8(x: *const f32, x2: *const f32, ldx: usize, m: usize, k: usize,
                                               input_mode: c_int, gqa_group: usize, head_dim: usize, gamma: *const f32,
                                               eps: f32, sum_order: c_int, q: *mut i8, a_scale: *mut f32,

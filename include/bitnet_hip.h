@@ -97,6 +97,16 @@ int bitnet_hip_device_info(char *arch_name, size_t arch_name_len, int *compute_u
  * (tera_ops_per_second is a HOST pointer).  No counterpart in the reference; bench.py reports it beside the
  * prefill rates. */
 int bitnet_hip_measure_mfma_i8_rate(int random_operands, double *tera_ops_per_second, void *stream);
+/* Diagnostic: microseconds one replay of a recorded chain of `launches` dependent kernel launches takes on the current
+ * device (each launch starts when the one before it has finished, as the 120 launches of a batch-1 token step do), the
+ * floor a decode step of that many launches cannot go below.  buf == NULL: kernels that do nothing.  Otherwise launch i
+ * only reads bytes_per_launch[i % pattern_len] bytes (multiples of 16) of buf, each launch the bytes behind those of
+ * the launch before it (buf, 16-byte aligned DEVICE memory, holds at least the sum over all launches), with the
+ * non-temporal loads the decode GEMV uses for its weight tiles.  The chain is replayed twice untimed, then `replays`
+ * times between two events on `stream`; us_per_replay is a HOST pointer; allocates a few hundred bytes and waits for
+ * the result.  No counterpart in the reference; bench.py reports both floors beside the measured token step. */
+int bitnet_hip_measure_launch_chain(const void *buf, const size_t *bytes_per_launch, size_t pattern_len,
+                                    size_t launches, size_t replays, double *us_per_replay, void *stream);
 
 /* ---- activation side -------------------------------------------------------------------------- */
 
