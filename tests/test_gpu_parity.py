@@ -449,9 +449,11 @@ def test_small_prefill_launches_bit_exact(m, n, k):
 @pytest.mark.parametrize("n,k", [(6912, 2560), (2560, 6912)])
 @pytest.mark.parametrize("with_sum", [True, False], ids=["lds_direct_kernel", "register_staged_kernel"])
 def test_prefill_gemm_full_size(n, k, with_sum):
-    """M = 2048 at the two prefill shapes: sampled rows bit-exact against the oracle, whole result through
-    order-free identities (column sums of acc against a one-row contraction of the summed activations).
-    Supplying the activation row sums selects the LDS-direct kernel, omitting them the register-staged one."""
+    """M = 2048 at the two prefill shapes (BASELINE config 4): every one of the 2048 x N accumulators against an f64 BLAS
+    product of the unpacked operands (|acc| <= 127 K < 2^24, so every partial sum of the f64 product is an exact
+    integer whatever the library's order), sampled rows also against the oracle's own loop, the f32 output of the whole
+    matrix against the oracle's epilogue.  Supplying the activation row sums selects the LDS-direct kernel, omitting
+    them the register-staged one."""
     m = 2048
     rng = np.random.default_rng(n)
     packed, ws, a, a_scale = make_problem(rng, m, n, k, outliers=False)
@@ -463,9 +465,10 @@ def test_prefill_gemm_full_size(n, k, with_sum):
     acc_ref = orc.gemm_w2a8(packed, a[rows], n)
     assert np.array_equal(acc_h[rows], acc_ref)
     assert np.array_equal(out_h[rows], orc.epilogue(acc_ref, ws, a_scale[rows]))
-    # sum over tokens of acc[t, n] == sum_k (sum_t a[t, k]) * w[n, k]
-    w = orc.unpack_2bit(packed, n * k).reshape(n, k).astype(np.int64)
-    assert np.array_equal(acc_h.astype(np.int64).sum(axis=0), w @ a.astype(np.int64).sum(axis=0))
+    w = orc.unpack_2bit(packed, n * k).reshape(n, k)
+    full = a.astype(np.float64) @ w.astype(np.float64).T  # exact: integers below 2^53 throughout
+    assert np.array_equal(full[rows], acc_ref.astype(np.float64))  # the f64 product agrees with the oracle's loop
+    assert np.array_equal(acc_h.astype(np.float64), full), "an accumulator of the full matrix differs"
     assert np.array_equal(out_h, orc.epilogue(acc_h, ws, a_scale))
 
 
