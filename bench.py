@@ -184,6 +184,42 @@ def prefill_rates(bh, torch, dec, gen, reps):
     return res
 
 
+def large_gemv_pair(bh, torch, gen, loops=5):
+    """The decode GEMV where a launch is large enough to be bound by bandwidth rather than by launch latency: 32768 x 16384
+    ternary weights, int8 activations already quantised, one token; on the 2-bit streaming layout (128 MiB per matrix)
+    and on base-3 bytes (five weights per byte, 102 MiB: 20 % fewer bytes, every byte through a table in LDS).  Four
+    matrices in rotation each, more than the last-level cache holds."""
+    out = {}
+    n, k = 32768, 16384
+    layers = [bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), f"large{i}") for i in range(4)]  # 512 MiB > cache
+    packed = torch.randint(0, 256, (n * k // 4,), generator=gen, device="cuda", dtype=torch.uint8)
+    for bl in layers:
+        bl.set_quantized_weights(packed, 0.02)
+    a = torch.randint(-127, 128, (1, k), generator=gen, device="cuda", dtype=torch.int8)
+    a_scale = torch.ones((1,), device="cuda", dtype=torch.float32)
+    y = torch.empty((1, n), device="cuda", dtype=torch.float32)
+    for bl in layers:
+        bl.matmul_quantized(a, a_scale, out=y)
+    ms = time_events(torch, lambda: [bl.matmul_quantized(a, a_scale, out=y) for _ in range(loops) for bl in layers]) / (4 * loops)
+    out["gemv_32768x16384_m1"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1),
+                                  "frac_hbm_peak": round(n * k / 4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    del layers, packed
+    b3_bytes = bh.base3_packed_size(n * k)
+    tiled3 = [bh.retile_base3(torch.randint(0, 243, (b3_bytes,), generator=gen, device="cuda", dtype=torch.uint8), n, k)
+              for _ in range(4)]
+    for t3 in tiled3:
+        bh.gemv_base3(t3, a.view(-1), n, want_acc=False, w_scale=a_scale, out=y.view(-1))
+    ms3 = time_events(torch, lambda: [bh.gemv_base3(t3, a.view(-1), n, want_acc=False, w_scale=a_scale, out=y.view(-1))
+                                      for _ in range(loops) for t3 in tiled3]) / (4 * loops)
+    out["gemv_base3_32768x16384_m1"] = {
+        "us": round(ms3 * 1e3, 2), "bytes_per_launch": b3_bytes,
+        "gbs_base3_bytes": round(b3_bytes / (ms3 * 1e-3) / 1e9, 1),
+        "frac_hbm_peak": round(b3_bytes / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "speed_vs_2bit_gemv": round(ms / ms3, 3),
+        "note": "the decode GEMV consuming Base3PackedPacker bytes (1.6 bits per weight) directly; bound by the LDS table "
+                "look-ups that take a byte apart, not by memory"}
+    return out
+
+
 def stack_latency(bh, torch, dec, gen, reps=20):
     """configs[4]: per-token decode latency through all 30 layers' projections, batch 1 and batch 8, and
     configs[2]: the gate / down projections at M in {1, 4, 16, 64} tokens (activations with 1 % x20 outliers)."""
@@ -207,22 +243,7 @@ def stack_latency(bh, torch, dec, gen, reps=20):
                                     "timed": "the recorded step replayed (HIP graph); eager = launches enqueued one by one"}
         del recorded
     del big
-    # the decode GEMV where a launch is large enough to be bound by bandwidth rather than by launch latency:
-    # 32768 x 16384 ternary weights (128 MiB packed), int8 activations already quantised, one token
-    n, k = 32768, 16384
-    layers = [bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), f"large{i}") for i in range(4)]  # 512 MiB > cache
-    packed = torch.randint(0, 256, (n * k // 4,), generator=gen, device="cuda", dtype=torch.uint8)
-    for bl in layers:
-        bl.set_quantized_weights(packed, 0.02)
-    a = torch.randint(-127, 128, (1, k), generator=gen, device="cuda", dtype=torch.int8)
-    a_scale = torch.ones((1,), device="cuda", dtype=torch.float32)
-    y = torch.empty((1, n), device="cuda", dtype=torch.float32)
-    for bl in layers:
-        bl.matmul_quantized(a, a_scale, out=y)
-    ms = time_events(torch, lambda: [bl.matmul_quantized(a, a_scale, out=y) for _ in range(5) for bl in layers]) / 20
-    out["gemv_32768x16384_m1"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1),
-                                  "frac_hbm_peak": round(n * k / 4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
-    del layers, packed
+    out.update(large_gemv_pair(bh, torch, gen))
     for name, p in (("gate_2560x6912", 4), ("down_6912x2560", 6)):
         n, k = dec.proj_shape(p)
         bls = [dec.projection(layer, p) for layer in range(dec.layers)]  # rotating: 4.4 MB each, not L2-resident
@@ -420,6 +441,9 @@ def main():
                     help="run only the two M=2048 prefill GEMMs REPS times each and print their rates (profiling runs)")
     ap.add_argument("--only-batch8", type=int, default=0, metavar="STEPS",
                     help="run only STEPS token steps of the 30-layer stack at batch 8 (profiling runs)")
+    ap.add_argument("--only-large-gemv", type=int, default=0, metavar="LOOPS",
+                    help="run only the 32768 x 16384 one-token GEMV, on 2-bit tiles and on base-3 bytes, LOOPS times over four "
+                         "matrices each (profiling runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -434,6 +458,11 @@ def main():
     import bitnet_hip as bh
 
     bh.init(0)
+    if args.only_large_gemv > 0:
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(0)
+        print(json.dumps(large_gemv_pair(bh, torch, gen, loops=args.only_large_gemv)))
+        return
     dec, gen = build_stack(bh, torch, LAYERS)
     if args.only_prefill > 0:
         print(json.dumps({"prefill": prefill_rates(bh, torch, dec, gen, reps=args.only_prefill)}))

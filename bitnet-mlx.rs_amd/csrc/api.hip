@@ -406,6 +406,28 @@ int bitnet_hip_unpack_ternary_base3(const uint8_t *packed, size_t count, int8_t 
     return launch_unpack_base3(packed, count, q, as_stream(stream));
 }
 
+size_t bitnet_hip_base3_tiled_size(size_t n, size_t k) { return base3_tiled_bytes(n, k); }
+
+int bitnet_hip_retile_base3(const uint8_t *base3, size_t n, size_t k, uint8_t *tiled, void *stream)
+{
+    if (n == 0 || k == 0) return BITNET_HIP_OK;
+    if (!base3 || !tiled) return fail(BITNET_HIP_NULL_POINTER, "retile_base3: null argument");
+    return launch_retile_base3(base3, n, k, tiled, as_stream(stream));
+}
+
+int bitnet_hip_gemv_base3(const uint8_t *tiled, const int8_t *a, size_t n, size_t k, const float *w_scale,
+                          const float *a_scale, int32_t *acc, float *out, void *stream)
+{
+    if (n == 0) return BITNET_HIP_OK;
+    if (k == 0) return fail(BITNET_HIP_INVALID_CONFIG, "gemv_base3: k must be positive");
+    if (!tiled || !a) return fail(BITNET_HIP_NULL_POINTER, "gemv_base3: null weights or activations");
+    if (!acc && !out) return fail(BITNET_HIP_NULL_POINTER, "gemv_base3: neither acc nor out given");
+    if (out && !w_scale) return fail(BITNET_HIP_NULL_POINTER, "gemv_base3: out needs w_scale");
+    if ((reinterpret_cast<uintptr_t>(tiled) & 15) != 0)
+        return fail(BITNET_HIP_INVALID_CONFIG, "gemv_base3: the tiled weights must be 16-byte aligned");
+    return launch_gemv_base3(tiled, a, acc, out, w_scale, a_scale, n, k, as_stream(stream));
+}
+
 int bitnet_hip_quantize_weights(const float *w, size_t n, size_t k, int method, float threshold_factor,
                                 uint8_t *packed, float *w_scale, int8_t *q_i8, void *stream)
 {

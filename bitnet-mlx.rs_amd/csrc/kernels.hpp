@@ -45,6 +45,12 @@ int launch_quantize_weights_reference(const float *w, size_t n, size_t k, int me
 int launch_retile(const uint8_t *packed, size_t n, size_t k, int layout, uint8_t *tiled, hipStream_t stream);
 int launch_untile(const uint8_t *tiled, size_t n, size_t k, uint8_t *packed, hipStream_t stream);
 
+// gemv_base3.hip: the decode GEMV on base-3 bytes (five values per byte) in their own streaming layout
+size_t base3_tiled_bytes(size_t n, size_t k);
+int launch_retile_base3(const uint8_t *flat, size_t n, size_t k, uint8_t *tiled, hipStream_t stream);
+int launch_gemv_base3(const uint8_t *tiled, const int8_t *a, int32_t *acc, float *out, const float *w_scale, const float *a_scale,
+                      size_t n, size_t k, hipStream_t stream);
+
 // gemv_w2a8.hip
 int launch_gemv_rowmajor(const uint8_t *packed, const int8_t *a, int32_t *out, size_t n, size_t k,
                          hipStream_t stream);

@@ -99,6 +99,9 @@ def load_library() -> C.CDLL:
         "bitnet_hip_base3_packed_size": (sz, [sz]),
         "bitnet_hip_pack_ternary_base3": (i32, [vp, sz, vp, vp]),
         "bitnet_hip_unpack_ternary_base3": (i32, [vp, sz, vp, vp]),
+        "bitnet_hip_base3_tiled_size": (sz, [sz, sz]),
+        "bitnet_hip_retile_base3": (i32, [vp, sz, sz, vp, vp]),
+        "bitnet_hip_gemv_base3": (i32, [vp, vp, sz, sz, vp, vp, vp, vp, vp]),
         "bitnet_hip_quantize_weights": (i32, [vp, sz, sz, i32, f32, vp, vp, vp, vp]),
         "bitnet_hip_quantize_weights_reference": (i32, [vp, sz, sz, i32, i32, f32, f32, vp, vp, vp, vp, vp]),
         "bitnet_hip_tiled_size": (sz, [sz, sz]),
@@ -394,6 +397,43 @@ def unpack_ternary_base3(packed: torch.Tensor, count: int, stream=None) -> torch
     out = torch.empty((count,), dtype=torch.int8, device=packed.device)
     _check(load_library().bitnet_hip_unpack_ternary_base3(_ptr(packed), count, _ptr(out), _stream(stream)))
     return out
+
+
+def base3_tiled_size(n: int, k: int) -> int:
+    return load_library().bitnet_hip_base3_tiled_size(n, k)
+
+
+def retile_base3(base3: torch.Tensor, n: int, k: int, stream=None) -> torch.Tensor:
+    """The bytes Base3PackedPacker emits for the flat [n, k] tensor, re-ordered into the streaming layout of
+    gemv_base3 (tiles of 16 rows x 320 columns)."""
+    _dev(base3, torch.uint8, "base3")
+    if base3.numel() < base3_packed_size(n * k):
+        raise BitLinearError(SHAPE_MISMATCH, "base-3 buffer too short", [base3_packed_size(n * k)], [base3.numel()])
+    out = torch.empty((base3_tiled_size(n, k),), dtype=torch.uint8, device=base3.device)
+    _check(load_library().bitnet_hip_retile_base3(_ptr(base3), n, k, _ptr(out), _stream(stream)))
+    return out
+
+
+def gemv_base3(tiled: torch.Tensor, a: torch.Tensor, n: int, w_scale: Optional[torch.Tensor] = None,
+               a_scale: Optional[torch.Tensor] = None, want_acc: bool = True, out: Optional[torch.Tensor] = None, stream=None):
+    """One token against base-3 weights in their streaming layout: returns (acc int32 [n] or None, out f32 [n] or None)."""
+    _dev(tiled, torch.uint8, "tiled")
+    _dev(a, torch.int8, "a")
+    k = a.numel()
+    if tiled.numel() != base3_tiled_size(n, k):
+        raise BitLinearError(SHAPE_MISMATCH, "base-3 tiles", [base3_tiled_size(n, k)], [tiled.numel()])
+    _opt_dev(w_scale, torch.float32, "w_scale", 1, a)
+    _opt_dev(a_scale, torch.float32, "a_scale", 1, a)
+    acc = torch.empty((n,), dtype=torch.int32, device=a.device) if want_acc else None
+    if out is None and w_scale is not None:
+        out = torch.empty((n,), dtype=torch.float32, device=a.device)
+    elif out is not None:
+        _dev(out, torch.float32, "out")
+        if out.numel() != n or w_scale is None:
+            raise BitLinearError(SHAPE_MISMATCH, "gemv_base3 output (needs w_scale)", [n], [out.numel()])
+    _check(load_library().bitnet_hip_gemv_base3(_ptr(tiled), _ptr(a), n, k, _ptr(w_scale), _ptr(a_scale), _ptr(acc), _ptr(out),
+                                                _stream(stream)))
+    return acc, out
 
 
 def quantize_weights(w: torch.Tensor, method: int = TERNARY_ABSMEAN_ROUNDCLIP, threshold_factor: float = 0.5,

@@ -5,7 +5,7 @@ use std::path::PathBuf;
 use std::process::Command;
 
 const KERNELS: &[&str] =
-    &["api.hip", "act_quant.hip", "weight_prep.hip", "gemv_w2a8.hip", "gemm_w2a8.hip", "diag.hip"];
+    &["api.hip", "act_quant.hip", "weight_prep.hip", "gemv_w2a8.hip", "gemm_w2a8.hip", "gemv_base3.hip", "diag.hip"];
 
 fn main() {
     println!("cargo:rerun-if-changed=build.rs");

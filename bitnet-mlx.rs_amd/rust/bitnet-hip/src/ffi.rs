@@ -76,6 +76,10 @@ extern "C" {
     pub fn bitnet_hip_base3_packed_size(count: usize) -> usize;
     pub fn bitnet_hip_pack_ternary_base3(q: *const i8, count: usize, packed: *mut u8, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_unpack_ternary_base3(packed: *const u8, count: usize, q: *mut i8, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_base3_tiled_size(n: usize, k: usize) -> usize;
+    pub fn bitnet_hip_retile_base3(base3: *const u8, n: usize, k: usize, tiled: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_gemv_base3(tiled: *const u8, a: *const i8, n: usize, k: usize, w_scale: *const f32,
+                                 a_scale: *const f32, acc: *mut i32, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_quantize_weights(w: *const f32, n: usize, k: usize, method: c_int, threshold_factor: f32,
                                        packed: *mut u8, w_scale: *mut f32, q_i8: *mut i8, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_quantize_weights_reference(w: *const f32, n: usize, k: usize, ternary_method: c_int,

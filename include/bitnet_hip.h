@@ -175,6 +175,19 @@ int bitnet_hip_unpack_ternary_2bit(const uint8_t *packed, size_t count, int8_t *
 size_t bitnet_hip_base3_packed_size(size_t count);
 int bitnet_hip_pack_ternary_base3(const int8_t *q, size_t count, uint8_t *packed, void *stream);
 int bitnet_hip_unpack_ternary_base3(const uint8_t *packed, size_t count, int8_t *q, void *stream);
+/* The decode GEMV on base-3 bytes themselves (1.6 bits per weight, 20 % fewer bytes than the 2-bit codes): one token,
+ * acc[n] = sum_k a[k] * w[n, k] in int32, out[n] = (float(acc) * w_scale) / a_scale.
+ *   bitnet_hip_retile_base3 re-orders the bytes Base3PackedPacker::pack emits for the flat row-major [n, k] tensor
+ *   (packing.rs:421-501; base3 holds (n*k + 4) / 5 bytes) into a streaming layout of bitnet_hip_base3_tiled_size(n, k)
+ *   bytes: tiles of 16 rows x 320 columns, a byte = five consecutive columns of one row, weight 0 past the matrix.
+ *   bitnet_hip_gemv_base3 contracts that layout with int8 activations a[k]; acc or out may be NULL (out needs w_scale;
+ *   a_scale NULL = 1).  All pointers are DEVICE memory.  Semantics as bitnet_hip_gemv_w2a8
+ *   (bitnet-quant/src/simd/matrix.rs:471-490).  The kernel is bound by the table look-ups that take a base-3 byte
+ *   apart, not by memory: it is slower than the 2-bit GEMV at every size measured and no BitLinear object uses it. */
+size_t bitnet_hip_base3_tiled_size(size_t n, size_t k);
+int bitnet_hip_retile_base3(const uint8_t *base3, size_t n, size_t k, uint8_t *tiled, void *stream);
+int bitnet_hip_gemv_base3(const uint8_t *tiled, const int8_t *a, size_t n, size_t k, const float *w_scale,
+                          const float *a_scale, int32_t *acc, float *out, void *stream);
 
 /* Ternarise an f32 weight matrix [n, k] (row-major) and pack it in the reference's byte format.
  *   replaces SimdTernaryOps::{compute_absmean, quantize_batch} (bitnet-quant/src/simd/ternary.rs:27-66)

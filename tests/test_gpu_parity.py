@@ -593,6 +593,52 @@ def test_bitlinear_base3_weights_match_2bit_weights(n, k, on_device):
         assert err.value.status == bh.SHAPE_MISMATCH
 
 
+@pytest.mark.parametrize("n,k", [(16, 320), (1, 5), (33, 7), (48, 300), (640, 2560), (2560, 6912), (100, 2561), (4096, 4096)])
+def test_gemv_on_base3_bytes_bit_exact(n, k):
+    """bitnet_hip_gemv_base3: the decode GEMV that consumes the base-3 bytes of Base3PackedPacker (packing.rs:421-501)
+    themselves.  The streaming layout is built from the oracle's flat base-3 bytes; int32 accumulators equal the oracle's
+    contraction of the same ternary matrix (and hence the 2-bit GEMV), the f32 output its epilogue; the reference's
+    encoding fixture (140 = [1, 0, -1, 1, 0]) goes through the same path."""
+    rng = np.random.default_rng(7 * n + k)
+    q = rng.integers(-1, 2, size=(n, k)).astype(np.int8)
+    a = rng.integers(-127, 128, size=(1, k)).astype(np.int8)
+    b3 = orc.pack_base3(q.ravel())
+    tiled = bh.retile_base3(dev(b3), n, k)
+    assert tiled.numel() == bh.base3_tiled_size(n, k) == ((n + 15) // 16) * ((k + 319) // 320) * 1024
+    ws, a_scale = f32(0.0171), np.array([f32(3.37)], dtype=f32)
+    acc, out = bh.gemv_base3(tiled, dev(a.ravel()), n, w_scale=dev(np.array([ws], dtype=f32)), a_scale=dev(a_scale))
+    acc_ref = orc.gemm_w2a8(orc.pack_2bit(q.ravel()), a, n)
+    assert np.array_equal(host(acc), acc_ref[0])
+    assert np.array_equal(host(out), orc.epilogue(acc_ref, ws, a_scale)[0])
+    # the streaming layout, byte by byte: slot 16 kq + r of tile (row block, k-tile), byte t = columns 320 kt + 80 kq + 5 t ..
+    th = host(tiled).reshape(-1, 64, 16)
+    kt_count = (k + 319) // 320
+    for _ in range(64):
+        row, col = int(rng.integers(n)), int(rng.integers(k))
+        kt, rem = divmod(col, 320)
+        kq, rem = divmod(rem, 80)
+        t, d = divmod(rem, 5)
+        byte = int(th[(row // 16) * kt_count + kt, 16 * kq + row % 16, t])
+        assert (byte // 3 ** d) % 3 - 1 == q[row, col]
+
+
+def test_gemv_on_base3_bytes_reference_fixture_and_errors():
+    """The reference's own base-3 vector (packing_correctness_tests.rs:159-176: [1, 0, -1, 1, 0] -> 140) as a 1 x 5 matrix,
+    and the argument checks of the entry point."""
+    b3 = np.array([140], dtype=np.uint8)
+    assert np.array_equal(orc.unpack_base3(b3, 5), np.array([1, 0, -1, 1, 0], dtype=np.int8))
+    tiled = bh.retile_base3(dev(b3), 1, 5)
+    a = np.array([3, -7, 11, 5, 100], dtype=np.int8)
+    acc, out = bh.gemv_base3(tiled, dev(a), 1)
+    assert out is None and host(acc).tolist() == [3 - 11 + 5]
+    with pytest.raises(bh.BitLinearError) as err:
+        bh.gemv_base3(tiled[:-16].contiguous(), dev(a), 1)
+    assert err.value.status == bh.SHAPE_MISMATCH
+    with pytest.raises(bh.BitLinearError) as err:
+        bh.retile_base3(dev(b3), 2, 5)
+    assert err.value.status == bh.SHAPE_MISMATCH
+
+
 @pytest.mark.parametrize("kind,cls", [(bh.LOOKUP_TERNARY, bh.HipTernaryLookupKernel), (bh.LOOKUP_I2S, bh.HipI2SLookupKernel)],
                          ids=["ternary", "i2s"])
 def test_lookup_kernels_bit_exact(kind, cls):
