@@ -502,7 +502,55 @@ __global__ __launch_bounds__(64) void absmax_finish_kernel(const double *row_sum
     }
 }
 
+// DynamicActivationQuantizer::quantize with a scale given from outside (activations.rs:269-294, 315-360): y = x * r with
+// r = (float)(1.0 / (double)scale), as candle's affine(1.0 / scale as f64, 0.0) computes it on an f32 tensor.
+//   ternary: +1 where y > 0.5, -1 where y < -0.5, else 0
+//   8-bit:   round(clamp(y, -127, 127)) as int8, or, with reference_u8, the reference's literal clamp(0, 255).round()
+//            as the byte of a u8 (every negative activation becomes 0 there)
+__global__ __launch_bounds__(256) void scaled_quantize_kernel(const float *x, size_t n, int precision, float recip, int reference_u8,
+                                                              int8_t *q)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        const float y = f32_mul(x[i], recip);
+        int v;
+        if (precision == BITNET_HIP_PRECISION_EIGHT_BIT) {
+            const float lo = reference_u8 ? 0.0f : -127.0f, hi = reference_u8 ? 255.0f : 127.0f;
+            float c = y > hi ? hi : y;
+            c = c < lo ? lo : c;
+            const float r = roundf(c);  // halves away from zero, as f32::round
+            v = (r != r) ? 0 : (int)r;
+        } else {
+            v = y > 0.5f ? 1 : (y < -0.5f ? -1 : 0);
+        }
+        q[i] = (int8_t)(uint8_t)(unsigned)v;  // 0..255 keep their byte in the u8 form
+    }
+}
+
 }  // namespace
+
+int launch_abs_max(const float *x, size_t n, void *scratch, hipStream_t stream)
+{
+    AbsmaxState *state = static_cast<AbsmaxState *>(scratch);
+    float *part = reinterpret_cast<float *>(static_cast<uint8_t *>(scratch) + 256);
+    int blocks = (int)((n + 255) / 256);
+    blocks = blocks < 1 ? 1 : (blocks > 1024 ? 1024 : blocks);
+    hipLaunchKernelGGL(absmax_partial_kernel, dim3(blocks), dim3(256), 0, stream, x, n, part);
+    BITNET_HIP_CHECK_LAUNCH("absmax_partial_kernel");
+    hipLaunchKernelGGL(absmax_scale_kernel, dim3(1), dim3(64), 0, stream, part, blocks, BITNET_HIP_PRECISION_ONE_FIVE_FIVE_BIT, state);
+    BITNET_HIP_CHECK_LAUNCH("absmax_scale_kernel");
+    return BITNET_HIP_OK;  // state->abs_max is the first float of the scratch
+}
+
+int launch_scaled_quantize(const float *x, size_t n, int precision, float scale, int reference_u8, int8_t *q, hipStream_t stream)
+{
+    if (n == 0) return BITNET_HIP_OK;
+    const float recip = (float)(1.0 / (double)scale);
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(scaled_quantize_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, n, precision, recip, reference_u8, q);
+    BITNET_HIP_CHECK_LAUNCH("scaled_quantize_kernel");
+    return BITNET_HIP_OK;
+}
 
 size_t absmax_quantize_scratch_bytes(size_t n)
 {

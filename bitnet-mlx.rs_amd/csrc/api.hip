@@ -358,6 +358,31 @@ int bitnet_hip_absmax_quantize_activations(const float *x, size_t count, int pre
     return BITNET_HIP_OK;
 }
 
+int bitnet_hip_abs_max(const float *x, size_t count, float *abs_max, void *stream)
+{
+    if (!abs_max) return fail(BITNET_HIP_NULL_POINTER, "abs_max: the result pointer is required");
+    *abs_max = 0.0f;
+    if (count == 0) return BITNET_HIP_OK;
+    if (!x) return fail(BITNET_HIP_NULL_POINTER, "abs_max: null buffer");
+    DeviceTemp scratch;
+    int rc = scratch.alloc(absmax_quantize_scratch_bytes(count));
+    if (rc != BITNET_HIP_OK) return rc;
+    rc = launch_abs_max(x, count, scratch.ptr, as_stream(stream));
+    if (rc != BITNET_HIP_OK) return rc;
+    BITNET_HIP_TRY(hipMemcpyAsync(abs_max, scratch.ptr, sizeof(float), hipMemcpyDeviceToHost, as_stream(stream)));
+    BITNET_HIP_TRY(hipStreamSynchronize(as_stream(stream)));  // the value is the caller's on return, as to_scalar() is
+    return BITNET_HIP_OK;
+}
+
+int bitnet_hip_quantize_activations_scaled(const float *x, size_t count, int precision, float scale, int reference_u8,
+                                           int8_t *values, void *stream)
+{
+    if (precision != BITNET_HIP_PRECISION_ONE_FIVE_FIVE_BIT && precision != BITNET_HIP_PRECISION_EIGHT_BIT)
+        return fail(BITNET_HIP_UNSUPPORTED, "quantize_activations_scaled: unsupported precision %d", precision);
+    if (count != 0 && (!x || !values)) return fail(BITNET_HIP_NULL_POINTER, "quantize_activations_scaled: null buffer");
+    return launch_scaled_quantize(x, count, precision, scale, reference_u8 != 0, values, as_stream(stream));
+}
+
 // ---- lookup-table kernels ----------------------------------------------------------------------------
 
 int bitnet_hip_lookup_compute(int kind, const int8_t *weights, size_t n_weights, const float *inputs, size_t n_inputs,

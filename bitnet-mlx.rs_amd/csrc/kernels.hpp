@@ -23,6 +23,10 @@ int launch_act_quant(const float *x, const float *x2, size_t ldx, size_t m, size
 // bytes; stats: 4 floats (scale, mse, min, max)
 size_t absmax_quantize_scratch_bytes(size_t n);
 int launch_absmax_quantize(const float *x, size_t n, int precision, void *scratch, int8_t *q, float *stats, hipStream_t stream);
+// max |x| of a tensor into the first float of `scratch` (absmax_quantize_scratch_bytes(n) bytes), and the quantiser of
+// DynamicActivationQuantizer with the scale given from outside (activations.rs:269-294, 315-360)
+int launch_abs_max(const float *x, size_t n, void *scratch, hipStream_t stream);
+int launch_scaled_quantize(const float *x, size_t n, int precision, float scale, int reference_u8, int8_t *q, hipStream_t stream);
 
 // weight_prep.hip
 int launch_pack_2bit(const int8_t *q, size_t count, uint8_t *packed, hipStream_t stream);

@@ -10,6 +10,8 @@
 //   bitnet::TernaryProcessor          bitnet-inference/src/engine/ternary_operations.rs:56-172
 //   bitnet::QuantizedActivation, absmax_quantize_activations
 //                                     bitnet-quant/src/quantization/activations.rs:95-112,530-641
+//   bitnet::ActivationQuantizationConfig, DynamicActivationQuantizer
+//                                     bitnet-quant/src/quantization/activations.rs:14-91,203-454
 //   bitnet::WeightQuantizationConfig, BitNetWeightQuantizer, QuantizedWeight
 //                                     bitnet-quant/src/quantization/weights.rs:58-95,158-175,341-611
 //   bitnet::HipInferenceBackend       the InferenceBackend trait, bitnet-inference/src/engine/mod.rs:126-148
@@ -368,6 +370,108 @@ inline Result<QuantizedActivation> absmax_quantize_activations(const DeviceTenso
     q.stats = {n, h[1], 32.0f / q.effective_bit_width(), h[2], h[3], h[0]};
     return q;
 }
+
+// DynamicActivationQuantizer (activations.rs:203-454): the state (exponential moving average of the scale, window of
+// recent scales, warm-up counter, calibration flag) on the host in single precision, as the reference keeps it; abs-max and
+// the quantisation with the current scale on the device.
+struct ActivationQuantizationConfig {  // activations.rs:14-45, with its defaults
+    QuantizationPrecision precision = QuantizationPrecision::OneFiveFiveBit;
+    size_t moving_average_window = 100;
+    float outlier_percentile = 99.9f;
+    bool per_token = false;
+    size_t calibration_warmup = 50;
+    float ema_decay = 0.99f;
+    bool quantize_attention = true;
+    Result<Unit> validate() const  // :71-91
+    {
+        if (moving_average_window == 0) return BitLinearError{BitLinearError::ConfigError, "Moving average window cannot be zero", {}, {}};
+        if (outlier_percentile <= 0.0f || outlier_percentile > 100.0f)
+            return BitLinearError{BitLinearError::ConfigError, "Outlier percentile must be in range (0, 100]", {}, {}};
+        if (ema_decay < 0.0f || ema_decay > 1.0f) return BitLinearError{BitLinearError::ConfigError, "EMA decay must be in range [0, 1]", {}, {}};
+        return Unit{};
+    }
+};
+class DynamicActivationQuantizer {
+public:
+    explicit DynamicActivationQuantizer(ActivationQuantizationConfig c = {}) : config_(c) {}
+    const ActivationQuantizationConfig &config() const { return config_; }
+    // quantize (:315-360): the moving average if there is one, else the tensor's own abs-max
+    Result<QuantizedActivation> quantize(const DeviceTensor &activations, hipStream_t stream = nullptr) const
+    {
+        if (activations.dims().empty())
+            return BitLinearError{BitLinearError::QuantizationError, "Activation tensor must have at least 1 dimension", {}, {}};
+        const size_t n = activations.elem_count();
+        float scale = 0.0f;
+        if (ema_scale_) {
+            scale = *ema_scale_;
+        } else {
+            int rc = bitnet_hip_abs_max(activations.data(), n, &scale, stream);
+            if (rc != BITNET_HIP_OK) return last_error(rc);
+        }
+        QuantizedActivation q;
+        q.precision = config_.precision;
+        q.original_shape = activations.dims();
+        int8_t *v = nullptr;
+        if (hipMalloc(reinterpret_cast<void **>(&v), n ? n : 1) != hipSuccess)
+            return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
+        q.values.reset(v, [](int8_t *p) { (void)hipFree(p); });
+        int rc = bitnet_hip_quantize_activations_scaled(activations.data(), n, static_cast<int>(q.precision), scale, 0, v, stream);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        q.scales = scale;
+        q.stats.elements_count = n;
+        q.stats.scale_factor = scale;
+        q.stats.compression_ratio = 32.0f / q.effective_bit_width();
+        return q;
+    }
+    // quantize_dynamic (:372-383): count the step, update the moving average, quantise with it
+    Result<QuantizedActivation> quantize_dynamic(const DeviceTensor &activations, hipStream_t stream = nullptr)
+    {
+        ++step_count_;
+        auto up = update_dynamic_params(activations, stream);
+        if (up.is_err()) return up.unwrap_err();
+        return quantize(activations, stream);
+    }
+    // update_dynamic_params + compute_dynamic_scale (:241-267, 406-433)
+    Result<Unit> update_dynamic_params(const DeviceTensor &activations, hipStream_t stream = nullptr)
+    {
+        float abs_max = 0.0f;
+        int rc = bitnet_hip_abs_max(activations.data(), activations.elem_count(), &abs_max, stream);
+        if (rc != BITNET_HIP_OK) return last_error(rc);
+        const float current = config_.precision == QuantizationPrecision::EightBit ? abs_max / 127.0f : abs_max / 1.0f;
+        if (ema_scale_) {
+            const float kept = config_.ema_decay * *ema_scale_, fresh = (1.0f - config_.ema_decay) * current;
+            ema_scale_ = kept + fresh;
+        } else {
+            ema_scale_ = current;
+        }
+        if (scale_history_.size() >= config_.moving_average_window) scale_history_.erase(scale_history_.begin());
+        scale_history_.push_back(current);
+        if (step_count_ <= config_.calibration_warmup) {
+            if (calibration_samples_ < config_.calibration_warmup) ++calibration_samples_;
+        } else if (!calibrated_) {
+            calibrated_ = true;
+        }
+        return Unit{};
+    }
+    float get_dynamic_scales() const { return ema_scale_.value_or(1.0f); }
+    void reset_dynamic_state()
+    {
+        scale_history_.clear();
+        ema_scale_.reset();
+        calibrated_ = false;
+        step_count_ = 0;
+        calibration_samples_ = 0;
+    }
+    bool needs_calibration() const { return !calibrated_ || step_count_ <= config_.calibration_warmup; }
+    const std::vector<float> &scale_history() const { return scale_history_; }
+
+private:
+    ActivationQuantizationConfig config_;
+    std::vector<float> scale_history_;
+    std::optional<float> ema_scale_;
+    bool calibrated_ = false;
+    size_t step_count_ = 0, calibration_samples_ = 0;
+};
 
 // BitNetWeightQuantizer::quantize with its whole configuration (weights.rs:568-611).
 enum class TernaryMethod { MeanThreshold = 0, MedianThreshold, AdaptiveThreshold, OptimalThreshold, DetSTE };

@@ -123,6 +123,35 @@ int main()
         (void)hipMemcpy(h, qt.unwrap().values.get(), 4, hipMemcpyDeviceToHost);
         CHECK(h[0] == 1 && h[1] == 0 && h[2] == 0 && h[3] == -1);  // |x| / 4 > 0.5 only for 4 and -3
     }
+    {  // DynamicActivationQuantizer: the reference's own checks (activation_quantization_correctness_tests.rs:486-590)
+        DynamicActivationQuantizer dq;  // default: ternary
+        auto x = DeviceTensor::from_vec({0.2f, -1.5f, 3.0f, -0.4f, 2.9f, 0.0f, -3.0f, 1.4f}, {2, 4});
+        auto q0 = dq.quantize(x.unwrap());  // no state yet: the tensor's own abs-max
+        CHECK(q0.is_ok() && q0.unwrap().stats.scale_factor == 3.0f && q0.unwrap().original_shape == x.unwrap().dims());
+        int8_t h[8];
+        (void)hipMemcpy(h, q0.unwrap().values.get(), 8, hipMemcpyDeviceToHost);
+        CHECK(h[0] == 0 && h[1] == 0 && h[2] == 1 && h[3] == 0 && h[4] == 1 && h[5] == 0 && h[6] == -1 && h[7] == 0);  // |x| / 3 > 0.5
+        auto small = DeviceTensor::from_vec({0.01f, -0.02f, 0.015f, 0.005f}, {2, 2});
+        auto large = DeviceTensor::from_vec({10.0f, -20.0f, 15.0f, 5.0f}, {2, 2});
+        auto qs = dq.quantize_dynamic(small.unwrap());
+        auto ql = dq.quantize_dynamic(large.unwrap());
+        CHECK(qs.is_ok() && ql.is_ok() && qs.unwrap().stats.scale_factor == 0.02f);
+        const float kept = 0.99f * 0.02f, fresh = (1.0f - 0.99f) * 20.0f;
+        CHECK(ql.unwrap().stats.scale_factor == kept + fresh && qs.unwrap().stats.scale_factor < ql.unwrap().stats.scale_factor);
+        CHECK(dq.scale_history().size() == 2 && dq.needs_calibration());
+        dq.reset_dynamic_state();
+        auto again = dq.quantize_dynamic(large.unwrap());
+        CHECK(again.is_ok() && again.unwrap().stats.scale_factor == 20.0f && dq.get_dynamic_scales() == 20.0f);
+        ActivationQuantizationConfig c8; c8.precision = QuantizationPrecision::EightBit;
+        DynamicActivationQuantizer d8(c8);
+        auto y = DeviceTensor::from_vec({100.0f, -50.0f, 25.0f, -75.0f}, {4});
+        auto q8 = d8.quantize_dynamic(y.unwrap());
+        CHECK(q8.is_ok() && q8.unwrap().stats.scale_factor == 100.0f / 127.0f);
+        (void)hipMemcpy(h, q8.unwrap().values.get(), 4, hipMemcpyDeviceToHost);
+        CHECK(h[0] == 127 && h[1] == -64 && h[2] == 32 && h[3] == -95);
+        ActivationQuantizationConfig bad; bad.ema_decay = 1.5f;
+        CHECK(bad.validate().is_err() && ActivationQuantizationConfig{}.validate().is_ok());
+    }
     {  // BitNetWeightQuantizer: the packed bytes loaded into a layer give the forward the quantiser's codes imply
         const size_t n = 48, k = 256;
         auto w = DeviceTensor::from_vec(randn(n * k, 21, 1.0f), {n, k});

@@ -92,6 +92,8 @@ def load_library() -> C.CDLL:
         "bitnet_hip_measure_launch_chain": (i32, [vp, C.POINTER(sz), sz, sz, sz, C.POINTER(C.c_double), vp]),
         "bitnet_hip_quantize_activations_i8": (i32, [vp, vp, sz, sz, sz, i32, sz, sz, vp, f32, i32, vp, vp, vp, vp, vp]),
         "bitnet_hip_absmax_quantize_activations": (i32, [vp, sz, i32, vp, vp, vp]),
+        "bitnet_hip_abs_max": (i32, [vp, sz, C.POINTER(C.c_float), vp]),
+        "bitnet_hip_quantize_activations_scaled": (i32, [vp, sz, i32, f32, i32, vp, vp]),
         "bitnet_hip_lookup_compute": (i32, [i32, vp, sz, vp, sz, vp, sz, vp]),
         "bitnet_hip_packed_size": (sz, [sz]),
         "bitnet_hip_pack_ternary_2bit": (i32, [vp, sz, vp, vp]),
@@ -353,6 +355,191 @@ class ActivationQuantizer:
     def dequantize(self, quantized: QuantizedActivation) -> torch.Tensor:
         """values * scales (a host-side convenience through torch; not on the forward path)."""
         return quantized.values.to(torch.float32) * quantized.scales
+
+
+@dataclass
+class ActivationQuantizationConfig:
+    """ActivationQuantizationConfig (activations.rs:14-45) with its defaults; `precision` stands for base.precision
+    (QuantizationConfig::default() is OneFiveFiveBit, as ActivationQuantizationConfig::bitnet())."""
+    precision: int = QuantizationPrecision.OneFiveFiveBit
+    moving_average_window: int = 100
+    outlier_percentile: float = 99.9
+    per_token: bool = False
+    calibration_warmup: int = 50
+    ema_decay: float = 0.99
+    quantize_attention: bool = True
+
+    def validate(self):
+        """activations.rs:71-91."""
+        if self.moving_average_window == 0:
+            raise BitLinearError(INVALID_CONFIG, "Moving average window cannot be zero")
+        if self.outlier_percentile <= 0.0 or self.outlier_percentile > 100.0:
+            raise BitLinearError(INVALID_CONFIG, "Outlier percentile must be in range (0, 100]")
+        if self.ema_decay < 0.0 or self.ema_decay > 1.0:
+            raise BitLinearError(INVALID_CONFIG, "EMA decay must be in range [0, 1]")
+
+
+class DynamicScaleState:
+    """The host-side state of DynamicActivationQuantizer (activations.rs:203-267, 406-447, 456-493): the exponential moving
+    average of the scale, the window of recent scales, the warm-up counter and the calibration flag.  Every operation is
+    single-precision arithmetic in the reference's order; it touches no device."""
+
+    def __init__(self, config: ActivationQuantizationConfig):
+        self.config = config
+        self.scale_history: list = []
+        self.ema_scale = None
+        self.calibrated = False
+        self.step_count = 0
+        self.calibration_samples = 0  # the reference keeps the tensors themselves and never reads them again
+
+    def current_scale(self, abs_max) -> "np.float32":
+        """compute_dynamic_scale's per-step scale (:245-249): abs_max / 1.0 for ternary, abs_max / 127.0 for 8-bit."""
+        import numpy as np
+        a = np.float32(abs_max)
+        if self.config.precision == QuantizationPrecision.OneFiveFiveBit:
+            return a / np.float32(1.0)
+        if self.config.precision == QuantizationPrecision.EightBit:
+            return a / np.float32(127.0)
+        raise BitLinearError(UNSUPPORTED, f"UnsupportedPrecision({self.config.precision})")
+
+    def update(self, abs_max) -> "np.float32":
+        """update_dynamic_params (:420-433) for a tensor whose max |x| is abs_max; returns the moving average."""
+        import numpy as np
+        cur = self.current_scale(abs_max)
+        decay = np.float32(self.config.ema_decay)
+        if self.ema_scale is None:
+            self.ema_scale = cur
+        else:
+            self.ema_scale = decay * self.ema_scale + (np.float32(1.0) - decay) * cur
+        if len(self.scale_history) >= self.config.moving_average_window:
+            self.scale_history.pop(0)
+        self.scale_history.append(cur)
+        if self.step_count <= self.config.calibration_warmup:
+            if self.calibration_samples < self.config.calibration_warmup:
+                self.calibration_samples += 1
+        elif not self.calibrated:
+            self.calibrated = True
+        return self.ema_scale
+
+    def calibrate(self, abs_maxima: Sequence[float]):
+        """calibrate (:459-483): the scale becomes the abs-max at index floor(len * outlier_percentile / 100) of the sorted
+        list (the last one if that index is past the end)."""
+        import numpy as np
+        if len(abs_maxima) == 0:
+            raise BitLinearError(QUANTIZATION_ERROR, "Calibration data cannot be empty")
+        scales = sorted(np.float32(v) for v in abs_maxima)
+        idx = int(np.float32(len(scales)) * np.float32(self.config.outlier_percentile) / np.float32(100.0))
+        self.ema_scale = scales[min(idx, len(scales) - 1)]
+        self.calibrated = True
+
+    def needs_calibration(self) -> bool:
+        return (not self.calibrated) or self.step_count <= self.config.calibration_warmup
+
+    def reset(self):
+        self.scale_history.clear()
+        self.ema_scale = None
+        self.calibrated = False
+        self.step_count = 0
+        self.calibration_samples = 0
+
+
+def abs_max(x: torch.Tensor, stream=None) -> float:
+    """max |x| over the tensor, on the host (activations.abs().max_all().to_scalar())."""
+    _dev(x, torch.float32, "x")
+    out = C.c_float(0.0)
+    _check(load_library().bitnet_hip_abs_max(_ptr(x), x.numel(), C.byref(out), _stream(stream)))
+    return out.value
+
+
+def quantize_activations_scaled(x: torch.Tensor, precision: int, scale: float, reference_u8: bool = False, stream=None) -> torch.Tensor:
+    """DynamicActivationQuantizer::quantize with the scale given: int8 values (uint8 with reference_u8, the reference's
+    literal clamp(0, 255) of its 8-bit branch)."""
+    _dev(x, torch.float32, "x")
+    values = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    _check(load_library().bitnet_hip_quantize_activations_scaled(_ptr(x), x.numel(), precision, float(scale),
+                                                                 1 if reference_u8 else 0, _ptr(values), _stream(stream)))
+    return values.view(torch.uint8) if reference_u8 and precision == QuantizationPrecision.EightBit else values
+
+
+class DynamicActivationQuantizer:
+    """DynamicActivationQuantizer (activations.rs:203-454) over the HIP path: the tensor work (abs-max, quantisation with
+    the current scale) runs on the device, the state (DynamicScaleState) on the host as in the reference.
+    reference_u8: give the 8-bit values as the reference does (u8 after clamp(0, 255): negative activations become 0)
+    instead of signed int8."""
+
+    def __init__(self, config: Optional[ActivationQuantizationConfig] = None, reference_u8: bool = False):
+        self.config = config or ActivationQuantizationConfig()
+        self.state = DynamicScaleState(self.config)
+        self.reference_u8 = reference_u8
+
+    # -- Quantizer ------------------------------------------------------------------------------------------------
+    def validate_input(self, activations: torch.Tensor):
+        if activations.dim() < 1:
+            raise BitLinearError(QUANTIZATION_ERROR, "Activation tensor must have at least 1 dimension")
+        if activations.dtype not in (torch.float32, torch.float16):
+            raise BitLinearError(QUANTIZATION_ERROR, "Activation tensor must be float type")
+
+    validate_activations = validate_input
+
+    def quantize(self, activations: torch.Tensor) -> QuantizedActivation:
+        """quantize (:315-360): the moving-average scale if there is one, else the tensor's own abs-max."""
+        self.validate_input(activations)
+        if self.config.precision not in (QuantizationPrecision.OneFiveFiveBit, QuantizationPrecision.EightBit):
+            raise BitLinearError(UNSUPPORTED, f"UnsupportedPrecision({self.config.precision})")
+        x = activations if activations.dtype == torch.float32 else activations.float()
+        x = x.contiguous()
+        scale = float(self.state.ema_scale) if self.state.ema_scale is not None else abs_max(x)
+        values = quantize_activations_scaled(x, self.config.precision, scale, self.reference_u8)
+        bits = 1.58 if self.config.precision == QuantizationPrecision.OneFiveFiveBit else 8.0
+        stats = {"elements_count": activations.numel(), "scale_factor": scale, "compression_ratio": 32.0 / bits}
+        scales = torch.tensor([scale], dtype=torch.float32, device=activations.device)
+        return QuantizedActivation(values, scales, None, tuple(activations.shape), self.config.precision, stats)
+
+    def dequantize(self, quantized: QuantizedActivation) -> torch.Tensor:
+        """values * scales (:362-368); a convenience through torch, not on the forward path."""
+        return quantized.values.to(torch.float32) * quantized.scales
+
+    def get_stats(self) -> dict:
+        return {"elements_count": 0, "scale_factor": 1.0}  # the reference never updates the quantizer's own stats field
+
+    # -- ActivationQuantizer --------------------------------------------------------------------------------------
+    def quantize_dynamic(self, activations: torch.Tensor) -> QuantizedActivation:
+        self.state.step_count += 1
+        self.update_dynamic_params(activations)
+        return self.quantize(activations)
+
+    def quantize_attention(self, attention_scores: torch.Tensor, sequence_length: int) -> QuantizedActivation:
+        if not self.config.quantize_attention:
+            raise BitLinearError(QUANTIZATION_ERROR, "Attention quantization is disabled")
+        out = self.quantize(attention_scores)
+        out.sequence_length = sequence_length
+        return out
+
+    def update_dynamic_params(self, activations: torch.Tensor):
+        x = activations if activations.dtype == torch.float32 else activations.float()
+        self.state.update(abs_max(x.contiguous()))
+
+    def get_dynamic_scales(self) -> torch.Tensor:
+        return torch.tensor(float(self.state.ema_scale) if self.state.ema_scale is not None else 1.0, dtype=torch.float32)
+
+    def reset_dynamic_state(self):
+        self.state.reset()
+
+    # -- CalibrationQuantizer -------------------------------------------------------------------------------------
+    def calibrate(self, data: Sequence[torch.Tensor]):
+        self.state.calibrate([abs_max(t.float().contiguous()) for t in data])
+
+    def needs_calibration(self) -> bool:
+        return self.state.needs_calibration()
+
+    def reset_calibration(self):
+        self.reset_dynamic_state()
+
+
+def create_activation_quantizer(config: ActivationQuantizationConfig) -> DynamicActivationQuantizer:
+    """create_activation_quantizer (activations.rs:496-504): validates the configuration first."""
+    config.validate()
+    return DynamicActivationQuantizer(config)
 
 
 def packed_size(count: int) -> int:

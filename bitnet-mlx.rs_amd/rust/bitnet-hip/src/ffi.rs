@@ -68,6 +68,9 @@ extern "C" {
                                               a_sum: *mut i32, y_f32: *mut f32, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_absmax_quantize_activations(x: *const f32, count: usize, precision: c_int, values: *mut i8,
                                                   stats: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_abs_max(x: *const f32, count: usize, abs_max: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_quantize_activations_scaled(x: *const f32, count: usize, precision: c_int, scale: f32,
+                                                  reference_u8: c_int, values: *mut i8, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_lookup_compute(kind: c_int, weights: *const i8, n_weights: usize, inputs: *const f32,
                                      n_inputs: usize, output: *mut f32, n_output: usize, stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_packed_size(count: usize) -> usize;

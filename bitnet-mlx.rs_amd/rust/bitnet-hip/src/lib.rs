@@ -386,6 +386,293 @@ mod imp {
         pub fn optimal_batch_size(&self) -> usize { 1 << 20 }
     }
 
+    /// `QuantizationPrecision` values of the per-tensor activation quantisers (`BITNET_HIP_PRECISION_*`).
+    #[derive(Debug, Clone, Copy, PartialEq, Eq)]
+    pub enum HipPrecision {
+        OneFiveFiveBit,
+        EightBit,
+    }
+    impl HipPrecision {
+        fn code(self) -> c_int {
+            match self {
+                HipPrecision::OneFiveFiveBit => ffi::BITNET_HIP_PRECISION_ONE_FIVE_FIVE_BIT,
+                HipPrecision::EightBit => ffi::BITNET_HIP_PRECISION_EIGHT_BIT,
+            }
+        }
+        pub fn effective_bit_width(self) -> f32 {
+            match self {
+                HipPrecision::OneFiveFiveBit => 1.58,
+                HipPrecision::EightBit => 8.0,
+            }
+        }
+    }
+
+    /// What `absmax_quantize_activations` / `DynamicActivationQuantizer::quantize` return, in host memory: the signed
+    /// values, the one scale of the tensor and the statistics of `QuantizationStats` that the call fills.
+    #[derive(Debug, Clone)]
+    pub struct HipQuantizedActivation {
+        pub values: Vec<i8>,
+        pub scale: f32,
+        pub original_shape: Vec<usize>,
+        pub precision: HipPrecision,
+        pub quantization_error: f32,
+        pub min_value: f32,
+        pub max_value: f32,
+        pub sequence_length: Option<usize>,
+    }
+
+    /// `absmax_quantize_activations(&Tensor, &Device, Option<QuantizationPrecision>)`
+    /// (bitnet-quant/src/quantization/activations.rs:530-641) on the GPU: one scale per tensor.
+    pub fn absmax_quantize_activations(activations: &[f32], shape: &[usize], precision: Option<HipPrecision>) -> HipResult<HipQuantizedActivation> {
+        let precision = precision.unwrap_or(HipPrecision::OneFiveFiveBit);
+        if shape.iter().product::<usize>() != activations.len() {
+            return Err(HipError::ShapeMismatch { expected: shape.to_vec(), actual: vec![activations.len()] });
+        }
+        let mut x = DeviceBuffer::<f32>::new(activations.len())?;
+        x.upload(activations)?;
+        let q = DeviceBuffer::<i8>::new(activations.len().max(1))?;
+        let st = DeviceBuffer::<f32>::new(4)?;
+        check(unsafe {
+            ffi::bitnet_hip_absmax_quantize_activations(x.as_ptr(), activations.len(), precision.code(), q.as_ptr(), st.as_ptr(), ptr::null_mut())
+        })?;
+        let mut values = vec![0i8; activations.len()];
+        let mut stats = [0f32; 4];
+        q.download(&mut values)?;
+        st.download(&mut stats)?;
+        Ok(HipQuantizedActivation { values, scale: stats[0], original_shape: shape.to_vec(), precision, quantization_error: stats[1],
+                                    min_value: stats[2], max_value: stats[3], sequence_length: None })
+    }
+
+    /// `ActivationQuantizationConfig` (activations.rs:14-45) with its defaults.
+    #[derive(Debug, Clone)]
+    pub struct HipActivationQuantizationConfig {
+        pub precision: HipPrecision,
+        pub moving_average_window: usize,
+        pub outlier_percentile: f32,
+        pub per_token: bool,
+        pub calibration_warmup: usize,
+        pub ema_decay: f32,
+        pub quantize_attention: bool,
+    }
+    impl Default for HipActivationQuantizationConfig {
+        fn default() -> Self {
+            Self { precision: HipPrecision::OneFiveFiveBit, moving_average_window: 100, outlier_percentile: 99.9, per_token: false,
+                   calibration_warmup: 50, ema_decay: 0.99, quantize_attention: true }
+        }
+    }
+    impl HipActivationQuantizationConfig {
+        /// activations.rs:71-91
+        pub fn validate(&self) -> HipResult<()> {
+            if self.moving_average_window == 0 {
+                return Err(HipError::ConfigError("Moving average window cannot be zero".into()));
+            }
+            if self.outlier_percentile <= 0.0 || self.outlier_percentile > 100.0 {
+                return Err(HipError::ConfigError("Outlier percentile must be in range (0, 100]".into()));
+            }
+            if self.ema_decay < 0.0 || self.ema_decay > 1.0 {
+                return Err(HipError::ConfigError("EMA decay must be in range [0, 1]".into()));
+            }
+            Ok(())
+        }
+    }
+
+    /// `DynamicActivationQuantizer` (activations.rs:203-454): the state (moving average of the scale, window of recent
+    /// scales, warm-up counter, calibration flag) on the host in `f32`, as the reference keeps it; abs-max and the
+    /// quantisation with the current scale on the GPU (`bitnet_hip_abs_max`, `bitnet_hip_quantize_activations_scaled`).
+    #[derive(Debug)]
+    pub struct HipDynamicActivationQuantizer {
+        config: HipActivationQuantizationConfig,
+        scale_history: std::collections::VecDeque<f32>,
+        ema_scale: Option<f32>,
+        calibration_samples: usize,
+        calibrated: bool,
+        step_count: usize,
+    }
+    impl HipDynamicActivationQuantizer {
+        pub fn new(config: HipActivationQuantizationConfig) -> Self {
+            let window = config.moving_average_window;
+            Self { config, scale_history: std::collections::VecDeque::with_capacity(window), ema_scale: None, calibration_samples: 0,
+                   calibrated: false, step_count: 0 }
+        }
+        pub fn config(&self) -> &HipActivationQuantizationConfig { &self.config }
+        fn device_abs_max(x: &DeviceBuffer<f32>, len: usize) -> HipResult<f32> {
+            let mut m = 0f32;
+            check(unsafe { ffi::bitnet_hip_abs_max(x.as_ptr(), len, &mut m, ptr::null_mut()) })?;
+            Ok(m)
+        }
+        /// compute_dynamic_scale (:241-267)
+        fn compute_dynamic_scale(&mut self, abs_max: f32) -> f32 {
+            let current_scale = match self.config.precision {
+                HipPrecision::OneFiveFiveBit => abs_max / 1.0,
+                HipPrecision::EightBit => abs_max / 127.0,
+            };
+            self.ema_scale = Some(match self.ema_scale {
+                Some(prev) => self.config.ema_decay * prev + (1.0 - self.config.ema_decay) * current_scale,
+                None => current_scale,
+            });
+            if self.scale_history.len() >= self.config.moving_average_window {
+                self.scale_history.pop_front();
+            }
+            self.scale_history.push_back(current_scale);
+            self.ema_scale.unwrap()
+        }
+        fn quantize_buffer(&self, x: &DeviceBuffer<f32>, host: &[f32], shape: &[usize]) -> HipResult<HipQuantizedActivation> {
+            if shape.is_empty() {
+                return Err(HipError::QuantizationError("Activation tensor must have at least 1 dimension".into()));
+            }
+            let scale = match self.ema_scale {
+                Some(s) => s,
+                None => Self::device_abs_max(x, host.len())?,
+            };
+            let q = DeviceBuffer::<i8>::new(host.len().max(1))?;
+            check(unsafe {
+                ffi::bitnet_hip_quantize_activations_scaled(x.as_ptr(), host.len(), self.config.precision.code(), scale, 0, q.as_ptr(), ptr::null_mut())
+            })?;
+            let mut values = vec![0i8; host.len()];
+            q.download(&mut values)?;
+            Ok(HipQuantizedActivation { values, scale, original_shape: shape.to_vec(), precision: self.config.precision,
+                                        quantization_error: 0.0, min_value: 0.0, max_value: 0.0, sequence_length: None })
+        }
+        fn upload(host: &[f32], shape: &[usize]) -> HipResult<DeviceBuffer<f32>> {
+            if shape.iter().product::<usize>() != host.len() {
+                return Err(HipError::ShapeMismatch { expected: shape.to_vec(), actual: vec![host.len()] });
+            }
+            let mut x = DeviceBuffer::<f32>::new(host.len())?;
+            x.upload(host)?;
+            Ok(x)
+        }
+        /// quantize (:315-360): the moving-average scale if there is one, else the tensor's own abs-max.
+        pub fn quantize(&self, activations: &[f32], shape: &[usize]) -> HipResult<HipQuantizedActivation> {
+            let x = Self::upload(activations, shape)?;
+            self.quantize_buffer(&x, activations, shape)
+        }
+        /// quantize_dynamic (:372-383)
+        pub fn quantize_dynamic(&mut self, activations: &[f32], shape: &[usize]) -> HipResult<HipQuantizedActivation> {
+            self.step_count += 1;
+            let x = Self::upload(activations, shape)?;
+            let abs_max = Self::device_abs_max(&x, activations.len())?;
+            self.update_with_abs_max(abs_max);
+            self.quantize_buffer(&x, activations, shape)
+        }
+        /// quantize_attention (:385-404)
+        pub fn quantize_attention(&self, attention_scores: &[f32], shape: &[usize], sequence_length: usize) -> HipResult<HipQuantizedActivation> {
+            if !self.config.quantize_attention {
+                return Err(HipError::QuantizationError("Attention quantization is disabled".into()));
+            }
+            let mut result = self.quantize(attention_scores, shape)?;
+            result.sequence_length = Some(sequence_length);
+            Ok(result)
+        }
+        /// update_dynamic_params (:406-433) for a tensor whose max |x| is `abs_max`.
+        fn update_with_abs_max(&mut self, abs_max: f32) {
+            let _scale = self.compute_dynamic_scale(abs_max);
+            if self.step_count <= self.config.calibration_warmup {
+                if self.calibration_samples < self.config.calibration_warmup {
+                    self.calibration_samples += 1;
+                }
+            } else if !self.calibrated {
+                self.calibrated = true;
+            }
+        }
+        pub fn update_dynamic_params(&mut self, activations: &[f32], shape: &[usize]) -> HipResult<()> {
+            let x = Self::upload(activations, shape)?;
+            let abs_max = Self::device_abs_max(&x, activations.len())?;
+            self.update_with_abs_max(abs_max);
+            Ok(())
+        }
+        pub fn get_dynamic_scales(&self) -> f32 { self.ema_scale.unwrap_or(1.0) }
+        pub fn reset_dynamic_state(&mut self) {
+            self.scale_history.clear();
+            self.ema_scale = None;
+            self.calibration_samples = 0;
+            self.calibrated = false;
+            self.step_count = 0;
+        }
+        /// calibrate (:459-483): the abs-max at index floor(len * outlier_percentile / 100) of the sorted list.
+        pub fn calibrate(&mut self, data: &[(&[f32], &[usize])]) -> HipResult<()> {
+            if data.is_empty() {
+                return Err(HipError::QuantizationError("Calibration data cannot be empty".into()));
+            }
+            let mut all_scales = Vec::with_capacity(data.len());
+            for (host, shape) in data {
+                let x = Self::upload(host, shape)?;
+                all_scales.push(Self::device_abs_max(&x, host.len())?);
+            }
+            all_scales.sort_by(|a, b| a.partial_cmp(b).unwrap());
+            let percentile_idx = (all_scales.len() as f32 * self.config.outlier_percentile / 100.0) as usize;
+            self.ema_scale = Some(all_scales[percentile_idx.min(all_scales.len() - 1)]);
+            self.calibrated = true;
+            Ok(())
+        }
+        pub fn needs_calibration(&self) -> bool { !self.calibrated || self.step_count <= self.config.calibration_warmup }
+    }
+
+    /// `WeightQuantizationConfig`'s arithmetic-relevant fields (weights.rs:58-95) with their defaults.
+    #[derive(Debug, Clone)]
+    pub struct HipWeightQuantizationConfig {
+        /// TernaryMethod as 0 MeanThreshold, 1 MedianThreshold, 2 AdaptiveThreshold, 3 OptimalThreshold, 4 DetSTE
+        pub ternary_method: c_int,
+        pub normalize_weights: bool,
+        pub outlier_threshold: f32,
+        pub custom_threshold_factor: Option<f32>,
+    }
+    impl Default for HipWeightQuantizationConfig {
+        fn default() -> Self {
+            Self { ternary_method: 0, normalize_weights: true, outlier_threshold: 3.0, custom_threshold_factor: None }
+        }
+    }
+    /// What `BitNetWeightQuantizer::quantize` returns, in host memory: ternary values, the reference's 2-bit bytes, the
+    /// least-squares scale and the twelve statistics of the pipeline (see `bitnet_hip_quantize_weights_reference`).
+    #[derive(Debug, Clone)]
+    pub struct HipQuantizedWeight {
+        pub values: Vec<i8>,
+        pub packed: Vec<u8>,
+        pub scale: f32,
+        pub original_shape: [usize; 2],
+        pub stats: [f32; 12],
+    }
+    /// `BitNetWeightQuantizer` (weights.rs:341-611) on the GPU: normalise, clip, ternarise by the configured method,
+    /// least-squares scale.
+    #[derive(Debug, Clone, Default)]
+    pub struct HipWeightQuantizer {
+        config: HipWeightQuantizationConfig,
+    }
+    impl HipWeightQuantizer {
+        pub fn new(config: HipWeightQuantizationConfig) -> Self { Self { config } }
+        pub fn config(&self) -> &HipWeightQuantizationConfig { &self.config }
+        pub fn quantize(&self, weights: &[f32], rows: usize, cols: usize) -> HipResult<HipQuantizedWeight> {
+            if rows * cols != weights.len() {
+                return Err(HipError::ShapeMismatch { expected: vec![rows, cols], actual: vec![weights.len()] });
+            }
+            let mut w = DeviceBuffer::<f32>::new(weights.len())?;
+            w.upload(weights)?;
+            let n_packed = (weights.len() + 3) / 4;
+            let packed = DeviceBuffer::<u8>::new(n_packed.max(1))?;
+            let q = DeviceBuffer::<i8>::new(weights.len().max(1))?;
+            let scale = DeviceBuffer::<f32>::new(1)?;
+            let stats = DeviceBuffer::<f32>::new(12)?;
+            check(unsafe {
+                ffi::bitnet_hip_quantize_weights_reference(w.as_ptr(), rows, cols, self.config.ternary_method,
+                    self.config.normalize_weights as c_int, self.config.outlier_threshold,
+                    self.config.custom_threshold_factor.unwrap_or(0.0), packed.as_ptr(), scale.as_ptr(), q.as_ptr(), stats.as_ptr(),
+                    ptr::null_mut())
+            })?;
+            let mut out = HipQuantizedWeight { values: vec![0i8; weights.len()], packed: vec![0u8; n_packed], scale: 0.0,
+                                               original_shape: [rows, cols], stats: [0f32; 12] };
+            q.download(&mut out.values)?;
+            packed.download(&mut out.packed)?;
+            let mut s = [0f32; 1];
+            scale.download(&mut s)?;
+            out.scale = s[0];
+            stats.download(&mut out.stats)?;
+            Ok(out)
+        }
+        /// dequantize (weights.rs:613-626): values * scale.
+        pub fn dequantize(&self, quantized: &HipQuantizedWeight) -> Vec<f32> {
+            quantized.values.iter().map(|v| *v as f32 * quantized.scale).collect()
+        }
+    }
+
     /// The seven BitLinear projections of a stack of decoder blocks (bitnet_hip_decoder_*).
     pub struct HipDecoder {
         pub(crate) handle: *mut ffi::bitnet_hip_decoder,
@@ -410,6 +697,17 @@ mod imp {
             let mut bl = ptr::null_mut();
             check(unsafe { ffi::bitnet_hip_decoder_projection(self.handle, layer, proj, &mut bl) })?;
             check(unsafe { ffi::bitnet_hip_bitlinear_set_weights_packed(bl, packed.as_ptr(), packed.len(), w_scale, 0, ptr::null_mut()) })
+        }
+        /// A whole GGUF tensor of type BitnetB158 (8-byte scale / offset header + 2-bit codes; gguf.rs:1089-1165) as the
+        /// weights of projection `proj` of block `layer`; `transposed`: the tensor is [in, out] (inference_integration.rs:431).
+        pub fn set_projection_gguf(&self, layer: usize, proj: c_int, data: &[u8], rows: usize, cols: usize, transposed: bool) -> HipResult<()> {
+            let mut bl = ptr::null_mut();
+            check(unsafe { ffi::bitnet_hip_decoder_projection(self.handle, layer, proj, &mut bl) })?;
+            let layout = if transposed { ffi::BITNET_HIP_LAYOUT_IN_OUT } else { ffi::BITNET_HIP_LAYOUT_OUT_IN };
+            check(unsafe {
+                ffi::bitnet_hip_bitlinear_set_weights_gguf(bl, data.as_ptr(), data.len(), rows, cols, layout, 0, ptr::null_mut(), ptr::null_mut(),
+                                                           ptr::null_mut())
+            })
         }
         /// Row groups a step of several token rows is split into, each a chain of launches on its own stream
         /// (0 and 1 = one chain, the default).
@@ -485,7 +783,9 @@ mod imp {
             check(unsafe { ffi::bitnet_hip_backend_create(device, &mut handle) })?;
             Ok(Self { handle, model: None, staging: Mutex::new((DeviceBuffer::new(0)?, DeviceBuffer::new(0)?)) })
         }
-        /// Binds the decoder stack `execute_batch` runs (what `optimize_model` does once a model's weights are in it).
+        /// The decoder bound by `bind_decoder` / `optimize_model`, if any.
+        pub fn bound_decoder(&self) -> Option<&std::sync::Arc<HipDecoder>> { self.model.as_ref() }
+        /// Binds the decoder stack `execute_batch` runs (what `optimize_model` does for the stack it builds from a `Model`).
         pub fn bind_decoder(&mut self, model: std::sync::Arc<HipDecoder>) -> HipResult<()> {
             check(unsafe { ffi::bitnet_hip_backend_optimize_model(self.handle, model.handle) })?;
             self.model = Some(model);
@@ -583,7 +883,10 @@ mod reference_traits {
     use bitnet_inference::engine::{BackendCapabilities, InferenceBackend, Model};
     use bitnet_quant::bitlinear::error::{BitLinearError, BitLinearResult};
     use bitnet_quant::bitlinear::forward::BitLinearForward;
-    use bitnet_quant::quantization::weights::QuantizedWeight;
+    use bitnet_quant::quantization::activations::{ActivationQuantizationConfig, QuantizedActivation};
+    use bitnet_quant::quantization::utils::QuantizationError;
+    use bitnet_quant::quantization::weights::{QuantizedWeight, TernaryMethod, WeightQuantizationConfig};
+    use bitnet_quant::quantization::{QuantizationPrecision, QuantizationStats, Quantizer};
     use candle_core::{Device, Tensor};
 
     fn to_bitlinear_error(e: HipError) -> BitLinearError {
@@ -650,6 +953,185 @@ mod reference_traits {
         fn optimal_batch_size(&self) -> usize { HipLookupKernel::optimal_batch_size(self) }
     }
 
+    /// The decoder stack a `Model` describes: the BitLinear layers of `ModelArchitecture::BitLinear` in groups of seven
+    /// (q, k, v, o, gate, up, down), all hidden -> hidden except k / v (hidden -> kv_heads * head_dim), gate / up
+    /// (hidden -> ffn) and down (ffn -> hidden); the RMSNorm layers give eps.
+    struct DecoderShape {
+        blocks: usize, hidden: usize, ffn: usize, heads: usize, kv_heads: usize, head_dim: usize, eps: f32, max_tokens: usize,
+    }
+    fn decoder_shape_of(model: &Model) -> HipResult<DecoderShape> {
+        use bitnet_inference::engine::{LayerParameters, LayerType, ModelArchitecture};
+        let (layers, heads, hidden) = match &model.architecture {
+            ModelArchitecture::BitLinear { layers, attention_heads, hidden_dim } => (layers, *attention_heads, *hidden_dim),
+            other => return Err(HipError::UnsupportedOperation(format!(
+                "optimize_model: only ModelArchitecture::BitLinear maps onto the decoder stack (got {other:?}); bind a decoder with bind_decoder"))),
+        };
+        let bitlinear: Vec<_> = layers.iter().filter(|l| matches!(l.layer_type, LayerType::BitLinear)).collect();
+        if bitlinear.is_empty() || bitlinear.len() % 7 != 0 {
+            return Err(HipError::UnsupportedOperation(format!(
+                "optimize_model: {} BitLinear layers are not whole blocks of seven projections; bind a decoder with bind_decoder", bitlinear.len())));
+        }
+        let last = |shape: &Vec<usize>| shape.last().copied().unwrap_or(0);
+        let (kv_dim, ffn) = (last(&bitlinear[1].output_shape), last(&bitlinear[4].output_shape));
+        let heads = heads.ok_or_else(|| HipError::ConfigError("optimize_model: the architecture names no attention heads".into()))?;
+        if heads == 0 || hidden % heads != 0 || kv_dim == 0 || ffn == 0 {
+            return Err(HipError::ConfigError(format!("optimize_model: hidden {hidden}, heads {heads}, kv width {kv_dim}, ffn {ffn}")));
+        }
+        let head_dim = hidden / heads;
+        for (i, l) in bitlinear.iter().enumerate() {
+            let want = match i % 7 { 1 | 2 => (hidden, kv_dim), 4 | 5 => (hidden, ffn), 6 => (ffn, hidden), _ => (hidden, hidden) };
+            if (last(&l.input_shape), last(&l.output_shape)) != want {
+                return Err(HipError::ShapeMismatch { expected: vec![want.0, want.1], actual: vec![last(&l.input_shape), last(&l.output_shape)] });
+            }
+        }
+        let eps = layers.iter().find_map(|l| match l.parameters { LayerParameters::RMSNorm { eps } => Some(eps), _ => None }).unwrap_or(1e-5);
+        Ok(DecoderShape { blocks: bitlinear.len() / 7, hidden, ffn, heads, kv_heads: kv_dim / head_dim, head_dim, eps, max_tokens: 16 })
+    }
+
+    impl HipInferenceBackend {
+        /// One projection's weights as the GGUF file holds them (type BitnetB158: scale, offset, 2-bit codes;
+        /// `decode_ternary_weights`, gguf.rs:1089-1165), into the decoder `optimize_model` built.  `transposed`: the
+        /// tensor is [in, out] (inference_integration.rs:431).
+        pub fn load_projection_gguf(&self, block: usize, proj: c_int, data: &[u8], rows: usize, cols: usize, transposed: bool) -> HipResult<()> {
+            let model = self.bound_decoder().ok_or_else(|| HipError::NotInitialized("no model bound: call optimize_model first".into()))?;
+            model.set_projection_gguf(block, proj, data, rows, cols, transposed)
+        }
+    }
+
+    fn to_quantization_error(e: HipError) -> QuantizationError {
+        match e {
+            HipError::ShapeMismatch { expected, actual } => QuantizationError::InvalidInput(format!("expected {expected:?}, got {actual:?}")),
+            HipError::ConfigError(m) => QuantizationError::ConfigurationError(m),
+            HipError::MemoryError(m) => QuantizationError::MemoryError(m),
+            HipError::QuantizationError(m) => QuantizationError::InvalidInput(m),
+            HipError::UnsupportedOperation(m) => QuantizationError::UnsupportedPrecision(m),
+            other => QuantizationError::DeviceError(other.to_string()),
+        }
+    }
+
+    /// `BitNetWeightQuantizer` behind the reference's `Quantizer` trait (quantization/mod.rs:96-116): the pipeline runs on
+    /// the GPU (`bitnet_hip_quantize_weights_reference`), tensors cross as host memory.
+    #[derive(Debug)]
+    pub struct HipBitNetWeightQuantizer {
+        config: WeightQuantizationConfig,
+        inner: HipWeightQuantizer,
+        stats: std::sync::Mutex<QuantizationStats>,
+    }
+    impl HipBitNetWeightQuantizer {
+        pub fn new(config: WeightQuantizationConfig) -> Self {
+            let method = match config.ternary_method {
+                TernaryMethod::MeanThreshold => 0,
+                TernaryMethod::MedianThreshold => 1,
+                TernaryMethod::AdaptiveThreshold => 2,
+                TernaryMethod::OptimalThreshold => 3,
+                TernaryMethod::DetSTE => 4,
+            };
+            let inner = HipWeightQuantizer::new(HipWeightQuantizationConfig { ternary_method: method, normalize_weights: config.normalize_weights,
+                outlier_threshold: config.outlier_threshold, custom_threshold_factor: config.custom_threshold_factor });
+            Self { config, inner, stats: std::sync::Mutex::new(QuantizationStats::default()) }
+        }
+    }
+    impl Quantizer for HipBitNetWeightQuantizer {
+        type Input = Tensor;
+        type Output = QuantizedWeight;
+        type Config = WeightQuantizationConfig;
+        type Error = QuantizationError;
+
+        fn quantize(&self, weights: &Tensor) -> Result<QuantizedWeight, QuantizationError> {
+            self.validate_input(weights)?;
+            let dims = weights.dims().to_vec();
+            let cols = *dims.last().unwrap();
+            let rows = dims[..dims.len() - 1].iter().product();
+            let flat = weights.to_dtype(candle_core::DType::F32)?.flatten_all()?.to_vec1::<f32>()?;
+            let q = self.inner.quantize(&flat, rows, cols).map_err(to_quantization_error)?;
+            let values: Vec<f32> = q.values.iter().map(|v| *v as f32).collect();
+            let stats = QuantizationStats { elements_count: flat.len(), scale_factor: q.scale, compression_ratio: 32.0 / 1.58,
+                                            min_value: q.stats[4], max_value: q.stats[5], ..Default::default() };
+            *self.stats.lock().unwrap() = stats.clone();
+            Ok(QuantizedWeight::new(Tensor::from_vec(values, dims.clone(), &Device::Cpu)?, Tensor::new(q.scale, &Device::Cpu)?, None,
+                                    weights.shape().clone(), candle_core::DType::U8, self.config.clone(), stats))
+        }
+        fn dequantize(&self, quantized: &QuantizedWeight) -> Result<Tensor, QuantizationError> {
+            Ok(quantized.values.broadcast_mul(&quantized.scales)?)
+        }
+        fn config(&self) -> &WeightQuantizationConfig { &self.config }
+        fn validate_input(&self, weights: &Tensor) -> Result<(), QuantizationError> {
+            if weights.rank() < 2 {
+                return Err(QuantizationError::InvalidInput("Weight tensor must have at least 2 dimensions".to_string()));
+            }
+            if weights.dtype() != candle_core::DType::F32 && weights.dtype() != candle_core::DType::F16 {
+                return Err(QuantizationError::InvalidInput("Weight tensor must be float type".to_string()));
+            }
+            Ok(())
+        }
+        fn get_stats(&self) -> QuantizationStats { self.stats.lock().unwrap().clone() }
+    }
+
+    /// `DynamicActivationQuantizer` behind the `Quantizer` trait (activations.rs:303-370): `quantize` uses the moving-average
+    /// scale held by the wrapped `HipDynamicActivationQuantizer` (or the tensor's own abs-max), on the GPU.
+    #[derive(Debug)]
+    pub struct HipActivationQuantizerAdapter {
+        config: ActivationQuantizationConfig,
+        pub inner: HipDynamicActivationQuantizer,
+    }
+    impl HipActivationQuantizerAdapter {
+        pub fn new(config: ActivationQuantizationConfig) -> Result<Self, QuantizationError> {
+            let precision = match config.base.precision {
+                QuantizationPrecision::OneFiveFiveBit => HipPrecision::OneFiveFiveBit,
+                QuantizationPrecision::EightBit => HipPrecision::EightBit,
+                other => return Err(QuantizationError::UnsupportedPrecision(format!("{other:?}"))),
+            };
+            let inner = HipDynamicActivationQuantizer::new(HipActivationQuantizationConfig { precision,
+                moving_average_window: config.moving_average_window, outlier_percentile: config.outlier_percentile,
+                per_token: config.per_token, calibration_warmup: config.calibration_warmup, ema_decay: config.ema_decay,
+                quantize_attention: config.quantize_attention });
+            Ok(Self { config, inner })
+        }
+        /// quantize_dynamic of the ActivationQuantizer trait (activations.rs:372-383)
+        pub fn quantize_dynamic(&mut self, activations: &Tensor) -> Result<QuantizedActivation, QuantizationError> {
+            self.validate_input(activations)?;
+            let dims = activations.dims().to_vec();
+            let flat = activations.to_dtype(candle_core::DType::F32)?.flatten_all()?.to_vec1::<f32>()?;
+            let q = self.inner.quantize_dynamic(&flat, &dims).map_err(to_quantization_error)?;
+            self.wrap(q, activations)
+        }
+        fn wrap(&self, q: HipQuantizedActivation, activations: &Tensor) -> Result<QuantizedActivation, QuantizationError> {
+            let values: Vec<f32> = q.values.iter().map(|v| *v as f32).collect();
+            let stats = QuantizationStats { elements_count: values.len(), scale_factor: q.scale,
+                                            compression_ratio: 32.0 / q.precision.effective_bit_width(), ..Default::default() };
+            Ok(QuantizedActivation::new(Tensor::from_vec(values, q.original_shape.clone(), &Device::Cpu)?, Tensor::new(q.scale, &Device::Cpu)?,
+                                        None, activations.shape().clone(), candle_core::DType::U8, self.config.clone(), stats, q.sequence_length))
+        }
+    }
+    impl Quantizer for HipActivationQuantizerAdapter {
+        type Input = Tensor;
+        type Output = QuantizedActivation;
+        type Config = ActivationQuantizationConfig;
+        type Error = QuantizationError;
+
+        fn quantize(&self, activations: &Tensor) -> Result<QuantizedActivation, QuantizationError> {
+            self.validate_input(activations)?;
+            let dims = activations.dims().to_vec();
+            let flat = activations.to_dtype(candle_core::DType::F32)?.flatten_all()?.to_vec1::<f32>()?;
+            let q = self.inner.quantize(&flat, &dims).map_err(to_quantization_error)?;
+            self.wrap(q, activations)
+        }
+        fn dequantize(&self, quantized: &QuantizedActivation) -> Result<Tensor, QuantizationError> {
+            Ok(quantized.values.to_dtype(candle_core::DType::F32)?.broadcast_mul(&quantized.scales)?)
+        }
+        fn config(&self) -> &ActivationQuantizationConfig { &self.config }
+        fn validate_input(&self, activations: &Tensor) -> Result<(), QuantizationError> {
+            if activations.rank() < 1 {
+                return Err(QuantizationError::InvalidInput("Activation tensor must have at least 1 dimension".to_string()));
+            }
+            if activations.dtype() != candle_core::DType::F32 && activations.dtype() != candle_core::DType::F16 {
+                return Err(QuantizationError::InvalidInput("Activation tensor must be float type".to_string()));
+            }
+            Ok(())
+        }
+        fn get_stats(&self) -> QuantizationStats { QuantizationStats::default() }
+    }
+
     impl InferenceBackend for HipInferenceBackend {
         fn execute_batch(&self, inputs: &[Tensor]) -> bitnet_inference::Result<Vec<Tensor>> {
             let mut host = Vec::with_capacity(inputs.len());
@@ -665,14 +1147,17 @@ mod reference_traits {
                     .map_err(|e| bitnet_inference::InferenceError::backend(e.to_string())))
                 .collect()
         }
+        /// Builds the decoder stack the model's architecture describes and binds it, as the CPU backend builds its
+        /// computation graph from the same description (cpu_backend.rs:116-160, 253-260).  A `Model` carries no
+        /// tensors (engine/mod.rs:191-206): the weights follow through `load_projection_gguf`, one BitnetB158 tensor
+        /// per projection, straight from the bytes `GgufLoader` holds (gguf.rs:1089-1165).  A decoder bound earlier
+        /// with `bind_decoder` is replaced.
         fn optimize_model(&mut self, model: &Model) -> bitnet_inference::Result<()> {
-            let _ = model;
-            // the weights reach the device through bind_decoder (the loader that fills a HipDecoder from a Model is the
-            // GGUF path's job); the trait call only confirms that a model is bound
-            if self.capabilities().map(|c| c.max_batch_size).unwrap_or(0) == 0 {
-                return Err(bitnet_inference::InferenceError::backend("no decoder bound: call bind_decoder first"));
-            }
-            Ok(())
+            let shape = decoder_shape_of(model).map_err(|e| bitnet_inference::InferenceError::backend(e.to_string()))?;
+            let decoder = HipDecoder::new(shape.blocks, shape.hidden, shape.ffn, shape.heads, shape.kv_heads, shape.head_dim, shape.eps,
+                                          SumOrder::Block256, shape.max_tokens)
+                .map_err(|e| bitnet_inference::InferenceError::backend(e.to_string()))?;
+            self.bind_decoder(std::sync::Arc::new(decoder)).map_err(|e| bitnet_inference::InferenceError::backend(e.to_string()))
         }
         fn get_memory_usage(&self) -> usize { HipInferenceBackend::get_memory_usage(self) }
         fn capabilities(&self) -> BackendCapabilities {
@@ -682,7 +1167,10 @@ mod reference_traits {
                 supports_streaming: false,
                 max_batch_size: c.as_ref().map_or(0, |c| c.max_batch_size),
                 memory_limit: c.as_ref().and_then(|c| c.memory_limit),
-                device_type: bitnet_inference::Device::Cpu,  // the reference's Device enum has no HIP variant; tensors cross as host memory
+                // `Device` here is candle's enum (Cpu, Cuda, Metal; bitnet-core re-exports it): it has no variant for this
+                // device and its GPU variants cannot be built without that runtime, so the field names where the trait's
+                // tensors live (host memory).  The GPU is `HipInferenceBackend::capabilities()?.device` (an ordinal).
+                device_type: bitnet_inference::Device::Cpu,
             }
         }
     }

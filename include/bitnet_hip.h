@@ -139,6 +139,18 @@ int bitnet_hip_quantize_activations_i8(const float *x, const float *x2, size_t l
  *   The per-token int8 quantiser of the BitLinear path is bitnet_hip_quantize_activations_i8, not this function. */
 int bitnet_hip_absmax_quantize_activations(const float *x, size_t count, int precision, int8_t *values, float *stats,
                                            void *stream);
+/* The two device steps of DynamicActivationQuantizer (bitnet-quant/src/quantization/activations.rs:203-454), whose
+ * state (exponential moving average of the scale, history window, warm-up counter) lives on the host, where the
+ * reference keeps it:
+ *   bitnet_hip_abs_max: max |x| over the tensor into *abs_max, a HOST float; waits for the stream, as
+ *     activations.abs().max_all().to_scalar() does (compute_dynamic_scale, :241-267; calibrate, :472-475).
+ *   bitnet_hip_quantize_activations_scaled: DynamicActivationQuantizer::quantize with the scale given
+ *     (quantize_int8 :269-275, quantize_ternary_activation :277-294): y = x * (float)(1.0 / (double)scale);
+ *     ternary +1 / -1 beyond +-0.5; 8-bit round(clamp(y, -127, 127)) as int8, or with reference_u8 != 0 the reference's
+ *     literal clamp(0, 255).round() stored as the byte of a u8 (it zeroes every negative activation).  NaN gives 0. */
+int bitnet_hip_abs_max(const float *x, size_t count, float *abs_max, void *stream);
+int bitnet_hip_quantize_activations_scaled(const float *x, size_t count, int precision, float scale, int reference_u8,
+                                           int8_t *values, void *stream);
 
 /* ---- lookup-table kernels --------------------------------------------------------------------- */
 

@@ -25,6 +25,10 @@
  *                                        for [4,-2,1,-3], signs of [3,-3,0.1,-0.1], zeros, statistics) + an
  *                                        independent numpy model; the U8 cast of the 8-bit branch is a reference
  *                                        defect that is not reproduced
+ *   orc_abs_max / orc_quantize_activations_scaled   pinned: the reference's dynamic-quantizer tests (ternary values
+ *                                        only, scale grows with the magnitude, a reset quantizer scales by the tensor's
+ *                                        own abs-max) + closed forms (scale = abs_max / 127 puts the extreme at 127,
+ *                                        exact halves, the u8 form equals max(signed, 0) below 128) + a numpy model
  *   orc_rmsnorm                          the reference holds NO fixture: pinned by closed forms (constant
  *                                        rows, one-hot rows), scale equivariance and an f64 bound; the
  *                                        bits of the ORC_SUM_BLOCK256 order are a declaration of this build
@@ -194,6 +198,39 @@ void orc_rmsnorm_quantize_i8(const float *x, const float *g, float eps, size_t m
  * consecutive elements in the order of orc_tensor_sum_f64 (elements past the end count as +0) and rounded once.
  * stats receives 4 floats. */
 static double orc_tensor_sum_f64(const float *v, size_t rows, size_t cols);
+/* DynamicActivationQuantizer (bitnet-quant/src/quantization/activations.rs:203-454), the two tensor steps:
+ *   orc_abs_max: activations.abs().max_all() (:242, :473), a fold of fmaxf from 0.
+ *   orc_quantize_activations_scaled: quantize() with the scale it is given (:315-360): candle's affine(1.0 / scale as f64,
+ *   0.0) multiplies every f32 element by (float)(1.0 / (double)scale); quantize_int8 (:269-275) then clamps to [0, 255],
+ *   rounds (halves away from zero) and casts to u8, which zeroes every negative value: reference_u8 reproduces that
+ *   literally, the signed form clamps to [-127, 127] instead (the form the HIP path hands on);
+ *   quantize_ternary_activation (:277-294) is +1 above 0.5, -1 below -0.5.  NaN gives 0 (a saturating cast). */
+float orc_abs_max(const float *x, size_t n)
+{
+    float m = 0.0f;
+    for (size_t i = 0; i < n; ++i) m = fmaxf(m, fabsf(x[i]));
+    return m;
+}
+
+void orc_quantize_activations_scaled(const float *x, size_t n, int precision, float scale, int reference_u8, int8_t *q)
+{
+    float recip = (float)(1.0 / (double)scale);
+    for (size_t i = 0; i < n; ++i) {
+        float y = x[i] * recip;
+        int v;
+        if (precision == 1) {
+            float lo = reference_u8 ? 0.0f : -127.0f, hi = reference_u8 ? 255.0f : 127.0f;
+            float c = y > hi ? hi : y;
+            c = c < lo ? lo : c;
+            float r = roundf(c);
+            v = (r != r) ? 0 : (int)r;
+        } else {
+            v = y > 0.5f ? 1 : (y < -0.5f ? -1 : 0);
+        }
+        q[i] = (int8_t)(uint8_t)(unsigned)v;
+    }
+}
+
 void orc_absmax_quantize_activations(const float *x, size_t n, int precision, int8_t *q, float *stats)
 {
     float abs_max = 0.0f, lo = INFINITY, hi = -INFINITY;

@@ -32,6 +32,7 @@ def lib() -> C.CDLL:
         _lib = C.CDLL(str(LIB_PATH))
         _lib.orc_sum_squares.restype = C.c_float
         _lib.orc_absmean.restype = C.c_float
+        _lib.orc_abs_max.restype = C.c_float
         _lib.orc_round_clip.restype = C.c_float
         _lib.orc_quantize_weights_reference.restype = C.c_float
         _lib.orc_pack_2bit.restype = C.c_size_t
@@ -77,6 +78,20 @@ def quantize_activations_i8(x):
     rs = np.empty((m,), dtype=np.int32)
     lib().orc_quantize_activations_i8(_p(x), _sz(m), _sz(k), _p(q), _p(s), _p(rs))
     return q, s, rs
+
+
+def abs_max(x):
+    x = _f32(x)
+    return np.float32(lib().orc_abs_max(_p(x), _sz(x.size)))
+
+
+def quantize_activations_scaled(x, precision, scale, reference_u8=False):
+    """DynamicActivationQuantizer::quantize with a given scale: int8 values (the u8 bytes viewed as int8 with reference_u8)."""
+    x = _f32(x)
+    q = np.empty(x.shape, dtype=np.int8)
+    lib().orc_quantize_activations_scaled(_p(x), _sz(x.size), C.c_int(precision), C.c_float(scale),
+                                          C.c_int(1 if reference_u8 else 0), _p(q))
+    return q
 
 
 def fake_quantize_activations(x):

@@ -187,6 +187,62 @@ def test_absmax_quantize_activations_bit_exact(precision, shape):
     assert ei.value.kind == "Unsupported"
 
 
+@pytest.mark.parametrize("precision", [bh.QuantizationPrecision.OneFiveFiveBit, bh.QuantizationPrecision.EightBit])
+@pytest.mark.parametrize("shape", [(5,), (32, 128), (3, 5, 7), (300, 4096 + 17), (1, 1)])
+def test_dynamic_activation_quantizer_matches_the_oracle(precision, shape):
+    """DynamicActivationQuantizer (activations.rs:203-454) on the device: abs-max and the quantiser with a given scale
+    bit-equal to the oracle (signed and the reference's literal u8 form), and the stateful object step by step against
+    the oracle driven by the same state machine: the moving average after every quantize_dynamic, the values it yields,
+    reset, calibration, attention, and the reference's own assertions (ternary values only for the default precision,
+    the scale grows with the magnitude, a reset quantizer scales by the tensor's own abs-max)."""
+    rng = np.random.default_rng(len(shape) * 7 + precision)
+    x = (rng.standard_normal(shape) * 3).astype(f32)
+    assert f32(bh.abs_max(dev(x))) == orc.abs_max(x)
+    for scale in (float(orc.abs_max(x)) / 127.0, 0.037, 1.0, 2.5):
+        for u8 in (False, True):
+            got = bh.quantize_activations_scaled(dev(x), precision, scale, reference_u8=u8)
+            want = orc.quantize_activations_scaled(x, precision, scale, reference_u8=u8)
+            assert np.array_equal(host(got).view(np.int8), want)
+    cfg = bh.ActivationQuantizationConfig(precision=precision, ema_decay=0.8, calibration_warmup=2, moving_average_window=4)
+    quant = bh.create_activation_quantizer(cfg)
+    model = bh.DynamicScaleState(cfg)
+    first = quant.quantize(dev(x))  # no state yet: the tensor's own abs-max is the scale
+    assert f32(first.stats["scale_factor"]) == orc.abs_max(x)
+    assert np.array_equal(host(first.values), orc.quantize_activations_scaled(x, precision, float(orc.abs_max(x))))
+    scales = []
+    for step, mag in enumerate((0.1, 1.0, 10.0, 3.0, 0.5)):
+        xs = (x * f32(mag)).astype(f32)
+        out = quant.quantize_dynamic(dev(xs))
+        model.step_count += 1
+        ema = model.update(orc.abs_max(xs))
+        assert f32(out.stats["scale_factor"]) == ema == quant.state.ema_scale
+        assert np.array_equal(host(out.values), orc.quantize_activations_scaled(xs, precision, float(ema)))
+        assert out.original_shape == shape and out.stats["elements_count"] == x.size
+        assert quant.needs_calibration() == model.needs_calibration()
+        assert f32(float(quant.get_dynamic_scales())) == ema
+        scales.append(float(ema))
+        if precision == bh.QuantizationPrecision.OneFiveFiveBit:
+            assert set(np.unique(host(out.values)).tolist()) <= {-1, 0, 1}
+    assert scales[0] < scales[1] < scales[2]  # the scale adapts to the magnitude (test_..._dynamic_scaling)
+    deq = quant.dequantize(out)
+    assert tuple(deq.shape) == shape
+    quant.reset_dynamic_state()
+    again = quant.quantize_dynamic(dev(x))
+    own = orc.abs_max(x) / f32(127.0) if precision == bh.QuantizationPrecision.EightBit else orc.abs_max(x)
+    assert f32(again.stats["scale_factor"]) == own and again.stats["scale_factor"] > 0
+    quant.calibrate([dev((x * f32(m)).astype(f32)) for m in (1.0, 4.0, 2.0)])
+    assert f32(quant.state.ema_scale) == orc.abs_max((x * f32(4.0)).astype(f32)) and quant.state.calibrated
+    att = quant.quantize_attention(dev(x), 64)
+    assert att.sequence_length == 64
+    off = bh.DynamicActivationQuantizer(bh.ActivationQuantizationConfig(quantize_attention=False))
+    with pytest.raises(bh.BitLinearError):
+        off.quantize_attention(dev(x), 8)
+    with pytest.raises(bh.BitLinearError):
+        quant.validate_input(torch.zeros((), device="cuda"))
+    with pytest.raises(bh.BitLinearError):
+        quant.validate_input(torch.zeros((4, 4), dtype=torch.uint8, device="cuda"))
+
+
 # ---- R1 + A1 -------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("m,k", [(1, 2560), (4, 2560), (3, 6912), (2, 1024), (5, 4096), (2, 8192), (2, 12000),

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from helpers import golden_vectors, synth_activations, synth_weights
+import bitnet_hip as bh
 from oracle import oracle as orc
 
 G = golden_vectors()
@@ -759,3 +760,77 @@ def test_quantiser_rounding_identity_over_all_floats(tmp_path):
     subprocess.run(["gcc", "-O2", "-fopenmp", "-fno-fast-math", str(src), "-o", str(exe), "-lm"], check=True)
     out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=900)
     assert out.returncode == 0 and "mismatches: 0" in out.stdout, out.stdout[-500:]
+
+
+# ---- DynamicActivationQuantizer (activations.rs:203-454): the scaled quantiser and the host-side state ---------------------
+
+def test_scaled_quantizer_closed_forms_and_numpy_model():
+    rng = np.random.default_rng(41)
+    x = (rng.standard_normal(5000, dtype=f32) * f32(3.0)).astype(f32)
+    am = orc.abs_max(x)
+    assert am == np.max(np.abs(x)) and orc.abs_max(np.zeros(7, dtype=f32)) == 0.0
+    # 8-bit with the tensor's own scale abs_max / 127: the extreme lands on +-127, nothing beyond
+    scale = f32(am / f32(127.0))
+    q = orc.quantize_activations_scaled(x, 1, scale)
+    assert np.max(np.abs(q.astype(np.int32))) == 127 and q[np.argmax(np.abs(x))] == np.sign(x[np.argmax(np.abs(x))]) * 127
+    # independent numpy model: y = x * f32(1 / f64(scale)); halves away from zero
+    recip = f32(1.0 / float(scale))
+    y = x * recip
+    model = (np.sign(y) * np.floor(np.abs(np.clip(y, -127, 127)).astype(np.float64) + 0.5)).astype(np.int8)
+    assert np.array_equal(q, model)
+    # the reference's literal u8 form: clamp(0, 255) before the rounding, i.e. max(signed, 0) while nothing exceeds 127
+    u8 = orc.quantize_activations_scaled(x, 1, scale, reference_u8=True).view(np.uint8)
+    assert np.array_equal(u8, np.maximum(q, 0).astype(np.uint8))
+    big = orc.quantize_activations_scaled(np.array([300.0, 200.4, 127.5, -3.0, 0.5, 1.5, 2.5], dtype=f32), 1, 1.0, reference_u8=True)
+    assert big.view(np.uint8).tolist() == [255, 200, 128, 0, 1, 2, 3]
+    assert orc.quantize_activations_scaled(np.array([300.0, -300.0, 0.5, -0.5, -1.5], dtype=f32), 1, 1.0).tolist() == [127, -127, 1, -1, -2]
+    # ternary: strict thresholds at +-0.5 of the scaled value
+    t = orc.quantize_activations_scaled(np.array([1.0, 0.5, 0.50001, -0.5, -0.50001, 0.0, -2.0], dtype=f32), 0, 1.0)
+    assert t.tolist() == [1, 0, 1, 0, -1, 0, -1]
+    t2 = orc.quantize_activations_scaled(x, 0, am)
+    assert np.array_equal(t2, (x * f32(1.0 / float(am)) > 0.5).astype(np.int8) - (x * f32(1.0 / float(am)) < -0.5).astype(np.int8))
+    # a zero scale (all-zero tensor): 0 * inf is NaN, which both branches turn into 0
+    assert not orc.quantize_activations_scaled(np.zeros(4, dtype=f32), 1, 0.0).any()
+    assert not orc.quantize_activations_scaled(np.zeros(4, dtype=f32), 0, 0.0).any()
+
+
+def test_dynamic_scale_state_follows_the_reference_state_machine():
+    """DynamicScaleState against hand-evaluated steps of compute_dynamic_scale / update_dynamic_params / calibrate /
+    reset_dynamic_state (activations.rs:241-267, 420-447, 459-493)."""
+    cfg = bh.ActivationQuantizationConfig(precision=bh.QuantizationPrecision.EightBit, moving_average_window=3, calibration_warmup=2,
+                                          ema_decay=0.9)
+    st = bh.DynamicScaleState(cfg)
+    assert st.ema_scale is None and st.needs_calibration()
+    seen = []
+    for step, am in enumerate([12.7, 25.4, 6.35, 127.0, 1.27], start=1):
+        st.step_count += 1  # quantize_dynamic increments before update_dynamic_params
+        ema = st.update(am)
+        cur = f32(am) / f32(127.0)
+        seen.append(cur)
+        if step == 1:
+            want = cur
+        else:
+            want = f32(0.9) * want + (f32(1.0) - f32(0.9)) * cur
+        assert ema == want and ema.dtype == np.float32
+        assert st.scale_history == seen[-3:]          # the window keeps the last three per-step scales
+        assert st.calibrated == (step > 2)            # flips on the first step past the warm-up
+        assert st.calibration_samples == min(step, 2)
+    assert not st.needs_calibration()
+    # ternary: the per-step scale is the abs-max itself
+    st3 = bh.DynamicScaleState(bh.ActivationQuantizationConfig())
+    st3.step_count += 1
+    assert st3.update(3.5) == f32(3.5)
+    # calibrate: index floor(len * 99.9 / 100) of the sorted abs-maxima, clipped to the last
+    st.calibrate([5.0, 1.0, 9.0, 3.0])
+    assert st.ema_scale == f32(9.0) and st.calibrated
+    st50 = bh.DynamicScaleState(bh.ActivationQuantizationConfig(outlier_percentile=50.0))
+    st50.calibrate([5.0, 1.0, 9.0, 3.0])
+    assert st50.ema_scale == f32(5.0)                 # floor(4 * 0.5) = 2 -> third smallest
+    with pytest.raises(bh.BitLinearError):
+        st.calibrate([])
+    st.reset()
+    assert st.ema_scale is None and st.step_count == 0 and not st.calibrated and st.scale_history == []
+    for bad in (dict(moving_average_window=0), dict(outlier_percentile=0.0), dict(outlier_percentile=100.5), dict(ema_decay=1.5)):
+        with pytest.raises(bh.BitLinearError):
+            bh.ActivationQuantizationConfig(**bad).validate()
+    bh.ActivationQuantizationConfig().validate()

@@ -112,3 +112,23 @@ def test_rust_crate_gates_the_library_behind_its_feature_and_keeps_raw_pointers_
     tensor = re.search(r"pub struct DeviceTensor \{(.*?)\}", lib, flags=re.S).group(1)
     assert "pub " not in tensor
     assert "HipNotEnabled" in lib and '#[cfg(not(feature = "hip"))]' in lib
+
+
+def test_rust_quantizer_wrappers_call_the_library_and_use_the_model():
+    """The safe layer reaches the quantiser entry points (not only declares them), implements the reference's Quantizer
+    trait (quantization/mod.rs:96-116: quantize, dequantize, config, validate_input, get_stats) for the weight pipeline and
+    the dynamic activation quantiser, and optimize_model builds its decoder from the Model it is given."""
+    lib = (FFI.parent / "lib.rs").read_text()
+    for sym in ("bitnet_hip_absmax_quantize_activations", "bitnet_hip_quantize_weights_reference", "bitnet_hip_abs_max",
+                "bitnet_hip_quantize_activations_scaled", "bitnet_hip_bitlinear_set_weights_gguf", "bitnet_hip_decoder_set_chains"):
+        assert f"ffi::{sym}(" in lib, sym
+    for target in ("HipBitNetWeightQuantizer", "HipActivationQuantizerAdapter"):
+        methods = _trait_methods(lib, rf"impl Quantizer for {target}\s*\{{")
+        assert set(methods) == {"quantize", "dequantize", "config", "validate_input", "get_stats"}, target
+        assert methods["quantize"][0] == "&self" and len(methods["quantize"]) == 2
+    body = lib[lib.index("fn optimize_model(&mut self, model: &Model)"):]
+    body = body[:body.index("fn get_memory_usage")]
+    assert "decoder_shape_of(model)" in body and "let _ = model" not in body and "bind_decoder" in body
+    assert "model.architecture" in lib
+    # the state machine of DynamicActivationQuantizer, as the reference writes it (activations.rs:252-257)
+    assert "self.config.ema_decay * prev + (1.0 - self.config.ema_decay) * current_scale" in lib
