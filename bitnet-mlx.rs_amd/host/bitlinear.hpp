@@ -143,6 +143,7 @@ public:
     {
         bitnet_hip_bitlinear_destroy(handle_);
         if (workspace_) (void)hipFree(workspace_);
+        if (workspace_done_) (void)hipEventDestroy(workspace_done_);
     }
     BitLinear(const BitLinear &) = delete;
     BitLinear &operator=(const BitLinear &) = delete;
@@ -196,10 +197,20 @@ public:
                 return BitLinearError{BitLinearError::MemoryError, "hipMalloc failed", {}, {}};
             workspace_bytes_ = need;
         }
+        // the scratch is shared by every forward of this layer: a call on another stream than the one before it waits,
+        // on the GPU, for that call to finish with it (the lock above orders only the enqueue)
+        if (!workspace_done_ && hipEventCreateWithFlags(&workspace_done_, hipEventDisableTiming) != hipSuccess)
+            return BitLinearError{BitLinearError::DeviceError, "hipEventCreate failed", {}, {}};
+        if (workspace_used_ && workspace_stream_ != stream && hipStreamWaitEvent(stream, workspace_done_, 0) != hipSuccess)
+            return BitLinearError{BitLinearError::DeviceError, "hipStreamWaitEvent failed", {}, {}};
         int rc = bitnet_hip_bitlinear_forward(handle_, input.data(), input.dims().data(), (int)input.dims().size(), gamma,
                                               config_.rms_norm_eps, config_.sum_order, nullptr, out.unwrap().data(),
                                               workspace_, workspace_bytes_, nullptr, nullptr, nullptr, stream);
         if (rc != BITNET_HIP_OK) return last_error(rc);
+        if (hipEventRecord(workspace_done_, stream) != hipSuccess)
+            return BitLinearError{BitLinearError::DeviceError, "hipEventRecord failed", {}, {}};
+        workspace_stream_ = stream;
+        workspace_used_ = true;
         return out;
     }
     Result<DeviceTensor> forward_batch(const DeviceTensor &inputs) const
@@ -222,6 +233,9 @@ private:
     mutable std::mutex workspace_lock_;  // forward calls of one layer share the scratch: one at a time through this mirror
     mutable void *workspace_ = nullptr;
     mutable size_t workspace_bytes_ = 0;
+    mutable hipEvent_t workspace_done_ = nullptr;  // recorded behind every forward, on its stream
+    mutable hipStream_t workspace_stream_ = nullptr;
+    mutable bool workspace_used_ = false;
 };
 
 // TernaryProcessor: per-token int8 absmax quantisation and the ternary matmul on top of it.
