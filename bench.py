@@ -277,7 +277,14 @@ def launch_floor(bh, torch, step_us):
     reads = sorted(bh.measure_launch_chain(LAUNCHES_PER_STEP, replays=20, buf=buf, bytes_per_launch=per_launch) for _ in range(5))[2]
     one = sorted(bh.measure_launch_chain(1, replays=20, buf=buf, bytes_per_launch=[STEP_BYTES]) for _ in range(5))[2]
     del buf
-    return {"launches": LAUNCHES_PER_STEP, "bytes": STEP_BYTES,
+    # the alternative to a kernel boundary: workgroups that stay resident and hand the vector on through memory inside one
+    # launch (bitnet_hip_measure_hop), at the three widths a layer hands over (v: 640, hidden state: 2560, gate / up: 6912)
+    hop = {}
+    for values in (640, 2560, 6912):
+        for two_level in (False, True):
+            us, intact = bh.measure_hop(values, hops=200, two_level=two_level)
+            hop[f"{'two_level' if two_level else 'flat'}_{values}_values_us"] = round(us, 2) if intact else None
+    return {"launches": LAUNCHES_PER_STEP, "bytes": STEP_BYTES, "in_launch_hand_over": hop,
             "empty_kernels_us_per_step": round(empty, 1), "empty_kernel_us_per_launch": round(empty / LAUNCHES_PER_STEP, 3),
             "read_only_kernels_us_per_step": round(reads, 1), "read_only_kernel_us_per_launch": round(reads / LAUNCHES_PER_STEP, 3),
             "read_only_frac_hbm_peak": round(STEP_BYTES / (reads * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),

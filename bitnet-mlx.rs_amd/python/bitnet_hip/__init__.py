@@ -90,6 +90,7 @@ def load_library() -> C.CDLL:
         "bitnet_hip_device_info": (i32, [C.c_char_p, sz, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz)]),
         "bitnet_hip_measure_mfma_i8_rate": (i32, [i32, C.POINTER(C.c_double), vp]),
         "bitnet_hip_measure_launch_chain": (i32, [vp, C.POINTER(sz), sz, sz, sz, C.POINTER(C.c_double), vp]),
+        "bitnet_hip_measure_hop": (i32, [i32, sz, sz, i32, C.POINTER(C.c_double), C.POINTER(i32), vp]),
         "bitnet_hip_quantize_activations_i8": (i32, [vp, vp, sz, sz, sz, i32, sz, sz, vp, f32, i32, vp, vp, vp, vp, vp]),
         "bitnet_hip_absmax_quantize_activations": (i32, [vp, sz, i32, vp, vp, vp]),
         "bitnet_hip_abs_max": (i32, [vp, sz, C.POINTER(C.c_float), vp]),
@@ -263,6 +264,16 @@ def measure_launch_chain(launches: int, replays: int = 20, buf: Optional[torch.T
     _check(load_library().bitnet_hip_measure_launch_chain(_ptr(buf), arr, len(sizes), launches, replays, C.byref(us),
                                                           _stream(stream)))
     return us.value
+
+
+def measure_hop(values: int, hops: int = 200, two_level: bool = False, spin_limit: int = 0, stream=None):
+    """(microseconds per hand-over, intact) of a vector of `values` 32-bit values passed from step to step through memory
+    inside ONE launch of resident workgroups (bitnet_hip_measure_hop); intact is False if a bounded wait ran out or the
+    final values are wrong (spin_limit = 1 forces that: every wait gives up after one look and the kernel still ends)."""
+    us, ok = C.c_double(0.0), C.c_int(0)
+    _check(load_library().bitnet_hip_measure_hop(1 if two_level else 0, values, hops, spin_limit, C.byref(us), C.byref(ok),
+                                                 _stream(stream)))
+    return us.value, bool(ok.value)
 
 
 # ---- raw operators ------------------------------------------------------------------------------

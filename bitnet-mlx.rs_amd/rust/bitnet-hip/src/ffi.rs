@@ -62,6 +62,8 @@ extern "C" {
     pub fn bitnet_hip_measure_launch_chain(buf: *const c_void, bytes_per_launch: *const usize, pattern_len: usize,
                                            launches: usize, replays: usize, us_per_replay: *mut f64,
                                            stream: *mut c_void) -> c_int;
+    pub fn bitnet_hip_measure_hop(two_level: c_int, values: usize, hops: usize, spin_limit: c_int, us_per_hop: *mut f64, intact: *mut c_int,
+                                  stream: *mut c_void) -> c_int;
     pub fn bitnet_hip_quantize_activations_i8(x: *const f32, x2: *const f32, ldx: usize, m: usize, k: usize,
                                               input_mode: c_int, gqa_group: usize, head_dim: usize, gamma: *const f32,
                                               eps: f32, sum_order: c_int, q: *mut i8, a_scale: *mut f32,

@@ -107,6 +107,18 @@ int bitnet_hip_measure_mfma_i8_rate(int random_operands, double *tera_ops_per_se
  * the result.  No counterpart in the reference; bench.py reports both floors beside the measured token step. */
 int bitnet_hip_measure_launch_chain(const void *buf, const size_t *bytes_per_launch, size_t pattern_len,
                                     size_t launches, size_t replays, double *us_per_replay, void *stream);
+/* Diagnostic: microseconds one hand-over of a vector costs INSIDE a single launch whose workgroups stay resident (one per
+ * compute unit) and pass `values` 32-bit values from step to step through memory: every workgroup produces its share with
+ * device-scope stores and must have seen all values of a step before it produces the next (what a persistent decoder
+ * would do in place of a kernel boundary).  two_level == 0: every workgroup polls all values; != 0: one workgroup per
+ * XCD polls them and republishes them in its XCD's L2, the others poll that copy.  Runs `hops` steps twice (the second run
+ * is timed, launch included), checks the final values, and reports whether every wait was met within spin_limit looks
+ * (<= 0 or above 100000: 20000; every wait is bounded, and a thread whose wait ran out looks only once from then on, so
+ * the kernel ends in any case): *intact = 1 if so, 0 if a wait ran out or a value is wrong (spin_limit = 1 forces that).
+ * us_per_hop and intact are HOST pointers; allocates a few hundred KB and waits for the result.  No counterpart in the
+ * reference. */
+int bitnet_hip_measure_hop(int two_level, size_t values, size_t hops, int spin_limit, double *us_per_hop, int *intact,
+                           void *stream);
 
 /* ---- activation side -------------------------------------------------------------------------- */
 

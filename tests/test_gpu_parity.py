@@ -1375,3 +1375,29 @@ def test_bitlinear_housekeeping_methods_of_the_reference():
     assert ei.value.kind == "DeviceError"
     stats = bh.BitNetWeightQuantizer().get_stats()
     assert (stats.elements_count, stats.quantization_error, stats.compression_ratio, stats.scale_factor, stats.zero_point) == (0, 0.0, 1.0, 1.0, None)
+
+
+# ---- device diagnostics behind the C ABI -----------------------------------------------------------------------------------
+
+def test_launch_chain_and_hand_over_diagnostics():
+    """bitnet_hip_measure_launch_chain and bitnet_hip_measure_hop: plausible figures, argument checks, and the bounded
+    waits of the hand-over kernel: with a spin limit of one look every wait gives up, the call reports that the vector did
+    not arrive intact, and the kernel has ended normally (the next call on the device works)."""
+    empty = bh.measure_launch_chain(60, replays=5)
+    assert 10.0 < empty < 2000.0  # 60 dependent empty kernels: microseconds each, not nanoseconds and not milliseconds
+    buf = torch.zeros(60 * 65536, dtype=torch.uint8, device="cuda")
+    reads = bh.measure_launch_chain(60, replays=5, buf=buf, bytes_per_launch=[65536])
+    assert reads >= 0.5 * empty
+    with pytest.raises(bh.BitLinearError):
+        bh.measure_launch_chain(61, replays=5, buf=buf, bytes_per_launch=[65536])  # needs more bytes than the buffer holds
+    with pytest.raises(bh.BitLinearError):
+        bh.measure_launch_chain(2, replays=5, buf=buf, bytes_per_launch=[24])
+    for two_level in (False, True):
+        us, intact = bh.measure_hop(640, hops=20, two_level=two_level)
+        assert intact and 0.2 < us < 200.0
+    us, intact = bh.measure_hop(2560, hops=8, two_level=False, spin_limit=1)
+    assert not intact  # every wait gave up after one look; the kernel ended all the same
+    us, intact = bh.measure_hop(640, hops=20)
+    assert intact
+    with pytest.raises(bh.BitLinearError):
+        bh.measure_hop(0, hops=5)
