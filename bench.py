@@ -76,7 +76,7 @@ STEP_BYTES = LAYER_BYTES * LAYERS
 # script with --no-extras --calibration-copy), each scaled by what the same counter reads for the plain
 # 256 MiB copy: FETCH_SIZE reads 0.5 KiB per KiB fetched (factor 2.0), WRITE_SIZE 1.0 (factor 1.0).
 # Summary: profiles/decode_layer_b1_gemv_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_685_937
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_685_627
 
 
 def decode_roofline(event_ms, steps):
@@ -206,7 +206,9 @@ def large_gemv_pair(bh, torch, gen, loops=5):
     ms = regions[2]
     out["gemv_32768x16384_m1"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1),
                                   "frac_hbm_peak": round(n * k / 4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                                  "timed": f"median of 5 regions of {4 * loops} launches over 4 x 128 MiB of distinct weights",
+                                  "best_region_frac_hbm_peak": round(n * k / 4 / (regions[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                  "timed": f"median of 5 regions of {4 * loops} launches over 4 x 128 MiB of distinct weights (the rate "
+                                           "sags by a few per cent while the stream is sustained: every region is listed)",
                                   "regions_us": [round(r * 1e3, 2) for r in regions]}
     del layers, packed
     b3_bytes = bh.base3_packed_size(n * k)
