@@ -23,7 +23,18 @@ struct ActQuantParams {
     float *y;
     size_t m;
     int seq_in_lds;  // the launch carries LDS for the row's squares (literal summation order: sum_sequential_lds)
+    unsigned *zero;  // optional: zero[0 .. zero_n) is cleared by the first workgroup (counters of the launch that follows)
+    int zero_n;
 };
+
+// The clearing job: the threads of workgroup 0 (any block shape) write the zeros with vector stores.
+__device__ __forceinline__ void clear_counters(const ActQuantParams &p)
+{
+    if (blockIdx.x == 0 && p.zero) {
+        const int flat = threadIdx.y * blockDim.x + threadIdx.x, count = blockDim.x * blockDim.y;
+        for (int i = flat; i < p.zero_n; i += count) p.zero[i] = 0u;
+    }
+}
 
 // NCH > 0: a lane keeps its NCH chunks in registers (K <= 256*NCH).  NCH == 0: any K, the row is
 // re-read (from cache) in each pass.
@@ -32,6 +43,7 @@ __global__ __launch_bounds__(256) void act_quant_wave_kernel(ActQuantParams p)
 {
     const RowSource &src = p.src;
     const int lane = threadIdx.x;
+    clear_counters(p);
     const size_t row = (size_t)blockIdx.x * blockDim.y + threadIdx.y;
     if (row >= p.m) return;  // uniform per wavefront: a wavefront is one row
     const int k = src.k;
@@ -130,6 +142,7 @@ __global__ __launch_bounds__(256) void act_quant_block_kernel(ActQuantParams p)
     __shared__ int red_i[4];
     const RowSource &src = p.src;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    clear_counters(p);
     const size_t row = blockIdx.x;
     const int k = src.k;
     const int chunks = (k + 3) >> 2;
@@ -267,6 +280,7 @@ __global__ __launch_bounds__(1024) void act_quant_block16_kernel(const float *ho
         for (int i = 0; i < NCHB; ++i) gm[i] = load_gamma_chunk(src, min(tid + 1024 * i, chunks - 1), true);
     }
     __builtin_amdgcn_sched_barrier(0);  // nothing below moves above: the first wait for the argument buffer comes here
+    clear_counters(p);
     const bool chain = norm && src.sum_order != BITNET_HIP_SUM_SEQUENTIAL && wave < 4;
 #pragma unroll
     for (int i = 0; i < NCHB; ++i)
@@ -582,9 +596,10 @@ int launch_absmax_quantize(const float *x, size_t n, int precision, void *scratc
 
 int launch_act_quant(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
                      size_t gqa_group, size_t head_dim, const float *gamma, float eps, int sum_order,
-                     int8_t *q, float *a_scale, int32_t *a_sum, float *y, hipStream_t stream)
+                     int8_t *q, float *a_scale, int32_t *a_sum, float *y, hipStream_t stream, unsigned *zero, size_t zero_n)
 {
     ActQuantParams p;
+    p.zero = zero; p.zero_n = (int)zero_n;
     p.src.x = x; p.src.x2 = x2; p.src.gamma = gamma; p.src.ldx = ldx; p.src.k = (int)k;
     p.src.head_dim = (int)(head_dim ? head_dim : 1); p.src.gqa_group = (int)(gqa_group ? gqa_group : 1);
     p.src.sum_order = sum_order; p.src.eps = eps;

@@ -154,7 +154,8 @@ size_t launch_group_blocks(bitnet_hip_bitlinear *const *layers, size_t count)
 int run_projections(bitnet_hip_bitlinear *const *layers, int count, const float *x, const float *x2, size_t ldx,
                     size_t m, int input_mode, size_t gqa_group, size_t head_dim, const float *gamma, float eps,
                     int sum_order, const float *const *residual, float *const *out, int32_t *const *acc, int8_t *q,
-                    float *a_scale, int32_t *a_sum, bool want_quant_outputs, hipStream_t s)
+                    float *a_scale, int32_t *a_sum, bool want_quant_outputs, hipStream_t s,
+                    const GemmSplitScratch *split = nullptr)
 {
     const size_t k = layers[0]->in_features;
     auto proj_of = [&](int j) {
@@ -176,11 +177,14 @@ int run_projections(bitnet_hip_bitlinear *const *layers, int count, const float 
         return BITNET_HIP_OK;
     }
     if (!q || !a_scale || !a_sum) return fail(BITNET_HIP_MEMORY_ERROR, "projection: no scratch for the quantised activations");
-    int rc = launch_act_quant(x, x2, ldx, m, k, input_mode, gqa_group, head_dim, gamma, eps, sum_order, q, a_scale, a_sum,
-                              nullptr, s);
-    if (rc != BITNET_HIP_OK) return rc;
     size_t n_blocks = 0;
     for (int j = 0; j < count; ++j) n_blocks += row_blocks(layers[j]->out_features);
+    // A GEMM that splits k across workgroups finds its tile counters zeroed by the quantiser launched in front of it.  One
+    // scratch serves one launch: more projections than one launch takes run without the split.
+    const bool use_split = split && split->counters && count <= GEMM_MAX_PROJ && !gemv_takes(m, k, n_blocks, q);
+    int rc = launch_act_quant(x, x2, ldx, m, k, input_mode, gqa_group, head_dim, gamma, eps, sum_order, q, a_scale, a_sum,
+                              nullptr, s, use_split ? split->counters : nullptr, use_split ? split->counter_count : 0);
+    if (rc != BITNET_HIP_OK) return rc;
     if (gemv_takes(m, k, n_blocks, q)) {
         for (int j0 = 0; j0 < count; j0 += GEMV_MAX_PROJ) {
             GemvProj pjs[GEMV_MAX_PROJ];
@@ -195,7 +199,7 @@ int run_projections(bitnet_hip_bitlinear *const *layers, int count, const float 
         GemvProj pjs[GEMM_MAX_PROJ];
         const int nj = count - j0 < GEMM_MAX_PROJ ? count - j0 : GEMM_MAX_PROJ;
         for (int j = 0; j < nj; ++j) pjs[j] = proj_of(j0 + j);
-        rc = launch_gemm_multi(pjs, nj, q, a_sum, a_scale, m, k, s);  // all of them in one launch where that applies
+        rc = launch_gemm_multi(pjs, nj, q, a_sum, a_scale, m, k, s, use_split ? split : nullptr);  // all of them in one launch where that applies
         if (rc == BITNET_HIP_UNSUPPORTED) {
             for (int j = 0; j < nj; ++j) {
                 const GemvProj &pj = pjs[j];
@@ -225,6 +229,24 @@ QuantScratch carve_scratch(void *ws, size_t m, size_t k)
     sc.a_scale = reinterpret_cast<float *>(base + align_up(m * k, 256));
     sc.a_sum = reinterpret_cast<int32_t *>(base + align_up(m * k, 256) + align_up(m * sizeof(float), 256));
     return sc;
+}
+
+// Scratch of a GEMM that splits k across workgroups, behind the quantised activations in the same workspace.
+size_t split_scratch_bytes(size_t m, size_t k, size_t n)
+{
+    size_t partial_bytes = 0, counters = 0;
+    gemm_split_plan(m, k, &n, 1, &partial_bytes, &counters);
+    return partial_bytes ? partial_bytes + align_up(counters * sizeof(unsigned), 256) : 0;
+}
+GemmSplitScratch carve_split(void *ws, size_t m, size_t k, size_t n)
+{
+    GemmSplitScratch sp;
+    gemm_split_plan(m, k, &n, 1, &sp.partial_bytes, &sp.counter_count);
+    if (sp.partial_bytes == 0) return sp;
+    const uintptr_t base = align_up(reinterpret_cast<uintptr_t>(ws), 256) + quant_scratch_bytes(m, k) - 256;  // behind a_sum: quant_scratch_bytes counts 256 bytes of alignment slack
+    sp.partials = reinterpret_cast<int32_t *>(base);
+    sp.counters = reinterpret_cast<unsigned *>(base + sp.partial_bytes);
+    return sp;
 }
 
 }  // namespace
@@ -763,7 +785,8 @@ int bitnet_hip_bitlinear_get_quantized(bitnet_hip_bitlinear *layer, float *w_sca
 size_t bitnet_hip_bitlinear_workspace_size(const bitnet_hip_bitlinear *layer, size_t m)
 {
     if (!layer) return 0;
-    return quant_scratch_bytes(m, layer->in_features);
+    // the quantised activations, and the partial tiles of a GEMM that splits k across workgroups where one would run
+    return quant_scratch_bytes(m, layer->in_features) + split_scratch_bytes(m, layer->in_features, layer->out_features);
 }
 
 int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, const size_t *dims, int rank,
@@ -799,16 +822,21 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
     void *ws = workspace;
     bool own_ws = false;
     QuantScratch sc = {dbg_q, dbg_a_scale, nullptr};
+    GemmSplitScratch split;
     if (!fused || debug) {  // the fused decode launch needs no scratch unless the caller wants q / a_scale back
-        const size_t need = quant_scratch_bytes(m, in);
+        const size_t need = quant_scratch_bytes(m, in), extra = split_scratch_bytes(m, in, layer->out_features);
+        bool with_split = extra != 0;
         if (!ws) {
-            hipError_t e = hipMallocAsync(&ws, need, s);
-            if (e != hipSuccess) return fail(BITNET_HIP_MEMORY_ERROR, "forward: hipMallocAsync(%zu) failed: %s", need, hipGetErrorString(e));
+            hipError_t e = hipMallocAsync(&ws, need + extra, s);
+            if (e != hipSuccess) return fail(BITNET_HIP_MEMORY_ERROR, "forward: hipMallocAsync(%zu) failed: %s", need + extra, hipGetErrorString(e));
             own_ws = true;
         } else if (workspace_bytes < need) {
             return fail(BITNET_HIP_MEMORY_ERROR, "forward: workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+        } else if (workspace_bytes < need + extra) {
+            with_split = false;  // room for the quantised activations only: the GEMM walks k without the split
         }
         sc = carve_scratch(ws, m, in);
+        if (with_split) split = carve_split(ws, m, in, layer->out_features);
         if (dbg_q) sc.q = dbg_q;
         if (dbg_a_scale) sc.a_scale = dbg_a_scale;
     }
@@ -817,7 +845,7 @@ int bitnet_hip_bitlinear_forward(bitnet_hip_bitlinear *layer, const float *x, co
     float *outs[1] = {out};
     int32_t *accs[1] = {dbg_acc};
     int rc = run_projections(layers, 1, x, nullptr, in, m, BITNET_HIP_INPUT_PLAIN, 1, 1, gamma, eps, sum_order, res, outs,
-                             accs, sc.q, sc.a_scale, sc.a_sum, debug, s);
+                             accs, sc.q, sc.a_scale, sc.a_sum, debug, s, split.partials ? &split : nullptr);
     if (own_ws) {
         hipError_t e = hipFreeAsync(ws, s);
         if (rc == BITNET_HIP_OK && e != hipSuccess)

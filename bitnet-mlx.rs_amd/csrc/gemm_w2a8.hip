@@ -75,6 +75,10 @@ struct GemmParams {
     int kt_count;   // 256-column weight tiles per row block
     int tiles_m, tiles_n;
     int rotate;     // gemm_dma_kernel: every workgroup of the launch is resident at once (see there)
+    // gemm_dma_kernel<..., SPLIT = true>: k split across nsplit workgroups per output tile, st_per (even) stages each
+    int nsplit, st_per;
+    int *partials;        // [tile][part][fragment][thread] int4
+    unsigned *counters;   // one per output tile, zero at launch; the last workgroup of a tile leaves it zero again
 };
 
 constexpr int STAGE_K = 256;              // columns per pipeline stage = one weight tile
@@ -441,7 +445,20 @@ constexpr int dma_in_flight()
     return n;
 }
 
-template <int BM, int BN, int D, int OCC>
+// Four ints exchanged between workgroups inside one launch: device-scope (relaxed atomic) stores and loads, which the
+// hardware writes through to, and reads from, the level every XCD shares, 8 bytes at a time.
+__device__ __forceinline__ void store_shared4(int *ptr, v4i v)
+{
+    typedef volatile __attribute__((address_space(1))) v4i gv4i;
+    *(gv4i *)(uintptr_t)ptr = v;
+}
+__device__ __forceinline__ v4i load_shared4(const int *ptr)
+{
+    typedef const volatile __attribute__((address_space(1))) v4i gv4i;
+    return *(gv4i *)(uintptr_t)ptr;
+}
+
+template <int BM, int BN, int D, int OCC, bool SPLIT = false>
 __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
 {
     constexpr int WTM = BM / 2, WTN = BN / 2, FM = WTM / 16, FN = WTN / 16;
@@ -459,13 +476,15 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1, lr = lane & 15, lg = lane >> 4;
 
-    int tile_id;
+    int tile_id, ks = 0;
     {
-        const int total = p.tiles_m * p.tiles_n;
+        const int nsplit = SPLIT ? p.nsplit : 1;
+        const int total = p.tiles_m * p.tiles_n * nsplit;
         const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
         const int per_xcd = (total + 7) >> 3;
         tile_id = xcd * per_xcd + idx;
         if (tile_id >= total) return;
+        if (SPLIT) { ks = tile_id % nsplit; tile_id /= nsplit; }  // the parts of a tile are neighbours: one XCD
     }
     // tiles_n counts the column tiles of all projections of the launch, one after the other
     const int tm = tile_id / p.tiles_n, tn_all = tile_id % p.tiles_n;
@@ -475,7 +494,8 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
     const GemmProjDev PJ = p.proj[pj];  // uniform over the workgroup
     const int tn = tn_all - (pj ? p.proj[pj - 1].tn_end : 0);
     const int m0 = tm * BM, n0 = tn * BN;
-    const int nstage = p.kt_count * 2;
+    const int s_first = SPLIT ? __builtin_amdgcn_readfirstlane(ks * p.st_per) : 0;  // even
+    const int nstage = SPLIT ? min(p.st_per, p.kt_count * 2 - s_first) : p.kt_count * 2;  // stages of this workgroup (even)
 
     // Activation loads: load q of this wavefront covers tile rows 8*(wave*A_DMA + q) .. +7; lane l lands in
     // row l/8 at physical 16-byte chunk l%8 and therefore fetches logical chunk (l%8) ^ (row & 7).
@@ -508,11 +528,11 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
             const int kt = s >> 1;
             const uint32_t dst = lds_base + D * A_STAGE + (kt % NB) * B_STAGE;
 #pragma unroll
-            for (int q = 0; q < B_DMA; ++q) dma16(PJ.w + (size_t)kt * 1024, b_off[q], dst + b_dst[q]);
+            for (int q = 0; q < B_DMA; ++q) dma16(PJ.w + (size_t)(kt + (s_first >> 1)) * 1024, b_off[q], dst + b_dst[q]);
         }
         const uint32_t dst = lds_base + (s % D) * A_STAGE + wave * A_DMA * 1024;
 #pragma unroll
-        for (int q = 0; q < A_DMA; ++q) dma16(p.a + (size_t)s * DMA_SK, a_off[q], dst + q * 1024);
+        for (int q = 0; q < A_DMA; ++q) dma16(p.a + (size_t)(s + s_first) * DMA_SK, a_off[q], dst + q * 1024);
     };
 
     v4i acc[FM][FN];
@@ -589,6 +609,36 @@ __global__ __launch_bounds__(256, OCC) void gemm_dma_kernel(GemmParams p)
     static_assert(rowp_bytes<BM>() <= A_STAGE, "row operands fit an activation stage");
     wait_vm<0>();
     __syncthreads();
+    if constexpr (SPLIT) {
+        // Every part stores its int32 fragments (device-scope stores: written through to where every XCD reads them),
+        // waits until they have been acknowledged, and draws a ticket from the tile's counter; the part that draws the
+        // last one adds up all parts (integers: any order, same sum), leaves the counter at zero and runs the epilogue.
+        // Nobody waits for anybody.
+        __shared__ int last_ticket;
+        constexpr int SLAB = FM * FN * 256 * 4;
+        int *mine = p.partials + ((size_t)tile_id * p.nsplit + ks) * SLAB;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) store_shared4(mine + ((i * FN + j) * 256 + tid) * 4, acc[i][j]);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (tid == 0)
+            last_ticket = __hip_atomic_fetch_add(&p.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(p.nsplit - 1);
+        __syncthreads();
+        if (!last_ticket) return;  // uniform over the workgroup
+        if (tid == 0) __hip_atomic_store(&p.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int *slab = p.partials + (size_t)tile_id * p.nsplit * SLAB;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) acc[i][j] = (v4i){0, 0, 0, 0};
+        for (int part = 0; part < p.nsplit; ++part, slab += SLAB)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j) acc[i][j] += load_shared4(slab + ((i * FN + j) * 256 + tid) * 4);
+    }
     int lrows[FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i) lrows[i] = wm * WTM + i * 16 + lr;
@@ -637,6 +687,29 @@ int launch_dma(GemmParams p, hipStream_t stream)
 // 35.8 us with the two loaders).  The multiplying wavefronts meet the loaders at the stage barrier and otherwise
 // only read LDS and run MFMAs.
 constexpr int LD8_NST = 3;
+// The same kernel with k split across nsplit workgroups per output tile (st_per stages each; see the kernel's SPLIT branch).
+template <int BM, int BN, int D, int OCC>
+int launch_dma_split(GemmParams p, int nsplit, int st_per, const GemmSplitScratch &scratch, hipStream_t stream)
+{
+    p.tiles_m = (p.m + BM - 1) / BM;
+    p.tiles_n = 0;
+    for (int j = 0; j < p.nproj; ++j) p.proj[j].tn_end = p.tiles_n += (p.proj[j].n + BN - 1) / BN;
+    const size_t tiles = (size_t)p.tiles_m * p.tiles_n;
+    if (tiles * nsplit * BM * BN * sizeof(int32_t) > scratch.partial_bytes || tiles > scratch.counter_count)
+        return fail(BITNET_HIP_MEMORY_ERROR, "split-k GEMM: scratch of %zu bytes / %zu counters for %zu tiles in %d parts",
+                    scratch.partial_bytes, scratch.counter_count, tiles, nsplit);
+    p.nsplit = nsplit; p.st_per = st_per; p.rotate = 0;
+    p.partials = scratch.partials; p.counters = scratch.counters;
+    const int total = (int)tiles * nsplit;
+    const int grid = ((total + 7) / 8) * 8;
+    constexpr size_t lds = dma_lds_bytes<BM, BN, D>();
+    static const hipError_t attr = lds > 64 * 1024 ? raise_lds_limit(&gemm_dma_kernel<BM, BN, D, OCC, true>, lds) : hipSuccess;
+    BITNET_HIP_TRY(attr);
+    hipLaunchKernelGGL((gemm_dma_kernel<BM, BN, D, OCC, true>), dim3(grid), dim3(256), lds, stream, p);
+    BITNET_HIP_CHECK_LAUNCH("gemm_dma_kernel (k split)");
+    return BITNET_HIP_OK;
+}
+
 template <int BM, int BN>
 constexpr size_t ld8_lds_bytes() { return (size_t)LD8_NST * (BM * 256 + (BN / 16) * 1024) + rowp_bytes<BM>(); }
 
@@ -835,8 +908,35 @@ int launch_tile(GemmParams p, hipStream_t stream)
 // Up to GEMM_MAX_PROJ projections of the same activation matrix in one launch of the LDS-direct kernels (q, k, v
 // or gate, up at prefill: small projections alone would leave most compute units idle).  Returns
 // BITNET_HIP_UNSUPPORTED (without a message) when the shapes do not fit those kernels.
+namespace {
+// k split across workgroups: where, and into how many parts of how many 128-column stages (even).  tiles32: 64 x 32
+// tiles of the launch.  One round of workgroups at four per compute unit holds 1024: three parts of at most 352 tiles.
+bool plan_split(size_t m, size_t k, size_t tiles32, int *nsplit, int *st_per)
+{
+    if (m <= 96 || k < 4096 || k % 256 != 0 || tiles32 == 0 || tiles32 > 352) return false;
+    const int nstage = (int)(k / 128);
+    const int per = ((nstage + 2) / 3 + 1) & ~1;
+    const int parts = (nstage + per - 1) / per;
+    if (parts < 2) return false;
+    *nsplit = parts; *st_per = per;
+    return true;
+}
+}  // namespace
+
+void gemm_split_plan(size_t m, size_t k, const size_t *n, int nproj, size_t *partial_bytes, size_t *counters)
+{
+    *partial_bytes = 0; *counters = 0;
+    if (nproj <= 0 || nproj > GEMM_MAX_PROJ) return;
+    size_t tiles32 = 0;
+    for (int j = 0; j < nproj; ++j) tiles32 += ((m + 63) / 64) * ((n[j] + 31) / 32);
+    int nsplit = 0, st_per = 0;
+    if (!plan_split(m, k, tiles32, &nsplit, &st_per)) return;
+    *partial_bytes = (tiles32 * nsplit * 64 * 32 * sizeof(int32_t) + 255) / 256 * 256;
+    *counters = tiles32;
+}
+
 int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const int32_t *a_sum, const float *a_scale,
-                      size_t m, size_t k, hipStream_t stream)
+                      size_t m, size_t k, hipStream_t stream, const GemmSplitScratch *split)
 {
     if (m == 0 || nproj <= 0) return BITNET_HIP_OK;
     if (nproj > GEMM_MAX_PROJ) return BITNET_HIP_UNSUPPORTED;
@@ -870,6 +970,13 @@ int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const i
     //   0.4 to one tile per compute unit     -> 128 x 160, one workgroup of 8 multiplying wavefronts (k split inside it)
     //                                           and two loader wavefronts;
     //   otherwise                            -> 64 x 160, four workgroups of 4 wavefronts per compute unit.
+    // A long k with few tiles: the 64 x 32 tiles of the launch in three parts of k each (plan_split).  Measured at
+    // 6912 -> 2560: 128 / 192 / 256 tokens 15.7 / 15.7 / 17.9 us -> 12.1 / 13.2 / 14.6 us; from 320 tokens on, and at
+    // k = 2560 at any token count, the partial tiles cost more to exchange than the shorter loops save.
+    if (split && split->partials) {
+        int nsplit = 0, st_per = 0;
+        if (plan_split(m, k, tiles32, &nsplit, &st_per)) return launch_dma_split<64, 32, 4, 4>(p, nsplit, st_per, *split, stream);
+    }
     if (tiles >= 640) return launch_dma<128, 160, 2, 3>(p, stream);
     // Few tiles: a workgroup walks the whole of k by itself and its time is a chain of load latencies, so small
     // launches take narrow tiles (more workgroups, all resident at once) with four stages of loads in flight.

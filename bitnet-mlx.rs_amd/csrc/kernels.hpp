@@ -17,7 +17,8 @@ inline size_t tiled_bytes(size_t n, size_t k) { return row_blocks(n) * k_tiles(k
 // act_quant.hip
 int launch_act_quant(const float *x, const float *x2, size_t ldx, size_t m, size_t k, int input_mode,
                      size_t gqa_group, size_t head_dim, const float *gamma, float eps, int sum_order,
-                     int8_t *q, float *a_scale, int32_t *a_sum, float *y, hipStream_t stream);
+                     int8_t *q, float *a_scale, int32_t *a_sum, float *y, hipStream_t stream, unsigned *zero = nullptr,
+                     size_t zero_n = 0);  // zero[0 .. zero_n): cleared by the launch (tile counters of the GEMM behind it)
 
 // absmax_quantize_activations (activations.rs:530-641): one scale per tensor; scratch of absmax_quantize_scratch_bytes(n)
 // bytes; stats: 4 floats (scale, mse, min, max)
@@ -102,8 +103,19 @@ int launch_gemv_fused(const GemvProj *projs, int nproj, const float *x, const fl
 // gemm_w2a8.hip
 constexpr int GEMM_MAX_PROJ = 3;  // projections sharing one activation matrix per launch of the LDS-direct kernels
 // several projections in one launch; BITNET_HIP_UNSUPPORTED (no message) if the LDS-direct kernels do not apply
+// Scratch of a GEMM launch that splits k across workgroups (gemm_split_plan): int32 partial tiles, and one counter per
+// output tile that MUST be zero when the launch starts (the activation quantiser in front of the GEMM zeroes them:
+// launch_act_quant's zero / zero_n) and is zero again when it ends.  Both belong to the caller's workspace.
+struct GemmSplitScratch {
+    int32_t *partials = nullptr;
+    unsigned *counters = nullptr;
+    size_t partial_bytes = 0, counter_count = 0;
+};
+// What launch_gemm_multi needs to split k for this launch: bytes of partials (a multiple of 256) and the number of
+// counters; both 0 when it would not split.  n: output widths of the projections that share the launch.
+void gemm_split_plan(size_t m, size_t k, const size_t *n, int nproj, size_t *partial_bytes, size_t *counters);
 int launch_gemm_multi(const GemvProj *projs, int nproj, const int8_t *a, const int32_t *a_sum, const float *a_scale,
-                      size_t m, size_t k, hipStream_t stream);
+                      size_t m, size_t k, hipStream_t stream, const GemmSplitScratch *split = nullptr);
 // a_sum (sum_k a[t, k] per row, from the activation quantiser) may be NULL: the slower kernel then computes it
 int launch_gemm_tiled(const uint8_t *tiled, const int8_t *a, const int32_t *a_sum, size_t m, size_t n, size_t k,
                       int32_t *acc, const float *w_scale, const float *a_scale, const float *bias,

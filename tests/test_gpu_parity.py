@@ -740,6 +740,37 @@ def test_bitlinear_forward_prefill_uses_quantiser_row_sums():
     assert np.array_equal(host(out), out_ref)
 
 
+@pytest.mark.parametrize("m,k,n", [(97, 6912, 2560), (128, 6912, 2560), (200, 4096, 1000), (256, 6912, 2560), (130, 8192, 644)])
+def test_forward_split_k_bit_exact(m, k, n):
+    """A long k with few output tiles (97 to 256 tokens at 6912 -> 2560): forward() splits k across workgroups, which
+    exchange int32 partial tiles through the workspace.  Checked against the oracle (activations, accumulators, f32
+    output with bias and residual); with a workspace that holds only the quantised activations (no split: same bits);
+    on a workspace full of ones (the tile counters are cleared by the quantiser of the same call); and on the same
+    workspace three times in a row (the counters are left at zero)."""
+    rng = np.random.default_rng(m + k + n)
+    w = synth_weights(rng, n, k)
+    x = synth_activations(rng, m, k, outliers=True)
+    bias = rng.standard_normal(n, dtype=f32)
+    res = rng.standard_normal((m, n), dtype=f32)
+    layer = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n, use_bias=True), "split")
+    layer.update_weights(dev(w))
+    layer.update_bias(dev(bias))
+    qw, ws = orc.quantize_weights_absmean(w)
+    out_ref, q_ref, s_ref, acc_ref = orc.bitlinear_forward(x, orc.pack_2bit(qw), n, ws, bias=bias, residual=res)
+    out, q, a_scale, acc = layer.forward(dev(x), residual=dev(res), debug=True)
+    assert np.array_equal(host(q), q_ref) and np.array_equal(host(a_scale), s_ref)
+    assert np.array_equal(host(acc), acc_ref)
+    assert np.array_equal(host(out), out_ref)
+    full = layer.workspace_size(m)
+    quant_only = ((m * k + 255) // 256) * 256 + 2 * (((4 * m) + 255) // 256) * 256 + 256
+    assert full > quant_only, "this shape is expected to take the split"
+    small = torch.full((quant_only,), 1, dtype=torch.uint8, device="cuda")
+    assert np.array_equal(host(layer.forward(dev(x), residual=dev(res), workspace=small)), out_ref)
+    big = torch.full((full,), 1, dtype=torch.uint8, device="cuda")
+    for _ in range(3):
+        assert np.array_equal(host(layer.forward(dev(x), residual=dev(res), workspace=big)), out_ref)
+
+
 # ---- L1: BitLinear object ----------------------------------------------------------------------------------
 
 def test_bitlinear_forward_config1_bit_exact():
