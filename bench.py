@@ -264,6 +264,22 @@ def stack_latency(bh, torch, dec, gen, reps=20):
             ms, how = time_forward_graph(torch, bls, x, y, ws)
             out[f"{name}_m{m}"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1),
                                    "timed": how}
+    # short prompts on the long-k projection: forward (quantiser + GEMM) with the workspace forward asks for, which
+    # lets the GEMM split k across workgroups, and with one that holds the quantised activations only (no split)
+    n, k = dec.proj_shape(6)
+    bls = [dec.projection(layer, 6) for layer in range(dec.layers)]
+    for m in (128, 256):
+        x = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32)
+        y = torch.empty((m, n), device="cuda", dtype=torch.float32)
+        quant_only = (m * k + 255) // 256 * 256 + 2 * ((4 * m + 255) // 256 * 256) + 256
+        entry = {}
+        for label, size in (("us", bls[0].workspace_size(m)), ("us_without_k_split", quant_only)):
+            ws = torch.empty((size,), device="cuda", dtype=torch.uint8)
+            ms, how = time_forward_graph(torch, bls, x, y, ws)
+            entry[label] = round(ms * 1e3, 2)
+        entry["tops_incl_quantiser"] = round(2.0 * m * n * k / (entry["us"] * 1e-6) / 1e12, 1)
+        entry["timed"] = how
+        out[f"down_6912x2560_m{m}_forward"] = entry
     return out
 
 
