@@ -76,7 +76,7 @@ STEP_BYTES = LAYER_BYTES * LAYERS
 # script with --no-extras --calibration-copy), each scaled by what the same counter reads for the plain
 # 256 MiB copy: FETCH_SIZE reads 0.5 KiB per KiB fetched (factor 2.0), WRITE_SIZE 1.0 (factor 1.0).
 # Summary: profiles/decode_layer_b1_gemv_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_685_627
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 4_685_621
 
 
 def decode_roofline(event_ms, steps):
