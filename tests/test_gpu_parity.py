@@ -741,7 +741,8 @@ def test_bitlinear_forward_prefill_uses_quantiser_row_sums():
     assert np.array_equal(host(out), out_ref)
 
 
-@pytest.mark.parametrize("m,k,n", [(97, 6912, 2560), (128, 6912, 2560), (200, 4096, 1000), (256, 6912, 2560), (130, 8192, 644)])
+@pytest.mark.parametrize("m,k,n", [(97, 6912, 2560), (128, 6912, 2560), (200, 4096, 1000), (256, 6912, 2560), (130, 8192, 644),
+                                   (255, 5120, 1408), (97, 4096, 16), (256, 8192, 2816), (300, 4352, 2240)])
 def test_forward_split_k_bit_exact(m, k, n):
     """A long k with few output tiles (97 to 256 tokens at 6912 -> 2560): forward() splits k across workgroups, which
     exchange int32 partial tiles through the workspace.  Checked against the oracle (activations, accumulators, f32
