@@ -264,8 +264,15 @@ def stack_latency(bh, torch, dec, gen, reps=20):
             ms, how = time_forward_graph(torch, bls, x, y, ws)
             out[f"{name}_m{m}"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1),
                                    "timed": how}
-    # short prompts on the long-k projection: forward (quantiser + GEMM) with the workspace forward asks for, which
-    # lets the GEMM split k across workgroups, and with one that holds the quantised activations only (no split)
+    out.update(short_prompt_forward(torch, dec, gen))
+    return out
+
+
+def short_prompt_forward(torch, dec, gen):
+    """Short prompts on the long-k projection (6912 -> 2560 at 128 and 256 tokens): forward (quantiser + GEMM) with the
+    workspace forward asks for, which lets the GEMM split k across workgroups, and with one that holds the quantised
+    activations only (no split)."""
+    out = {}
     n, k = dec.proj_shape(6)
     bls = [dec.projection(layer, 6) for layer in range(dec.layers)]
     for m in (128, 256):
@@ -474,6 +481,9 @@ def main():
     ap.add_argument("--only-large-gemv", type=int, default=0, metavar="LOOPS",
                     help="run only the 32768 x 16384 one-token GEMV, on 2-bit tiles and on base-3 bytes, LOOPS times over four "
                          "matrices each (profiling runs)")
+    ap.add_argument("--only-short-prompt", action="store_true",
+                    help="run only forward at 128 and 256 tokens on the 6912 -> 2560 projection, with and without the k split "
+                         "(profiling runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -496,6 +506,9 @@ def main():
     dec, gen = build_stack(bh, torch, LAYERS)
     if args.only_prefill > 0:
         print(json.dumps({"prefill": prefill_rates(bh, torch, dec, gen, reps=args.only_prefill)}))
+        return
+    if args.only_short_prompt:
+        print(json.dumps(short_prompt_forward(torch, dec, gen)))
         return
     if args.only_batch8 > 0:
         big = bh.DecoderProjections(LAYERS, HIDDEN, FFN, Q_HEADS, KV_HEADS, HEAD_DIM, eps=1e-5, max_tokens=8)
