@@ -529,8 +529,8 @@ def test_sum_order_divergence_is_what_the_documents_quote():
     """How far the build's declared summation order (BLOCK256, the default) is from the reference's literal running sum
     (inference_integration.rs:476) on the oracle: 4000 rows ~ N(0,1), K = 2560, eps = 1e-5, RMSNorm weights one.  The
     sum of squares differs in its last bits for most rows, so a_scale does too; the int8 row differs in a handful of
-    rows, one element each (a product that sits on a rounding tie).  DESIGN.md and INTEGRATION.md quote these counts
-    beside the cost of the literal order; this test keeps them honest."""
+    rows, one element each (a product that sits on a rounding tie).  The project's documents quote these counts beside
+    the cost of the literal order; this test keeps them honest."""
     rng = np.random.default_rng(2025)
     rows, k = 4000, 2560
     x = rng.standard_normal((rows, k), dtype=f32)
