@@ -253,7 +253,7 @@ def stack_latency(bh, torch, dec, gen, reps=20):
     out.update(large_gemv_pair(bh, torch, gen))
     for name, p in (("gate_2560x6912", 4), ("down_6912x2560", 6)):
         n, k = dec.proj_shape(p)
-        bls = [dec.projection(layer, p) for layer in range(dec.layers)]  # rotating: 4.4 MB each, not L2-resident
+        bls = rotating_layers(bh, torch, dec, gen, p)  # 60 x 4.4 MB = 265 MB: more than the last-level cache holds
         bl = bls[0]
         for m in (1, 4, 16, 64):
             x = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32)
@@ -264,17 +264,41 @@ def stack_latency(bh, torch, dec, gen, reps=20):
             ms, how = time_forward_graph(torch, bls, x, y, ws)
             out[f"{name}_m{m}"] = {"us": round(ms * 1e3, 2), "gbs_packed_weights": round(n * k / 4 / (ms * 1e-3) / 1e9, 1),
                                    "timed": how}
-    out.update(short_prompt_forward(torch, dec, gen))
+    out.update(short_prompt_forward(bh, torch, dec, gen))
     return out
 
 
-def short_prompt_forward(torch, dec, gen):
+_ROTATING = {}
+
+
+def rotating_layers(bh, torch, dec, gen, proj):
+    """Sixty layers of one projection's shape, each with its own weights (265 MB of packed tiles at 6912 x 2560: the
+    256 MB last-level cache cannot hold them, so every pass fetches from HBM).  Gate and up have the same shape and serve
+    each other; for down the stack's thirty are joined by thirty more with random ternary codes."""
+    if proj in _ROTATING:
+        return _ROTATING[proj]
+    layers = [dec.projection(layer, proj) for layer in range(dec.layers)]
+    if proj in (4, 5):
+        layers += [dec.projection(layer, 9 - proj) for layer in range(dec.layers)]
+    else:
+        n, k = dec.proj_shape(proj)
+        for i in range(dec.layers):
+            bl = bh.BitLinear(bh.BitLinearConfig(in_features=k, out_features=n), f"rotating{proj}_{i}")
+            codes = torch.randint(0, 3, (n * k,), generator=gen, device="cuda", dtype=torch.uint8).view(-1, 4)
+            packed = (codes[:, 0] | (codes[:, 1] << 2) | (codes[:, 2] << 4) | (codes[:, 3] << 6)).contiguous()
+            bl.set_quantized_weights(packed, 0.02)
+            layers.append(bl)
+    _ROTATING[proj] = layers
+    return layers
+
+
+def short_prompt_forward(bh, torch, dec, gen):
     """Short prompts on the long-k projection (6912 -> 2560 at 128 and 256 tokens): forward (quantiser + GEMM) with the
     workspace forward asks for, which lets the GEMM split k across workgroups, and with one that holds the quantised
     activations only (no split)."""
     out = {}
     n, k = dec.proj_shape(6)
-    bls = [dec.projection(layer, 6) for layer in range(dec.layers)]
+    bls = rotating_layers(bh, torch, dec, gen, 6)
     for m in (128, 256):
         x = torch.randn((m, k), generator=gen, device="cuda", dtype=torch.float32)
         y = torch.empty((m, n), device="cuda", dtype=torch.float32)
@@ -390,7 +414,7 @@ def time_forward_graph(torch, bls, x, y, ws, replays=10):
         checked_replay()
         best = min(time_events(torch, graph.replay) for _ in range(replays))
         checked_replay()
-        return best / calls, f"hip graph of {calls} forwards (one per layer), best of {replays} replays"
+        return best / calls, f"hip graph of {calls} forwards (each over its own weights), best of {replays} replays"
     except Exception as exc:  # capture unsupported: keep the measurement, say how it was made
         torch.cuda.synchronize()
         ms = time_events(torch, lambda: [bl.forward(x, out=y, workspace=ws) for bl in bls]) / calls
@@ -508,7 +532,7 @@ def main():
         print(json.dumps({"prefill": prefill_rates(bh, torch, dec, gen, reps=args.only_prefill)}))
         return
     if args.only_short_prompt:
-        print(json.dumps(short_prompt_forward(torch, dec, gen)))
+        print(json.dumps(short_prompt_forward(bh, torch, dec, gen)))
         return
     if args.only_batch8 > 0:
         big = bh.DecoderProjections(LAYERS, HIDDEN, FFN, Q_HEADS, KV_HEADS, HEAD_DIM, eps=1e-5, max_tokens=8)
